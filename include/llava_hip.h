@@ -1,0 +1,165 @@
+/*
+ * llava_hip.h — C-ABI of the MI355X (gfx950) device layer that stands where the reference keeps its Vulkan
+ * objects (llava_context / llava_device_memory / llava_buffer / llava_pipeline / llava_command_buffer).
+ *
+ * The reference's host classes that stay (ggml_file, llava_session, the server wrapper) call only the
+ * functions below.  Everything is plain C: opaque handles, pointers and sizes.  Every function returns
+ * LV_OK (0) or a negative lv_status; nothing throws and nothing aborts.  lv_last_error() gives the text of
+ * the calling thread's last failure.
+ *
+ * Ownership: a handle belongs to whoever created it and is destroyed explicitly, children before parents
+ * (sessions, then the model, then the context).  Host pointers are borrowed for the duration of the call.
+ * All device work of a session runs on that session's own stream; a session must not be used from two
+ * threads at once, different sessions of one model may be.  Weights are immutable after upload.
+ *
+ * Each declaration names the reference interface it replaces (paths relative to the reference tree).
+ */
+#ifndef LLAVA_HIP_H
+#define LLAVA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+    LV_OK = 0,
+    LV_ERR_ARG = -1,      /* null pointer, bad shape, unsupported type */
+    LV_ERR_HIP = -2,      /* a HIP runtime call failed; text in lv_last_error() */
+    LV_ERR_OOM = -3,      /* device or host allocation failed */
+    LV_ERR_STATE = -4,    /* call order violated (step already in flight, nothing to wait for, ...) */
+    LV_ERR_RANGE = -5,    /* position / token id / backlog out of range */
+    LV_ERR_MISSING = -6   /* a tensor the model needs is not in the table */
+} lv_status;
+
+/* GGML element types the layer understands (types.h:28-43 of the reference) */
+enum { LV_F32 = 0, LV_F16 = 1, LV_Q4_0 = 2, LV_Q8_0 = 8 };
+
+typedef struct lv_ctx lv_ctx;
+typedef struct lv_model lv_model;
+typedef struct lv_session lv_session;
+
+const char *lv_last_error(void);
+
+/* ---- device context: replaces instance/device/queue/pool bring-up, llava_context.cpp:230-282 ---------- */
+int lv_ctx_create(int device, lv_ctx **out);
+int lv_ctx_destroy(lv_ctx *ctx);
+/* name, CU count, HBM bytes of the device (llava_context.cpp:240-251 prints the Vulkan equivalents) */
+int lv_ctx_info(const lv_ctx *ctx, char *name, size_t name_cap, uint32_t *compute_units, uint64_t *hbm_bytes);
+
+/* ---- model upload: replaces llava_layer::llava_layer + load_to_gpu (llava_layer.cpp:10-23,82-98),
+ *      llava_buffer::load_from_disk (llava_buffer.cpp:179-325) and the per-session norm/output upload
+ *      (llava_session.cpp:69-78).  One entry of the table per tensor of the GGJT file, exactly the fields of
+ *      ggml_data_descriptor (ggml_file.h:29-41). ---------------------------------------------------------- */
+typedef struct {
+    const char *name;     /* e.g. "layers.0.attention.wq.weight" */
+    uint32_t ftype;       /* LV_F32 / LV_Q4_0 / LV_Q8_0 */
+    uint64_t offset;      /* byte offset of the payload from `base` */
+    uint32_t rows, cols;  /* shape1, shape2: 2-D = (ne1, ne0); 1-D = (ne0, 1) */
+    uint64_t size;        /* payload bytes */
+} lv_tensor_desc;
+
+typedef struct {
+    uint32_t file_version;   /* only 3 (fp16 block scales) is accepted for quantised tensors */
+    uint32_t vocab, dim, heads, layers, rot, ff;
+} lv_hparams;
+
+/* Copies every tensor the decode path needs from the caller's mapping into an HBM weight arena (scales and
+ * codes are split into two aligned streams on the way).  Synchronous: the mapping may go away afterwards
+ * unless lv_step_begin is given token ids whose embedding rows live in it (see keep_host_embeddings). */
+int lv_model_upload(lv_ctx *ctx, const void *base, uint64_t base_size, const lv_hparams *hp,
+                    const lv_tensor_desc *table, uint32_t n_tensors, lv_model **out);
+int lv_model_destroy(lv_model *model);
+int lv_model_hparams(const lv_model *model, lv_hparams *out);
+/* bytes of HBM the weight arena holds */
+int lv_model_arena_bytes(const lv_model *model, uint64_t *bytes);
+
+/* ---- session: replaces llava_session::recreate_buffers (llava_session.cpp:49-79), set_backlog_size
+ *      (:303-327) and llava_layer_session_data::flush_buffers_on_gpu (llava_layer_session_data.cpp:52-163) */
+int lv_session_create(lv_model *model, lv_session **out);
+int lv_session_destroy(lv_session *s);
+/* (re)size the fp16 K/V caches to `backlog` rows per layer (any value >= 1; the reference uses powers of two
+ * 128..2048): the first min(old,new) rows are kept, the rest zero-filled.  Waits for the stream. */
+int lv_session_reserve(lv_session *s, uint32_t backlog);
+int lv_session_backlog(const lv_session *s, uint32_t *backlog);
+
+/* ---- one step: replaces the body of llava_session::start_next_token_prediction (llava_session.cpp:197-229),
+ *      llava_command_buffer::record_execution / run (llava_command_buffer.cpp:29-55) and the whole shader chain
+ *      of llava_layer::execute (llava_layer.cpp:39-75).
+ *      Asynchronous.  Evaluates n tokens whose cache rows are pos .. pos+n-1 (pos = tokens already cached).
+ *      Row z attends to cache rows 0 .. pos+z, like the batched shaders.  n == 1 replays a captured hipGraph. */
+int lv_step_begin(lv_session *s, const uint32_t *token_ids, uint32_t n, uint32_t pos);
+/* replaces llava_command_buffer::wait_idle (llava_command_buffer.cpp:25-27): the only sync point */
+int lv_step_wait(lv_session *s);
+/* replaces output_probs->map in get_last_predicted_token (llava_session.cpp:129-135): logits of the LAST row
+ * of the last step, `vocab` floats.  Implies lv_step_wait. */
+int lv_logits_read(lv_session *s, float *dst);
+/* index of the first strict maximum of those logits, computed on the device (the greedy rule of
+ * llava_session.cpp:144-152).  Implies lv_step_wait. */
+int lv_argmax(lv_session *s, uint32_t *token);
+/* Enables/disables hipGraph replay for n == 1 steps (on by default); off = plain stream launches. */
+int lv_session_use_graph(lv_session *s, int enable);
+
+/* ---- cache dump / restore: replaces llava_layer_session_data::dump_kv_cache / restore_kv_cache
+ *      (llava_layer_session_data.cpp:165-181).  which: 0 = K, 1 = V.  n_tokens rows of `dim` fp16 values. */
+int lv_kv_read(lv_session *s, uint32_t layer, int which, uint32_t n_tokens, void *dst);
+int lv_kv_write(lv_session *s, uint32_t layer, int which, uint32_t n_tokens, const void *src);
+
+/* ---- record mode: replaces the per-layer trace buffers of llava_layer_session_data.cpp:79-86 and their
+ *      routing in llava_layer.cpp:43-51.  When enabled, every step keeps, per layer and for the last row:
+ *      LV_TRACE_* below.  lv_trace_read copies one of them (count floats) to the host. */
+enum {
+    LV_TRACE_NORM_IN = 0,        /* normalized_input_logit  [dim] */
+    LV_TRACE_POST_ATTN = 1,      /* post_attn_logit         [dim] */
+    LV_TRACE_POST_ATTN_NORM = 2, /* post_attn_norm_logit    [dim] */
+    LV_TRACE_FF = 3,             /* ff_result               [ff]  */
+    LV_TRACE_OUT = 4,            /* output_logit            [dim] */
+    LV_TRACE_COUNT = 5
+};
+int lv_trace_enable(lv_session *s, int enable);
+int lv_trace_read(lv_session *s, uint32_t layer, int which, float *dst, uint32_t count);
+
+/* ---- device memory helpers for callers of the lv_kernel_* entry points (tests, microbenchmarks) -------- */
+int lv_dev_alloc(lv_ctx *ctx, uint64_t bytes, void **dptr);
+int lv_dev_free(lv_ctx *ctx, void *dptr);
+int lv_dev_upload(lv_ctx *ctx, void *dptr, const void *src, uint64_t bytes);
+int lv_dev_download(lv_ctx *ctx, void *dst, const void *dptr, uint64_t bytes);
+int lv_dev_zero(lv_ctx *ctx, void *dptr, uint64_t bytes);
+int lv_ctx_sync(lv_ctx *ctx);
+
+/* A quantised matrix in the device layout.  Built from GGML blocks by lv_matrix_upload; owns its memory. */
+typedef struct lv_matrix lv_matrix;
+/* replaces llava_buffer::load_from_disk for one tensor (llava_buffer.cpp:179-325) */
+int lv_matrix_upload(lv_ctx *ctx, const void *ggml_blocks, uint32_t ftype, uint32_t file_version, uint32_t rows,
+                     uint32_t cols, lv_matrix **out);
+int lv_matrix_destroy(lv_matrix *m);
+/* bytes the device layout occupies (equals the GGML payload size: 18 / 34 bytes per 32 weights) */
+int lv_matrix_bytes(const lv_matrix *m, uint64_t *bytes);
+
+/* ---- single kernels on the context's stream; all pointers are device pointers.  Asynchronous: follow with
+ *      lv_ctx_sync.  `batch` rows are independent (the shaders' gl_GlobalInvocationID.z). ------------------- */
+
+/* dequantise rows [row0, row0+n_rows) of m to fp32: the arithmetic of llava_buffer::write_f32
+ * (llava_buffer.cpp:339-401), bit-exact */
+int lv_kernel_dequant(lv_ctx *ctx, const lv_matrix *m, uint32_t row0, uint32_t n_rows, float *dst);
+/* matmul_dim* / matmul_ff* (matmul.glsl:41-74, matmul_q8.glsl:41-72); accumulate != 0 = matmul_add_* */
+int lv_kernel_gemv(lv_ctx *ctx, float *out, const lv_matrix *w, const float *x, uint32_t batch, int accumulate);
+/* matmul_silu_ff* (matmul_silu_ff.comp:49-97): out = (W3 x) * silu(W1 x) */
+int lv_kernel_gemv_silu(lv_ctx *ctx, float *out, const lv_matrix *w3, const lv_matrix *w1, const float *x,
+                        uint32_t batch);
+/* normalize (normalize.comp:34-64): out = x * w * rsqrt(mean((x - mean(x))^2)), no epsilon */
+int lv_kernel_normalize(lv_ctx *ctx, float *out, const float *x, const float *w, uint32_t dim, uint32_t batch);
+/* copy_to_cache (copy_to_cache.comp:29-37): cache[(pos+z)*dim + i] = fp16(in[z*dim + i]) */
+int lv_kernel_kv_append(lv_ctx *ctx, void *cache, const float *in, uint32_t pos, uint32_t dim, uint32_t batch,
+                        uint32_t backlog);
+/* mhsa + softmax + kqv_matching fused (mhsa.comp:32-60, softmax.comp:26-44, kqv_matching.comp:27-42):
+ * out[z][dim] = sum_{p <= pos+z} softmax_p( Q_z . Rot(-(pos+z-p) theta) K_p / sqrt(rot) ) V_p  per head */
+int lv_kernel_attention(lv_ctx *ctx, float *out, const void *kcache, const void *vcache, const float *q,
+                        uint32_t pos, uint32_t backlog, uint32_t heads, uint32_t rot, uint32_t batch);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LLAVA_HIP_H */

@@ -1,0 +1,1001 @@
+// lv_api.hip — implementation of the C-ABI declared in include/llava_hip.h for gfx950.
+//
+// What lives here: the HBM weight arena and its upload path, per-session K/V cache + activation buffers on
+// one stream, the decode step as a chain of hand-written kernels (lv_kernels.h) captured into a hipGraph,
+// and thin single-kernel entry points.  No Vulkan-style objects survive: a "buffer" is a pointer into an
+// arena, a "pipeline" is a template instantiation, the "command buffer" is the captured graph.
+#include "../../include/llava_hip.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "lv_kernels.h"
+
+using namespace lv;
+
+// -----------------------------------------------------------------------------------------------------------
+// errors
+// -----------------------------------------------------------------------------------------------------------
+static thread_local char g_err[512] = "";
+
+static int fail(int code, const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+#define HIP_TRY(expr)                                                                                         \
+    do {                                                                                                      \
+        hipError_t e_ = (expr);                                                                               \
+        if (e_ != hipSuccess) return fail(LV_ERR_HIP, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_), \
+                                          __FILE__, __LINE__);                                                \
+    } while (0)
+
+#define LV_TRY(expr)              \
+    do {                          \
+        int rc_ = (expr);         \
+        if (rc_ != LV_OK) return rc_; \
+    } while (0)
+
+extern "C" const char *lv_last_error(void) { return g_err; }
+
+// -----------------------------------------------------------------------------------------------------------
+// objects
+// -----------------------------------------------------------------------------------------------------------
+struct lv_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    hipDeviceProp_t props{};
+    // scratch for the stand-alone attention entry point
+    float2 *trig = nullptr;
+    uint32_t trig_rows = 0, trig_rot = 0;
+    float *attn_part = nullptr;
+    uint32_t *attn_counters = nullptr;
+    size_t attn_part_floats = 0, attn_counter_words = 0;
+};
+
+struct lv_matrix {
+    lv_ctx *ctx = nullptr;
+    void *owned = nullptr;  // allocation to free, or null when the matrix lives in a model arena
+    MatView view{};
+    uint32_t ftype = 0;
+    uint64_t bytes = 0;
+};
+
+struct LayerWeights {
+    lv_matrix wq, wk, wv, wo, w1, w2, w3;
+    const float *attn_norm = nullptr, *ffn_norm = nullptr;
+};
+
+struct lv_model {
+    lv_ctx *ctx = nullptr;
+    lv_hparams hp{};
+    uint8_t *arena = nullptr;
+    uint64_t arena_bytes = 0;
+    std::vector<LayerWeights> layers;
+    const float *norm = nullptr;
+    lv_matrix output;
+    uint32_t tok_ftype = LV_F32;
+    const float *tok_f32 = nullptr;
+    lv_matrix tok_quant;
+};
+
+constexpr uint32_t kAttnChunk = 64;   // cache positions per attention workgroup
+constexpr uint32_t kMaxStepTokens = 4096;
+
+struct lv_session {
+    lv_model *model = nullptr;
+    hipStream_t stream = nullptr;
+    uint32_t backlog = 0;
+    uint16_t *kv = nullptr;  // [layers][2][backlog][dim]
+    float2 *trig = nullptr;  // [backlog][rot/2]
+    // activations (batch 1)
+    float *x = nullptr, *xn = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *vo = nullptr, *ff = nullptr,
+          *logits = nullptr;
+    float *attn_part = nullptr;
+    uint32_t *attn_counters = nullptr;
+    uint32_t *cfg = nullptr;       // device: [0] = pos, [1..] = token ids of the step
+    uint32_t *cfg_host = nullptr;  // pinned staging of the same
+    uint32_t *argmax_dev = nullptr;
+    uint32_t *argmax_host = nullptr;  // pinned
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t graph_exec = nullptr;
+    bool use_graph = true;
+    bool in_flight = false;
+    bool have_logits = false;
+    bool trace = false;
+    float *trace_buf = nullptr;  // [layers][LV_TRACE_COUNT][max(dim, ff)]
+};
+
+static uint16_t *kv_ptr(const lv_session *s, uint32_t layer, int which)
+{
+    const size_t plane = (size_t)s->backlog * s->model->hp.dim;
+    return s->kv + ((size_t)layer * 2 + (which ? 1 : 0)) * plane;
+}
+
+// -----------------------------------------------------------------------------------------------------------
+// context
+// -----------------------------------------------------------------------------------------------------------
+extern "C" int lv_ctx_create(int device, lv_ctx **out)
+{
+    if (!out) return fail(LV_ERR_ARG, "lv_ctx_create: out is null");
+    *out = nullptr;
+    int count = 0;
+    HIP_TRY(hipGetDeviceCount(&count));
+    if (device < 0 || device >= count) return fail(LV_ERR_ARG, "lv_ctx_create: device %d of %d", device, count);
+    HIP_TRY(hipSetDevice(device));
+    lv_ctx *c = new (std::nothrow) lv_ctx;
+    if (!c) return fail(LV_ERR_OOM, "lv_ctx_create: host allocation");
+    c->device = device;
+    hipError_t e = hipGetDeviceProperties(&c->props, device);
+    if (e == hipSuccess) e = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking);
+    if (e != hipSuccess) {
+        delete c;
+        return fail(LV_ERR_HIP, "lv_ctx_create: %s", hipGetErrorString(e));
+    }
+    *out = c;
+    return LV_OK;
+}
+
+extern "C" int lv_ctx_destroy(lv_ctx *c)
+{
+    if (!c) return LV_OK;
+    (void)hipSetDevice(c->device);
+    (void)hipStreamSynchronize(c->stream);
+    (void)hipFree(c->trig);
+    (void)hipFree(c->attn_part);
+    (void)hipFree(c->attn_counters);
+    (void)hipStreamDestroy(c->stream);
+    delete c;
+    return LV_OK;
+}
+
+extern "C" int lv_ctx_info(const lv_ctx *c, char *name, size_t cap, uint32_t *cus, uint64_t *hbm)
+{
+    if (!c) return fail(LV_ERR_ARG, "lv_ctx_info: ctx is null");
+    if (name && cap) snprintf(name, cap, "%s (%s)", c->props.name, c->props.gcnArchName);
+    if (cus) *cus = (uint32_t)c->props.multiProcessorCount;
+    if (hbm) *hbm = (uint64_t)c->props.totalGlobalMem;
+    return LV_OK;
+}
+
+extern "C" int lv_ctx_sync(lv_ctx *c)
+{
+    if (!c) return fail(LV_ERR_ARG, "lv_ctx_sync: ctx is null");
+    HIP_TRY(hipStreamSynchronize(c->stream));
+    return LV_OK;
+}
+
+extern "C" int lv_dev_alloc(lv_ctx *c, uint64_t bytes, void **dptr)
+{
+    if (!c || !dptr) return fail(LV_ERR_ARG, "lv_dev_alloc: null argument");
+    *dptr = nullptr;
+    if (bytes == 0) return LV_OK;
+    hipError_t e = hipMalloc(dptr, bytes);
+    if (e == hipErrorOutOfMemory) return fail(LV_ERR_OOM, "lv_dev_alloc: %llu bytes", (unsigned long long)bytes);
+    HIP_TRY(e);
+    return LV_OK;
+}
+
+extern "C" int lv_dev_free(lv_ctx *c, void *dptr)
+{
+    if (!c) return fail(LV_ERR_ARG, "lv_dev_free: ctx is null");
+    if (dptr) HIP_TRY(hipFree(dptr));
+    return LV_OK;
+}
+
+extern "C" int lv_dev_upload(lv_ctx *c, void *dptr, const void *src, uint64_t bytes)
+{
+    if (!c || (bytes && (!dptr || !src))) return fail(LV_ERR_ARG, "lv_dev_upload: null argument");
+    if (bytes == 0) return LV_OK;
+    HIP_TRY(hipMemcpyAsync(dptr, src, bytes, hipMemcpyHostToDevice, c->stream));
+    HIP_TRY(hipStreamSynchronize(c->stream));
+    return LV_OK;
+}
+
+extern "C" int lv_dev_download(lv_ctx *c, void *dst, const void *dptr, uint64_t bytes)
+{
+    if (!c || (bytes && (!dptr || !dst))) return fail(LV_ERR_ARG, "lv_dev_download: null argument");
+    if (bytes == 0) return LV_OK;
+    HIP_TRY(hipMemcpyAsync(dst, dptr, bytes, hipMemcpyDeviceToHost, c->stream));
+    HIP_TRY(hipStreamSynchronize(c->stream));
+    return LV_OK;
+}
+
+// zero fill with a kernel (usable inside graph capture, unlike a memset node)
+__global__ void fill_zero_kernel(uint32_t *p, uint64_t words)
+{
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < words; i += (uint64_t)gridDim.x * blockDim.x)
+        p[i] = 0u;
+}
+
+static int zero_async(void *p, uint64_t bytes, hipStream_t st)
+{
+    if (bytes == 0) return LV_OK;
+    if (bytes % 4) return fail(LV_ERR_ARG, "zero fill: size not a multiple of 4");
+    const uint64_t words = bytes / 4;
+    uint64_t blocks = (words + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    fill_zero_kernel<<<dim3((unsigned)blocks), dim3(256), 0, st>>>(static_cast<uint32_t *>(p), words);
+    HIP_TRY(hipGetLastError());
+    return LV_OK;
+}
+
+extern "C" int lv_dev_zero(lv_ctx *c, void *dptr, uint64_t bytes)
+{
+    if (!c || (bytes && !dptr)) return fail(LV_ERR_ARG, "lv_dev_zero: null argument");
+    return zero_async(dptr, bytes, c->stream);
+}
+
+// -----------------------------------------------------------------------------------------------------------
+// matrices
+// -----------------------------------------------------------------------------------------------------------
+static uint64_t ggml_bytes(uint32_t ftype, uint64_t n)
+{
+    switch (ftype) {
+    case LV_F32: return n * 4;
+    case LV_F16: return n * 2;
+    case LV_Q4_0: return n / 32 * 18;
+    case LV_Q8_0: return n / 32 * 34;
+    default: return 0;
+    }
+}
+
+// device bytes of the split layout: codes first (16-byte aligned), scales after (2-byte values)
+static uint64_t codes_bytes(uint32_t ftype, uint64_t n_blocks) { return n_blocks * (ftype == LV_Q4_0 ? 16 : 32); }
+
+static uint64_t align_up(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
+
+// Copies one GGML-format quantised tensor to `dst` (device, 256-byte aligned, matrix_device_bytes long)
+// through a device staging buffer and splits it there.
+static uint64_t matrix_device_bytes(uint32_t ftype, uint64_t rows, uint64_t cols)
+{
+    const uint64_t nblk = rows * (cols / 32);
+    return align_up(codes_bytes(ftype, nblk), 256) + align_up(nblk * 2, 256);
+}
+
+static int place_matrix(lv_ctx *c, lv_matrix *m, uint8_t *dst, const void *host_blocks, uint32_t ftype, uint32_t rows,
+                        uint32_t cols, uint8_t *staging)
+{
+    const uint64_t nblk = (uint64_t)rows * (cols / 32);
+    const uint64_t raw = ggml_bytes(ftype, (uint64_t)rows * cols);
+    HIP_TRY(hipMemcpyAsync(staging, host_blocks, raw, hipMemcpyHostToDevice, c->stream));
+    uint4 *codes = reinterpret_cast<uint4 *>(dst);
+    uint16_t *scales = reinterpret_cast<uint16_t *>(dst + align_up(codes_bytes(ftype, nblk), 256));
+    const unsigned grid = (unsigned)((nblk + 255) / 256);
+    if (ftype == LV_Q4_0)
+        repack_kernel<4><<<dim3(grid), dim3(256), 0, c->stream>>>(staging, codes, scales, nblk);
+    else
+        repack_kernel<8><<<dim3(grid), dim3(256), 0, c->stream>>>(staging, codes, scales, nblk);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipStreamSynchronize(c->stream));  // staging is reused by the next tensor
+    m->ctx = c;
+    m->view.codes = codes;
+    m->view.scales = scales;
+    m->view.rows = rows;
+    m->view.cols = cols;
+    m->ftype = ftype;
+    m->bytes = raw;
+    return LV_OK;
+}
+
+static int check_quant_shape(const char *who, uint32_t ftype, uint32_t file_version, uint32_t rows, uint32_t cols)
+{
+    if (ftype != LV_Q4_0 && ftype != LV_Q8_0) return fail(LV_ERR_ARG, "%s: type %u is not q4_0/q8_0", who, ftype);
+    if (file_version != 3)
+        return fail(LV_ERR_ARG, "%s: file version %u (only version 3, fp16 block scales, is supported)", who, file_version);
+    if (rows == 0 || cols == 0 || cols % 32) return fail(LV_ERR_ARG, "%s: shape %u x %u", who, rows, cols);
+    if (cols / 32 > 768) return fail(LV_ERR_ARG, "%s: %u columns exceed the 24576 the GEMV kernels cover", who, cols);
+    return LV_OK;
+}
+
+extern "C" int lv_matrix_upload(lv_ctx *c, const void *blocks, uint32_t ftype, uint32_t file_version, uint32_t rows,
+                                uint32_t cols, lv_matrix **out)
+{
+    if (!c || !blocks || !out) return fail(LV_ERR_ARG, "lv_matrix_upload: null argument");
+    *out = nullptr;
+    LV_TRY(check_quant_shape("lv_matrix_upload", ftype, file_version, rows, cols));
+    HIP_TRY(hipSetDevice(c->device));
+    lv_matrix *m = new (std::nothrow) lv_matrix;
+    if (!m) return fail(LV_ERR_OOM, "lv_matrix_upload: host allocation");
+    uint8_t *staging = nullptr;
+    const uint64_t raw = ggml_bytes(ftype, (uint64_t)rows * cols);
+    hipError_t e = hipMalloc(&m->owned, matrix_device_bytes(ftype, rows, cols));
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&staging), raw);
+    int rc = LV_OK;
+    if (e != hipSuccess) rc = fail(e == hipErrorOutOfMemory ? LV_ERR_OOM : LV_ERR_HIP, "lv_matrix_upload: %s", hipGetErrorString(e));
+    if (rc == LV_OK) rc = place_matrix(c, m, static_cast<uint8_t *>(m->owned), blocks, ftype, rows, cols, staging);
+    (void)hipFree(staging);
+    if (rc != LV_OK) {
+        (void)hipFree(m->owned);
+        delete m;
+        return rc;
+    }
+    *out = m;
+    return LV_OK;
+}
+
+extern "C" int lv_matrix_destroy(lv_matrix *m)
+{
+    if (!m) return LV_OK;
+    if (m->owned) (void)hipFree(m->owned);
+    delete m;
+    return LV_OK;
+}
+
+extern "C" int lv_matrix_bytes(const lv_matrix *m, uint64_t *bytes)
+{
+    if (!m || !bytes) return fail(LV_ERR_ARG, "lv_matrix_bytes: null argument");
+    *bytes = m->bytes;
+    return LV_OK;
+}
+
+// -----------------------------------------------------------------------------------------------------------
+// kernel launchers
+// -----------------------------------------------------------------------------------------------------------
+template <int QT, int MODE, int CW, int P>
+static void launch_gemv_cfg(const GemvArgs &a, uint32_t batch, hipStream_t st)
+{
+    constexpr int RPW = 4;
+    constexpr int rows_per_wg = (4 / CW) * RPW;
+    const unsigned grid = (a.w.rows + rows_per_wg - 1) / rows_per_wg;
+    gemv_kernel<QT, MODE, CW, P, RPW><<<dim3(grid, batch), dim3(256), 0, st>>>(a);
+}
+
+template <int QT, int MODE>
+static void launch_gemv_mode(const GemvArgs &a, uint32_t batch, hipStream_t st)
+{
+    const uint32_t nb = a.w.cols / 32;
+    if (nb <= 64) launch_gemv_cfg<QT, MODE, 1, 1>(a, batch, st);
+    else if (nb <= 128) launch_gemv_cfg<QT, MODE, 2, 1>(a, batch, st);
+    else if (nb <= 256) launch_gemv_cfg<QT, MODE, 4, 1>(a, batch, st);
+    else if (nb <= 512) launch_gemv_cfg<QT, MODE, 4, 2>(a, batch, st);
+    else launch_gemv_cfg<QT, MODE, 4, 3>(a, batch, st);
+}
+
+static int launch_gemv(hipStream_t st, float *out, const lv_matrix &w, const lv_matrix *w1, const float *x, uint32_t batch,
+                       int mode)
+{
+    GemvArgs a{};
+    a.w = w.view;
+    if (w1) a.w1 = w1->view;
+    a.x = x;
+    a.out = out;
+    const bool q4 = w.ftype == LV_Q4_0;
+    switch (mode) {
+    case kGemvStore: q4 ? launch_gemv_mode<4, kGemvStore>(a, batch, st) : launch_gemv_mode<8, kGemvStore>(a, batch, st); break;
+    case kGemvAdd: q4 ? launch_gemv_mode<4, kGemvAdd>(a, batch, st) : launch_gemv_mode<8, kGemvAdd>(a, batch, st); break;
+    default: q4 ? launch_gemv_mode<4, kGemvSilu>(a, batch, st) : launch_gemv_mode<8, kGemvSilu>(a, batch, st); break;
+    }
+    HIP_TRY(hipGetLastError());
+    return LV_OK;
+}
+
+static size_t attn_part_floats(uint32_t batch, uint32_t heads, uint32_t splits, uint32_t rot)
+{
+    return (size_t)batch * heads * splits * (rot + 1);
+}
+
+static int launch_attention(hipStream_t st, float *out, const uint16_t *kc, const uint16_t *vc, const float *q,
+                            const float2 *trig, float *part, uint32_t *counters, const uint32_t *pos_ptr, uint32_t pos_add,
+                            uint32_t backlog, uint32_t heads, uint32_t rot, uint32_t batch)
+{
+    AttnArgs a{};
+    a.out = out; a.kcache = kc; a.vcache = vc; a.q = q; a.trig = trig; a.part = part; a.counters = counters;
+    a.pos_ptr = pos_ptr; a.pos_add = pos_add; a.heads = heads; a.backlog = backlog; a.chunk = kAttnChunk;
+    a.splits = (backlog + kAttnChunk - 1) / kAttnChunk;
+    const dim3 grid(heads, a.splits, batch);
+    const size_t lds = sizeof(float) * (kAttnChunk + 4 * (rot + 1));
+    switch (rot) {
+    case 32: attention_kernel<32><<<grid, dim3(256), lds, st>>>(a); break;
+    case 64: attention_kernel<64><<<grid, dim3(256), lds, st>>>(a); break;
+    case 128: attention_kernel<128><<<grid, dim3(256), lds, st>>>(a); break;
+    default: return fail(LV_ERR_ARG, "attention: head size %u (32, 64 and 128 are built)", rot);
+    }
+    HIP_TRY(hipGetLastError());
+    return LV_OK;
+}
+
+// cos/sin of delta*theta_i with the argument rounded the way mhsa.comp:45 rounds it:
+// theta_i = pow(10000, -i/(R/2)) in fp32, delta*theta_i as one fp32 product.
+static void build_trig(std::vector<float2> &t, uint32_t rows, uint32_t rot)
+{
+    const uint32_t half = rot / 2;
+    t.resize((size_t)rows * half);
+    std::vector<float> freq(half);
+    for (uint32_t i = 0; i < half; i++) freq[i] = powf(10000.0f, -(float)i / (float)half);
+    for (uint32_t d = 0; d < rows; d++)
+        for (uint32_t i = 0; i < half; i++) {
+            const float ang = (float)d * freq[i];
+            t[(size_t)d * half + i] = make_float2((float)cos((double)ang), (float)sin((double)ang));
+        }
+}
+
+static int upload_trig(float2 **dev, uint32_t rows, uint32_t rot, hipStream_t st)
+{
+    std::vector<float2> t;
+    build_trig(t, rows, rot);
+    HIP_TRY(hipMalloc(reinterpret_cast<void **>(dev), t.size() * sizeof(float2)));
+    HIP_TRY(hipMemcpyAsync(*dev, t.data(), t.size() * sizeof(float2), hipMemcpyHostToDevice, st));
+    HIP_TRY(hipStreamSynchronize(st));
+    return LV_OK;
+}
+
+// -----------------------------------------------------------------------------------------------------------
+// single-kernel entry points
+// -----------------------------------------------------------------------------------------------------------
+extern "C" int lv_kernel_dequant(lv_ctx *c, const lv_matrix *m, uint32_t row0, uint32_t n_rows, float *dst)
+{
+    if (!c || !m || !dst) return fail(LV_ERR_ARG, "lv_kernel_dequant: null argument");
+    if ((uint64_t)row0 + n_rows > m->view.rows) return fail(LV_ERR_RANGE, "lv_kernel_dequant: rows %u+%u of %u", row0, n_rows, m->view.rows);
+    if (n_rows == 0) return LV_OK;
+    const uint64_t nb = m->view.cols / 32, first = (uint64_t)row0 * nb, count = (uint64_t)n_rows * nb;
+    const unsigned grid = (unsigned)((count + 255) / 256);
+    if (m->ftype == LV_Q4_0) dequant_kernel<4><<<dim3(grid), dim3(256), 0, c->stream>>>(m->view, first, count, dst);
+    else dequant_kernel<8><<<dim3(grid), dim3(256), 0, c->stream>>>(m->view, first, count, dst);
+    HIP_TRY(hipGetLastError());
+    return LV_OK;
+}
+
+extern "C" int lv_kernel_gemv(lv_ctx *c, float *out, const lv_matrix *w, const float *x, uint32_t batch, int accumulate)
+{
+    if (!c || !out || !w || !x) return fail(LV_ERR_ARG, "lv_kernel_gemv: null argument");
+    if (batch == 0) return LV_OK;
+    if (batch > 65535) return fail(LV_ERR_RANGE, "lv_kernel_gemv: batch %u", batch);
+    return launch_gemv(c->stream, out, *w, nullptr, x, batch, accumulate ? kGemvAdd : kGemvStore);
+}
+
+extern "C" int lv_kernel_gemv_silu(lv_ctx *c, float *out, const lv_matrix *w3, const lv_matrix *w1, const float *x, uint32_t batch)
+{
+    if (!c || !out || !w3 || !w1 || !x) return fail(LV_ERR_ARG, "lv_kernel_gemv_silu: null argument");
+    if (w3->ftype != w1->ftype || w3->view.rows != w1->view.rows || w3->view.cols != w1->view.cols)
+        return fail(LV_ERR_ARG, "lv_kernel_gemv_silu: the two matrices differ in type or shape");
+    if (batch == 0) return LV_OK;
+    if (batch > 65535) return fail(LV_ERR_RANGE, "lv_kernel_gemv_silu: batch %u", batch);
+    return launch_gemv(c->stream, out, *w3, w1, x, batch, kGemvSilu);
+}
+
+extern "C" int lv_kernel_normalize(lv_ctx *c, float *out, const float *x, const float *w, uint32_t dim, uint32_t batch)
+{
+    if (!c || !out || !x || !w) return fail(LV_ERR_ARG, "lv_kernel_normalize: null argument");
+    if (dim == 0) return fail(LV_ERR_ARG, "lv_kernel_normalize: dim is 0");
+    if (batch == 0) return LV_OK;
+    normalize_kernel<<<dim3(batch), dim3(256), 0, c->stream>>>(out, x, w, dim);
+    HIP_TRY(hipGetLastError());
+    return LV_OK;
+}
+
+extern "C" int lv_kernel_kv_append(lv_ctx *c, void *cache, const float *in, uint32_t pos, uint32_t dim, uint32_t batch,
+                                   uint32_t backlog)
+{
+    if (!c || !cache || !in) return fail(LV_ERR_ARG, "lv_kernel_kv_append: null argument");
+    if ((uint64_t)pos + batch > backlog) return fail(LV_ERR_RANGE, "lv_kernel_kv_append: rows %u+%u of %u", pos, batch, backlog);
+    if (batch == 0 || dim == 0) return LV_OK;
+    kv_append_kernel<<<dim3((dim + 255) / 256, batch), dim3(256), 0, c->stream>>>(static_cast<uint16_t *>(cache), in, nullptr,
+                                                                                    pos, dim, backlog);
+    HIP_TRY(hipGetLastError());
+    return LV_OK;
+}
+
+extern "C" int lv_kernel_attention(lv_ctx *c, float *out, const void *kcache, const void *vcache, const float *q, uint32_t pos,
+                                   uint32_t backlog, uint32_t heads, uint32_t rot, uint32_t batch)
+{
+    if (!c || !out || !kcache || !vcache || !q) return fail(LV_ERR_ARG, "lv_kernel_attention: null argument");
+    if (heads == 0 || batch == 0 || backlog == 0) return fail(LV_ERR_ARG, "lv_kernel_attention: empty shape");
+    if ((uint64_t)pos + batch > backlog) return fail(LV_ERR_RANGE, "lv_kernel_attention: rows %u+%u of %u", pos, batch, backlog);
+    if (rot != 32 && rot != 64 && rot != 128) return fail(LV_ERR_ARG, "lv_kernel_attention: head size %u", rot);
+    HIP_TRY(hipSetDevice(c->device));
+    if (c->trig_rot != rot || c->trig_rows < backlog) {
+        HIP_TRY(hipStreamSynchronize(c->stream));
+        (void)hipFree(c->trig);
+        c->trig = nullptr;
+        c->trig_rows = c->trig_rot = 0;
+        LV_TRY(upload_trig(&c->trig, backlog, rot, c->stream));
+        c->trig_rows = backlog;
+        c->trig_rot = rot;
+    }
+    const uint32_t splits = (backlog + kAttnChunk - 1) / kAttnChunk;
+    const size_t need_part = attn_part_floats(batch, heads, splits, rot), need_cnt = (size_t)batch * heads;
+    if (c->attn_part_floats < need_part) {
+        HIP_TRY(hipStreamSynchronize(c->stream));
+        (void)hipFree(c->attn_part);
+        c->attn_part = nullptr;
+        c->attn_part_floats = 0;
+        HIP_TRY(hipMalloc(reinterpret_cast<void **>(&c->attn_part), need_part * sizeof(float)));
+        c->attn_part_floats = need_part;
+    }
+    if (c->attn_counter_words < need_cnt) {
+        HIP_TRY(hipStreamSynchronize(c->stream));
+        (void)hipFree(c->attn_counters);
+        c->attn_counters = nullptr;
+        c->attn_counter_words = 0;
+        HIP_TRY(hipMalloc(reinterpret_cast<void **>(&c->attn_counters), need_cnt * 4));
+        c->attn_counter_words = need_cnt;
+        LV_TRY(zero_async(c->attn_counters, need_cnt * 4, c->stream));
+    }
+    return launch_attention(c->stream, out, static_cast<const uint16_t *>(kcache), static_cast<const uint16_t *>(vcache), q,
+                            c->trig, c->attn_part, c->attn_counters, nullptr, pos, backlog, heads, rot, batch);
+}
+
+// -----------------------------------------------------------------------------------------------------------
+// model
+// -----------------------------------------------------------------------------------------------------------
+static const lv_tensor_desc *find_desc(const lv_tensor_desc *t, uint32_t n, const std::string &name)
+{
+    for (uint32_t i = 0; i < n; i++)
+        if (t[i].name && name == t[i].name) return &t[i];
+    const std::string alt = name + ".weight";  // same fallback as ggml_file::get_buffer_descriptor
+    for (uint32_t i = 0; i < n; i++)
+        if (t[i].name && alt == t[i].name) return &t[i];
+    return nullptr;
+}
+
+struct Want {
+    std::string name;
+    uint32_t rows, cols;   // expected shape (cols == 1 for vectors)
+    bool quant;            // must be q4_0 / q8_0 (matrices); otherwise f32 (vectors) or anything (embeddings)
+    const lv_tensor_desc *desc = nullptr;
+    uint64_t arena_off = 0;
+};
+
+extern "C" int lv_model_upload(lv_ctx *c, const void *base, uint64_t base_size, const lv_hparams *hp,
+                               const lv_tensor_desc *table, uint32_t n_tensors, lv_model **out)
+{
+    if (!c || !base || !hp || !table || !out) return fail(LV_ERR_ARG, "lv_model_upload: null argument");
+    *out = nullptr;
+    const uint32_t D = hp->dim, F = hp->ff, V = hp->vocab, L = hp->layers;
+    if (!D || !F || !V || !L || !hp->heads || hp->heads * hp->rot != D || D % 32 || F % 32)
+        return fail(LV_ERR_ARG, "lv_model_upload: inconsistent hyper-parameters (dim %u heads %u rot %u ff %u)", D, hp->heads, hp->rot, F);
+    if (hp->rot != 32 && hp->rot != 64 && hp->rot != 128)
+        return fail(LV_ERR_ARG, "lv_model_upload: head size %u (32, 64 and 128 are built)", hp->rot);
+    HIP_TRY(hipSetDevice(c->device));
+
+    // the tensors the decode path reads, in arena order
+    std::vector<Want> wants;
+    wants.push_back({"tok_embeddings", V, D, false});
+    wants.push_back({"norm", D, 1, false});
+    wants.push_back({"output", V, D, true});
+    static const char *mats[7] = {"attention.wq", "attention.wk", "attention.wv", "attention.wo",
+                                  "feed_forward.w1", "feed_forward.w2", "feed_forward.w3"};
+    for (uint32_t i = 0; i < L; i++) {
+        const std::string p = "layers." + std::to_string(i) + ".";
+        for (int k = 0; k < 7; k++) {
+            uint32_t rows = D, cols = D;
+            if (k == 4 || k == 6) rows = F;
+            if (k == 5) cols = F;
+            wants.push_back({p + mats[k], rows, cols, true});
+        }
+        wants.push_back({p + "attention_norm", D, 1, false});
+        wants.push_back({p + "ffn_norm", D, 1, false});
+    }
+
+    uint64_t arena_bytes = 0, staging_bytes = 0;
+    for (Want &w : wants) {
+        w.desc = find_desc(table, n_tensors, w.name);
+        if (!w.desc) return fail(LV_ERR_MISSING, "lv_model_upload: tensor %s is not in the table", w.name.c_str());
+        const lv_tensor_desc &d = *w.desc;
+        if (d.rows != w.rows || d.cols != w.cols)
+            return fail(LV_ERR_ARG, "lv_model_upload: %s is %u x %u, expected %u x %u", d.name, d.rows, d.cols, w.rows, w.cols);
+        const uint64_t raw = ggml_bytes(d.ftype, (uint64_t)d.rows * d.cols);
+        if (raw == 0 || d.size != raw || d.offset + raw > base_size)
+            return fail(LV_ERR_ARG, "lv_model_upload: %s has type %u / %llu bytes at %llu (file holds %llu)", d.name, d.ftype,
+                        (unsigned long long)d.size, (unsigned long long)d.offset, (unsigned long long)base_size);
+        const bool is_quant = d.ftype == LV_Q4_0 || d.ftype == LV_Q8_0;
+        if (w.quant || (is_quant && w.cols > 1)) {
+            LV_TRY(check_quant_shape(d.name, d.ftype, hp->file_version, d.rows, d.cols));
+            w.arena_off = arena_bytes;
+            arena_bytes += matrix_device_bytes(d.ftype, d.rows, d.cols);
+            if (raw > staging_bytes) staging_bytes = raw;
+        } else {
+            if (d.ftype != LV_F32) return fail(LV_ERR_ARG, "lv_model_upload: %s must be f32 (type %u)", d.name, d.ftype);
+            w.arena_off = arena_bytes;
+            arena_bytes += align_up(raw, 256);
+        }
+    }
+
+    lv_model *m = new (std::nothrow) lv_model;
+    if (!m) return fail(LV_ERR_OOM, "lv_model_upload: host allocation");
+    m->ctx = c;
+    m->hp = *hp;
+    m->layers.resize(L);
+    uint8_t *staging = nullptr;
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&m->arena), arena_bytes);
+    if (e == hipSuccess && staging_bytes) e = hipMalloc(reinterpret_cast<void **>(&staging), staging_bytes);
+    if (e != hipSuccess) {
+        (void)hipFree(m->arena);
+        delete m;
+        return fail(e == hipErrorOutOfMemory ? LV_ERR_OOM : LV_ERR_HIP, "lv_model_upload: arena of %llu bytes: %s",
+                    (unsigned long long)arena_bytes, hipGetErrorString(e));
+    }
+    m->arena_bytes = arena_bytes;
+
+    int rc = LV_OK;
+    const uint8_t *hb = static_cast<const uint8_t *>(base);
+    auto put_matrix = [&](const Want &w, lv_matrix *dst) {
+        return place_matrix(c, dst, m->arena + w.arena_off, hb + w.desc->offset, w.desc->ftype, w.desc->rows, w.desc->cols, staging);
+    };
+    auto put_f32 = [&](const Want &w, const float **dst) -> int {
+        HIP_TRY(hipMemcpyAsync(m->arena + w.arena_off, hb + w.desc->offset, w.desc->size, hipMemcpyHostToDevice, c->stream));
+        HIP_TRY(hipStreamSynchronize(c->stream));
+        *dst = reinterpret_cast<const float *>(m->arena + w.arena_off);
+        return LV_OK;
+    };
+    size_t wi = 0;
+    {
+        const Want &tok = wants[wi++];
+        m->tok_ftype = tok.desc->ftype;
+        if (m->tok_ftype == LV_F32) rc = put_f32(tok, &m->tok_f32);
+        else rc = put_matrix(tok, &m->tok_quant);
+    }
+    if (rc == LV_OK) rc = put_f32(wants[wi++], &m->norm);
+    if (rc == LV_OK) rc = put_matrix(wants[wi++], &m->output);
+    for (uint32_t i = 0; i < L && rc == LV_OK; i++) {
+        LayerWeights &lw = m->layers[i];
+        lv_matrix *dsts[7] = {&lw.wq, &lw.wk, &lw.wv, &lw.wo, &lw.w1, &lw.w2, &lw.w3};
+        for (int k = 0; k < 7 && rc == LV_OK; k++) rc = put_matrix(wants[wi++], dsts[k]);
+        if (rc == LV_OK) rc = put_f32(wants[wi++], &lw.attn_norm);
+        if (rc == LV_OK) rc = put_f32(wants[wi++], &lw.ffn_norm);
+        if (rc == LV_OK && (lw.w1.ftype != lw.w3.ftype)) rc = fail(LV_ERR_ARG, "lv_model_upload: layer %u w1/w3 types differ", i);
+    }
+    (void)hipFree(staging);
+    if (rc != LV_OK) {
+        (void)hipFree(m->arena);
+        delete m;
+        return rc;
+    }
+    *out = m;
+    return LV_OK;
+}
+
+extern "C" int lv_model_destroy(lv_model *m)
+{
+    if (!m) return LV_OK;
+    (void)hipSetDevice(m->ctx->device);
+    (void)hipFree(m->arena);
+    delete m;
+    return LV_OK;
+}
+
+extern "C" int lv_model_hparams(const lv_model *m, lv_hparams *out)
+{
+    if (!m || !out) return fail(LV_ERR_ARG, "lv_model_hparams: null argument");
+    *out = m->hp;
+    return LV_OK;
+}
+
+extern "C" int lv_model_arena_bytes(const lv_model *m, uint64_t *bytes)
+{
+    if (!m || !bytes) return fail(LV_ERR_ARG, "lv_model_arena_bytes: null argument");
+    *bytes = m->arena_bytes;
+    return LV_OK;
+}
+
+// -----------------------------------------------------------------------------------------------------------
+// session
+// -----------------------------------------------------------------------------------------------------------
+static void drop_graph(lv_session *s)
+{
+    if (s->graph_exec) (void)hipGraphExecDestroy(s->graph_exec);
+    if (s->graph) (void)hipGraphDestroy(s->graph);
+    s->graph_exec = nullptr;
+    s->graph = nullptr;
+}
+
+extern "C" int lv_session_destroy(lv_session *s)
+{
+    if (!s) return LV_OK;
+    (void)hipSetDevice(s->model->ctx->device);
+    if (s->stream) (void)hipStreamSynchronize(s->stream);
+    drop_graph(s);
+    void *dev[] = {s->kv, s->trig, s->x, s->xn, s->q, s->k, s->v, s->vo, s->ff, s->logits, s->attn_part, s->attn_counters,
+                   s->cfg, s->argmax_dev, s->trace_buf};
+    for (void *p : dev) (void)hipFree(p);
+    if (s->cfg_host) (void)hipHostFree(s->cfg_host);
+    if (s->argmax_host) (void)hipHostFree(s->argmax_host);
+    if (s->stream) (void)hipStreamDestroy(s->stream);
+    delete s;
+    return LV_OK;
+}
+
+static int session_alloc(lv_session *s)
+{
+    const lv_hparams &hp = s->model->hp;
+    const size_t D = hp.dim, F = hp.ff, V = hp.vocab;
+    HIP_TRY(hipStreamCreateWithFlags(&s->stream, hipStreamNonBlocking));
+    HIP_TRY(hipMalloc(reinterpret_cast<void **>(&s->x), D * 4));
+    HIP_TRY(hipMalloc(reinterpret_cast<void **>(&s->xn), D * 4));
+    HIP_TRY(hipMalloc(reinterpret_cast<void **>(&s->q), D * 4));
+    HIP_TRY(hipMalloc(reinterpret_cast<void **>(&s->k), D * 4));
+    HIP_TRY(hipMalloc(reinterpret_cast<void **>(&s->v), D * 4));
+    HIP_TRY(hipMalloc(reinterpret_cast<void **>(&s->vo), D * 4));
+    HIP_TRY(hipMalloc(reinterpret_cast<void **>(&s->ff), F * 4));
+    HIP_TRY(hipMalloc(reinterpret_cast<void **>(&s->logits), V * 4));
+    HIP_TRY(hipMalloc(reinterpret_cast<void **>(&s->cfg), (1 + kMaxStepTokens) * 4));
+    HIP_TRY(hipMalloc(reinterpret_cast<void **>(&s->argmax_dev), 4));
+    HIP_TRY(hipHostMalloc(reinterpret_cast<void **>(&s->cfg_host), (1 + kMaxStepTokens) * 4, hipHostMallocDefault));
+    HIP_TRY(hipHostMalloc(reinterpret_cast<void **>(&s->argmax_host), 4, hipHostMallocDefault));
+    return LV_OK;
+}
+
+extern "C" int lv_session_create(lv_model *m, lv_session **out)
+{
+    if (!m || !out) return fail(LV_ERR_ARG, "lv_session_create: null argument");
+    *out = nullptr;
+    HIP_TRY(hipSetDevice(m->ctx->device));
+    lv_session *s = new (std::nothrow) lv_session;
+    if (!s) return fail(LV_ERR_OOM, "lv_session_create: host allocation");
+    s->model = m;
+    int rc = session_alloc(s);
+    if (rc != LV_OK) {
+        lv_session_destroy(s);
+        return rc;
+    }
+    *out = s;
+    return LV_OK;
+}
+
+extern "C" int lv_session_reserve(lv_session *s, uint32_t backlog)
+{
+    if (!s) return fail(LV_ERR_ARG, "lv_session_reserve: session is null");
+    if (backlog == 0 || backlog > (1u << 20)) return fail(LV_ERR_RANGE, "lv_session_reserve: backlog %u", backlog);
+    if (s->in_flight) return fail(LV_ERR_STATE, "lv_session_reserve: a step is in flight");
+    if (backlog == s->backlog) return LV_OK;
+    const lv_hparams &hp = s->model->hp;
+    HIP_TRY(hipSetDevice(s->model->ctx->device));
+    HIP_TRY(hipStreamSynchronize(s->stream));
+    drop_graph(s);
+
+    const size_t D = hp.dim, plane_new = (size_t)backlog * D, plane_old = (size_t)s->backlog * D;
+    uint16_t *kv_new = nullptr;
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&kv_new), (size_t)hp.layers * 2 * plane_new * 2);
+    if (e != hipSuccess)
+        return fail(e == hipErrorOutOfMemory ? LV_ERR_OOM : LV_ERR_HIP, "lv_session_reserve: cache of %u rows: %s", backlog, hipGetErrorString(e));
+    // keep the first min(old, new) rows of every plane, zero the rest (llava_layer_session_data.cpp:100-112)
+    const size_t keep_rows = s->backlog < backlog ? s->backlog : backlog;
+    int rc = zero_async(kv_new, (size_t)hp.layers * 2 * plane_new * 2, s->stream);
+    for (uint32_t pl = 0; pl < hp.layers * 2 && rc == LV_OK && keep_rows; pl++) {
+        hipError_t ce = hipMemcpyAsync(kv_new + pl * plane_new, s->kv + pl * plane_old, keep_rows * D * 2, hipMemcpyDeviceToDevice, s->stream);
+        if (ce != hipSuccess) rc = fail(LV_ERR_HIP, "lv_session_reserve: copy: %s", hipGetErrorString(ce));
+    }
+    if (rc == LV_OK && hipStreamSynchronize(s->stream) != hipSuccess) rc = fail(LV_ERR_HIP, "lv_session_reserve: sync failed");
+    if (rc != LV_OK) {
+        (void)hipFree(kv_new);
+        return rc;
+    }
+    (void)hipFree(s->kv);
+    s->kv = kv_new;
+
+    (void)hipFree(s->trig);
+    s->trig = nullptr;
+    (void)hipFree(s->attn_part);
+    s->attn_part = nullptr;
+    (void)hipFree(s->attn_counters);
+    s->attn_counters = nullptr;
+    s->backlog = 0;
+    LV_TRY(upload_trig(&s->trig, backlog, hp.rot, s->stream));
+    const uint32_t splits = (backlog + kAttnChunk - 1) / kAttnChunk;
+    HIP_TRY(hipMalloc(reinterpret_cast<void **>(&s->attn_part), attn_part_floats(1, hp.heads, splits, hp.rot) * sizeof(float)));
+    HIP_TRY(hipMalloc(reinterpret_cast<void **>(&s->attn_counters), (size_t)hp.heads * 4));
+    LV_TRY(zero_async(s->attn_counters, (size_t)hp.heads * 4, s->stream));
+    HIP_TRY(hipStreamSynchronize(s->stream));
+    s->backlog = backlog;
+    return LV_OK;
+}
+
+extern "C" int lv_session_backlog(const lv_session *s, uint32_t *backlog)
+{
+    if (!s || !backlog) return fail(LV_ERR_ARG, "lv_session_backlog: null argument");
+    *backlog = s->backlog;
+    return LV_OK;
+}
+
+extern "C" int lv_session_use_graph(lv_session *s, int enable)
+{
+    if (!s) return fail(LV_ERR_ARG, "lv_session_use_graph: session is null");
+    s->use_graph = enable != 0;
+    return LV_OK;
+}
+
+// -----------------------------------------------------------------------------------------------------------
+// the step
+// -----------------------------------------------------------------------------------------------------------
+static int trace_copy(lv_session *s, uint32_t layer, int which, const float *src, size_t count)
+{
+    if (!s->trace) return LV_OK;
+    const lv_hparams &hp = s->model->hp;
+    const size_t slot = hp.dim > hp.ff ? hp.dim : hp.ff;
+    float *dst = s->trace_buf + ((size_t)layer * LV_TRACE_COUNT + which) * slot;
+    HIP_TRY(hipMemcpyAsync(dst, src, count * 4, hipMemcpyDeviceToDevice, s->stream));
+    return LV_OK;
+}
+
+// One token through every layer (llava_layer.cpp:53-73 + llava_command_buffer.cpp:38-39).  The token id is
+// cfg[1 + idx], its cache row cfg[0] + idx.  With_head = also compute the logits.
+static int record_token(lv_session *s, uint32_t idx, bool with_head)
+{
+    const lv_model *m = s->model;
+    const lv_hparams &hp = m->hp;
+    const uint32_t D = hp.dim, F = hp.ff;
+    hipStream_t st = s->stream;
+    const uint32_t *pos_ptr = s->cfg, *tok_ptr = s->cfg + 1 + idx;
+
+    if (m->tok_ftype == LV_F32)
+        embed_f32_kernel<<<dim3((D + 255) / 256, 1), dim3(256), 0, st>>>(s->x, m->tok_f32, tok_ptr, D);
+    else if (m->tok_ftype == LV_Q4_0)
+        embed_quant_kernel<4><<<dim3((D / 32 + 63) / 64, 1), dim3(64), 0, st>>>(s->x, m->tok_quant.view, tok_ptr);
+    else
+        embed_quant_kernel<8><<<dim3((D / 32 + 63) / 64, 1), dim3(64), 0, st>>>(s->x, m->tok_quant.view, tok_ptr);
+    HIP_TRY(hipGetLastError());
+
+    const dim3 kv_grid((D + 255) / 256, 1);
+    for (uint32_t li = 0; li < hp.layers; li++) {
+        const LayerWeights &lw = m->layers[li];
+        normalize_kernel<<<dim3(1), dim3(256), 0, st>>>(s->xn, s->x, lw.attn_norm, D);
+        HIP_TRY(hipGetLastError());
+        LV_TRY(trace_copy(s, li, LV_TRACE_NORM_IN, s->xn, D));
+        LV_TRY(launch_gemv(st, s->k, lw.wk, nullptr, s->xn, 1, kGemvStore));
+        LV_TRY(launch_gemv(st, s->q, lw.wq, nullptr, s->xn, 1, kGemvStore));
+        LV_TRY(launch_gemv(st, s->v, lw.wv, nullptr, s->xn, 1, kGemvStore));
+        kv_append_kernel<<<kv_grid, dim3(256), 0, st>>>(kv_ptr(s, li, 0), s->k, pos_ptr, idx, D, s->backlog);
+        kv_append_kernel<<<kv_grid, dim3(256), 0, st>>>(kv_ptr(s, li, 1), s->v, pos_ptr, idx, D, s->backlog);
+        HIP_TRY(hipGetLastError());
+        LV_TRY(launch_attention(st, s->vo, kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->q, s->trig, s->attn_part, s->attn_counters,
+                                pos_ptr, idx, s->backlog, hp.heads, hp.rot, 1));
+        LV_TRY(launch_gemv(st, s->x, lw.wo, nullptr, s->vo, 1, kGemvAdd));
+        LV_TRY(trace_copy(s, li, LV_TRACE_POST_ATTN, s->x, D));
+        normalize_kernel<<<dim3(1), dim3(256), 0, st>>>(s->xn, s->x, lw.ffn_norm, D);
+        HIP_TRY(hipGetLastError());
+        LV_TRY(trace_copy(s, li, LV_TRACE_POST_ATTN_NORM, s->xn, D));
+        LV_TRY(launch_gemv(st, s->ff, lw.w3, &lw.w1, s->xn, 1, kGemvSilu));
+        LV_TRY(trace_copy(s, li, LV_TRACE_FF, s->ff, F));
+        LV_TRY(launch_gemv(st, s->x, lw.w2, nullptr, s->ff, 1, kGemvAdd));
+        LV_TRY(trace_copy(s, li, LV_TRACE_OUT, s->x, D));
+    }
+    if (with_head) {
+        normalize_kernel<<<dim3(1), dim3(256), 0, st>>>(s->xn, s->x, m->norm, D);
+        HIP_TRY(hipGetLastError());
+        LV_TRY(launch_gemv(st, s->logits, m->output, nullptr, s->xn, 1, kGemvStore));
+    }
+    return LV_OK;
+}
+
+extern "C" int lv_step_begin(lv_session *s, const uint32_t *tokens, uint32_t n, uint32_t pos)
+{
+    if (!s || !tokens) return fail(LV_ERR_ARG, "lv_step_begin: null argument");
+    if (s->in_flight) return fail(LV_ERR_STATE, "lv_step_begin: the previous step has not been waited for");
+    if (n == 0) return fail(LV_ERR_ARG, "lv_step_begin: no tokens");
+    if (n > kMaxStepTokens) return fail(LV_ERR_RANGE, "lv_step_begin: %u tokens in one step (limit %u)", n, kMaxStepTokens);
+    if (s->backlog == 0) return fail(LV_ERR_STATE, "lv_step_begin: lv_session_reserve has not been called");
+    if ((uint64_t)pos + n > s->backlog)
+        return fail(LV_ERR_RANGE, "lv_step_begin: rows %u..%u exceed the backlog of %u", pos, pos + n - 1, s->backlog);
+    for (uint32_t i = 0; i < n; i++)
+        if (tokens[i] >= s->model->hp.vocab) return fail(LV_ERR_RANGE, "lv_step_begin: token id %u of a vocabulary of %u", tokens[i], s->model->hp.vocab);
+    HIP_TRY(hipSetDevice(s->model->ctx->device));
+
+    s->cfg_host[0] = pos;
+    memcpy(s->cfg_host + 1, tokens, (size_t)n * 4);
+    HIP_TRY(hipMemcpyAsync(s->cfg, s->cfg_host, (size_t)(1 + n) * 4, hipMemcpyHostToDevice, s->stream));
+    s->have_logits = false;
+
+    if (n == 1 && s->use_graph && !s->trace) {
+        if (!s->graph_exec) {
+            HIP_TRY(hipStreamBeginCapture(s->stream, hipStreamCaptureModeThreadLocal));
+            int rc = record_token(s, 0, true);
+            hipGraph_t g = nullptr;
+            hipError_t e = hipStreamEndCapture(s->stream, &g);
+            if (rc != LV_OK) {
+                if (g) (void)hipGraphDestroy(g);
+                return rc;
+            }
+            HIP_TRY(e);
+            s->graph = g;
+            HIP_TRY(hipGraphInstantiate(&s->graph_exec, s->graph, nullptr, nullptr, 0));
+        }
+        HIP_TRY(hipGraphLaunch(s->graph_exec, s->stream));
+    } else {
+        // rows are evaluated one after the other: row z sees cache rows 0..pos+z, which is what the batched
+        // shaders compute (every row's K/V is appended before any row attends, and rows above are masked)
+        for (uint32_t i = 0; i < n; i++) LV_TRY(record_token(s, i, i + 1 == n));
+    }
+    s->in_flight = true;
+    s->have_logits = true;
+    return LV_OK;
+}
+
+extern "C" int lv_step_wait(lv_session *s)
+{
+    if (!s) return fail(LV_ERR_ARG, "lv_step_wait: session is null");
+    HIP_TRY(hipStreamSynchronize(s->stream));
+    s->in_flight = false;
+    return LV_OK;
+}
+
+extern "C" int lv_logits_read(lv_session *s, float *dst)
+{
+    if (!s || !dst) return fail(LV_ERR_ARG, "lv_logits_read: null argument");
+    if (!s->have_logits) return fail(LV_ERR_STATE, "lv_logits_read: no step has produced logits");
+    HIP_TRY(hipMemcpyAsync(dst, s->logits, (size_t)s->model->hp.vocab * 4, hipMemcpyDeviceToHost, s->stream));
+    return lv_step_wait(s);
+}
+
+extern "C" int lv_argmax(lv_session *s, uint32_t *token)
+{
+    if (!s || !token) return fail(LV_ERR_ARG, "lv_argmax: null argument");
+    if (!s->have_logits) return fail(LV_ERR_STATE, "lv_argmax: no step has produced logits");
+    argmax_kernel<<<dim3(1), dim3(1024), 0, s->stream>>>(s->logits, s->model->hp.vocab, s->argmax_dev);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipMemcpyAsync(s->argmax_host, s->argmax_dev, 4, hipMemcpyDeviceToHost, s->stream));
+    LV_TRY(lv_step_wait(s));
+    *token = *s->argmax_host;
+    return LV_OK;
+}
+
+// -----------------------------------------------------------------------------------------------------------
+// cache dump / restore, trace
+// -----------------------------------------------------------------------------------------------------------
+static int kv_args(const char *who, lv_session *s, uint32_t layer, uint32_t n_tokens, const void *p)
+{
+    if (!s || (n_tokens && !p)) return fail(LV_ERR_ARG, "%s: null argument", who);
+    if (layer >= s->model->hp.layers) return fail(LV_ERR_RANGE, "%s: layer %u of %u", who, layer, s->model->hp.layers);
+    if (n_tokens > s->backlog) return fail(LV_ERR_RANGE, "%s: %u rows of a backlog of %u", who, n_tokens, s->backlog);
+    if (s->in_flight) return fail(LV_ERR_STATE, "%s: a step is in flight", who);
+    return LV_OK;
+}
+
+extern "C" int lv_kv_read(lv_session *s, uint32_t layer, int which, uint32_t n_tokens, void *dst)
+{
+    LV_TRY(kv_args("lv_kv_read", s, layer, n_tokens, dst));
+    if (n_tokens == 0) return LV_OK;
+    HIP_TRY(hipMemcpyAsync(dst, kv_ptr(s, layer, which), (size_t)n_tokens * s->model->hp.dim * 2, hipMemcpyDeviceToHost, s->stream));
+    HIP_TRY(hipStreamSynchronize(s->stream));
+    return LV_OK;
+}
+
+extern "C" int lv_kv_write(lv_session *s, uint32_t layer, int which, uint32_t n_tokens, const void *src)
+{
+    LV_TRY(kv_args("lv_kv_write", s, layer, n_tokens, src));
+    if (n_tokens == 0) return LV_OK;
+    HIP_TRY(hipMemcpyAsync(kv_ptr(s, layer, which), src, (size_t)n_tokens * s->model->hp.dim * 2, hipMemcpyHostToDevice, s->stream));
+    HIP_TRY(hipStreamSynchronize(s->stream));
+    return LV_OK;
+}
+
+extern "C" int lv_trace_enable(lv_session *s, int enable)
+{
+    if (!s) return fail(LV_ERR_ARG, "lv_trace_enable: session is null");
+    if (s->in_flight) return fail(LV_ERR_STATE, "lv_trace_enable: a step is in flight");
+    const lv_hparams &hp = s->model->hp;
+    if (enable && !s->trace_buf) {
+        const size_t slot = hp.dim > hp.ff ? hp.dim : hp.ff;
+        HIP_TRY(hipSetDevice(s->model->ctx->device));
+        HIP_TRY(hipMalloc(reinterpret_cast<void **>(&s->trace_buf), (size_t)hp.layers * LV_TRACE_COUNT * slot * 4));
+    }
+    s->trace = enable != 0;
+    return LV_OK;
+}
+
+extern "C" int lv_trace_read(lv_session *s, uint32_t layer, int which, float *dst, uint32_t count)
+{
+    if (!s || !dst) return fail(LV_ERR_ARG, "lv_trace_read: null argument");
+    if (!s->trace || !s->trace_buf) return fail(LV_ERR_STATE, "lv_trace_read: record mode is off");
+    const lv_hparams &hp = s->model->hp;
+    if (layer >= hp.layers || which < 0 || which >= LV_TRACE_COUNT) return fail(LV_ERR_RANGE, "lv_trace_read: layer %u / buffer %d", layer, which);
+    const uint32_t have = which == LV_TRACE_FF ? hp.ff : hp.dim;
+    if (count != have) return fail(LV_ERR_ARG, "lv_trace_read: buffer %d holds %u floats, %u asked", which, have, count);
+    const size_t slot = hp.dim > hp.ff ? hp.dim : hp.ff;
+    HIP_TRY(hipMemcpyAsync(dst, s->trace_buf + ((size_t)layer * LV_TRACE_COUNT + which) * slot, (size_t)count * 4, hipMemcpyDeviceToHost, s->stream));
+    HIP_TRY(hipStreamSynchronize(s->stream));
+    s->in_flight = false;
+    return LV_OK;
+}
