@@ -101,6 +101,15 @@ int lv_logits_read(lv_session *s, float *dst);
 int lv_argmax(lv_session *s, uint32_t *token);
 /* Enables/disables hipGraph replay for n == 1 steps (on by default); off = plain stream launches. */
 int lv_session_use_graph(lv_session *s, int enable);
+/* How n == 1 steps are executed.  The reference has one way (replay the recorded command buffers,
+ * llava_command_buffer.cpp:47-55); here there are three, all computing the same step:
+ *   LV_PATH_KERNELS     one launch per operator on the session's stream
+ *   LV_PATH_GRAPH       the same launches captured once into a hipGraph and replayed
+ *   LV_PATH_PERSISTENT  one persistent kernel for the whole token (7B-class q4_0 models on a 256-CU device)
+ *   LV_PATH_AUTO        persistent when the model has that form, else graph (or kernels if graphs are off) */
+enum { LV_PATH_AUTO = 0, LV_PATH_KERNELS = 1, LV_PATH_GRAPH = 2, LV_PATH_PERSISTENT = 3 };
+int lv_session_set_path(lv_session *s, int path);
+int lv_session_path(const lv_session *s, int *path);
 
 /* ---- cache dump / restore: replaces llava_layer_session_data::dump_kv_cache / restore_kv_cache
  *      (llava_layer_session_data.cpp:165-181).  which: 0 = K, 1 = V.  n_tokens rows of `dim` fp16 values. */
@@ -128,6 +137,13 @@ int lv_dev_upload(lv_ctx *ctx, void *dptr, const void *src, uint64_t bytes);
 int lv_dev_download(lv_ctx *ctx, void *dst, const void *dptr, uint64_t bytes);
 int lv_dev_zero(lv_ctx *ctx, void *dptr, uint64_t bytes);
 int lv_ctx_sync(lv_ctx *ctx);
+
+/* ---- GPU time between two points of a stream, by HIP events recorded on that very stream (the reference has
+ *      no timers at all; benchmarks need them).  stop waits for the stream and returns milliseconds. ------- */
+int lv_ctx_timer_start(lv_ctx *ctx);
+int lv_ctx_timer_stop(lv_ctx *ctx, float *ms);
+int lv_session_timer_start(lv_session *s);
+int lv_session_timer_stop(lv_session *s, float *ms);
 
 /* A quantised matrix in the device layout.  Built from GGML blocks by lv_matrix_upload; owns its memory. */
 typedef struct lv_matrix lv_matrix;

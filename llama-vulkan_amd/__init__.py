@@ -20,6 +20,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 ROOT_DIR = os.path.dirname(PKG_DIR)
 
 LV_F32, LV_F16, LV_Q4_0, LV_Q8_0 = 0, 1, 2, 8
+PATH_AUTO, PATH_KERNELS, PATH_GRAPH, PATH_PERSISTENT = range(4)
 TRACE_NORM_IN, TRACE_POST_ATTN, TRACE_POST_ATTN_NORM, TRACE_FF, TRACE_OUT = range(5)
 
 
@@ -76,6 +77,10 @@ _HIP_SIGS = {
     "lv_ctx_destroy": [_VP],
     "lv_ctx_info": [_VP, C.c_char_p, C.c_size_t, C.POINTER(_U32), C.POINTER(_U64)],
     "lv_ctx_sync": [_VP],
+    "lv_ctx_timer_start": [_VP],
+    "lv_ctx_timer_stop": [_VP, C.POINTER(C.c_float)],
+    "lv_session_timer_start": [_VP],
+    "lv_session_timer_stop": [_VP, C.POINTER(C.c_float)],
     "lv_model_upload": [_VP, _VP, _U64, C.POINTER(HParams), C.POINTER(TensorDesc), _U32, C.POINTER(_VP)],
     "lv_model_destroy": [_VP],
     "lv_model_hparams": [_VP, C.POINTER(HParams)],
@@ -85,6 +90,8 @@ _HIP_SIGS = {
     "lv_session_reserve": [_VP, _U32],
     "lv_session_backlog": [_VP, C.POINTER(_U32)],
     "lv_session_use_graph": [_VP, _I],
+    "lv_session_set_path": [_VP, _I],
+    "lv_session_path": [_VP, C.POINTER(_I)],
     "lv_step_begin": [_VP, _VP, _U32, _U32],
     "lv_step_wait": [_VP],
     "lv_logits_read": [_VP, _VP],
@@ -153,6 +160,14 @@ class Context:
 
     def sync(self):
         check(self.lib.lv_ctx_sync(self.h))
+
+    def timer_start(self):
+        check(self.lib.lv_ctx_timer_start(self.h))
+
+    def timer_stop(self):
+        ms = C.c_float()
+        check(self.lib.lv_ctx_timer_stop(self.h, C.byref(ms)))
+        return ms.value
 
     def alloc(self, nbytes):
         p = C.c_void_p()
@@ -332,12 +347,28 @@ class Session:
     def use_graph(self, on):
         check(self.lib.lv_session_use_graph(self.h, int(on)))
 
+    def set_path(self, path):
+        check(self.lib.lv_session_set_path(self.h, int(path)))
+
+    def path(self):
+        p = C.c_int()
+        check(self.lib.lv_session_path(self.h, C.byref(p)))
+        return p.value
+
     def begin(self, tokens, pos):
         t = np.ascontiguousarray(tokens, dtype=np.uint32)
         check(self.lib.lv_step_begin(self.h, _ptr(t), t.shape[0], pos))
 
     def wait(self):
         check(self.lib.lv_step_wait(self.h))
+
+    def timer_start(self):
+        check(self.lib.lv_session_timer_start(self.h))
+
+    def timer_stop(self):
+        ms = C.c_float()
+        check(self.lib.lv_session_timer_stop(self.h, C.byref(ms)))
+        return ms.value
 
     def logits(self):
         out = np.empty(self.model.header["vocab"], dtype=np.float32)

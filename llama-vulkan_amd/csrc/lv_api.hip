@@ -18,6 +18,7 @@
 #include <vector>
 
 #include "lv_kernels.h"
+#include "lv_mega.h"
 
 using namespace lv;
 
@@ -63,6 +64,7 @@ struct lv_ctx {
     float *attn_part = nullptr;
     uint32_t *attn_counters = nullptr;
     size_t attn_part_floats = 0, attn_counter_words = 0;
+    hipEvent_t ev_start = nullptr, ev_stop = nullptr;
 };
 
 struct lv_matrix {
@@ -89,7 +91,13 @@ struct lv_model {
     uint32_t tok_ftype = LV_F32;
     const float *tok_f32 = nullptr;
     lv_matrix tok_quant;
+    // persistent-kernel form of the weights (null when the model's shape has no compiled MegaShape)
+    int mega_kind = 0;              // 0 none, 1 = 7B class (4096/11008/32 heads)
+    uint8_t *mega_stream = nullptr;
+    float *mega_norms = nullptr;    // [layers][2][D] + final norm [D]
 };
+
+using Mega7B = MegaShape<4096, 11008, 32, 12>;
 
 constexpr uint32_t kAttnChunk = 64;   // cache positions per attention workgroup
 constexpr uint32_t kMaxStepTokens = 4096;
@@ -112,10 +120,15 @@ struct lv_session {
     hipGraph_t graph = nullptr;
     hipGraphExec_t graph_exec = nullptr;
     bool use_graph = true;
+    int path = LV_PATH_AUTO;
+    float *xchg[2] = {nullptr, nullptr};  // hand-over buffer sets of the persistent kernel
+    uint32_t xchg_turn = 0;
+    uint32_t *status_host = nullptr;      // pinned, written by the persistent kernel when a poll expires
     bool in_flight = false;
     bool have_logits = false;
     bool trace = false;
     float *trace_buf = nullptr;  // [layers][LV_TRACE_COUNT][max(dim, ff)]
+    hipEvent_t ev_start = nullptr, ev_stop = nullptr;
 };
 
 static uint16_t *kv_ptr(const lv_session *s, uint32_t layer, int which)
@@ -156,6 +169,8 @@ extern "C" int lv_ctx_destroy(lv_ctx *c)
     (void)hipFree(c->trig);
     (void)hipFree(c->attn_part);
     (void)hipFree(c->attn_counters);
+    if (c->ev_start) (void)hipEventDestroy(c->ev_start);
+    if (c->ev_stop) (void)hipEventDestroy(c->ev_stop);
     (void)hipStreamDestroy(c->stream);
     delete c;
     return LV_OK;
@@ -175,6 +190,36 @@ extern "C" int lv_ctx_sync(lv_ctx *c)
     if (!c) return fail(LV_ERR_ARG, "lv_ctx_sync: ctx is null");
     HIP_TRY(hipStreamSynchronize(c->stream));
     return LV_OK;
+}
+
+// ---- stream timers ---------------------------------------------------------------------------------------
+static int timer_start(hipEvent_t *a, hipEvent_t *b, hipStream_t st)
+{
+    if (!*a) HIP_TRY(hipEventCreate(a));
+    if (!*b) HIP_TRY(hipEventCreate(b));
+    HIP_TRY(hipEventRecord(*a, st));
+    return LV_OK;
+}
+
+static int timer_stop(hipEvent_t a, hipEvent_t b, hipStream_t st, float *ms)
+{
+    if (!a || !b) return fail(LV_ERR_STATE, "timer stop without start");
+    HIP_TRY(hipEventRecord(b, st));
+    HIP_TRY(hipEventSynchronize(b));
+    HIP_TRY(hipEventElapsedTime(ms, a, b));
+    return LV_OK;
+}
+
+extern "C" int lv_ctx_timer_start(lv_ctx *c)
+{
+    if (!c) return fail(LV_ERR_ARG, "lv_ctx_timer_start: ctx is null");
+    return timer_start(&c->ev_start, &c->ev_stop, c->stream);
+}
+
+extern "C" int lv_ctx_timer_stop(lv_ctx *c, float *ms)
+{
+    if (!c || !ms) return fail(LV_ERR_ARG, "lv_ctx_timer_stop: null argument");
+    return timer_stop(c->ev_start, c->ev_stop, c->stream, ms);
 }
 
 extern "C" int lv_dev_alloc(lv_ctx *c, uint64_t bytes, void **dptr)
@@ -541,6 +586,60 @@ static const lv_tensor_desc *find_desc(const lv_tensor_desc *t, uint32_t n, cons
     return nullptr;
 }
 
+// Persistent-kernel form of the weights: a second copy laid out as per-wave tile streams (lv_mega.h).
+// Built when the model has a compiled shape class, all matrices are q4_0 and the embeddings fp32.
+template <class S>
+static int build_mega_stream(lv_model *m)
+{
+    lv_ctx *c = m->ctx;
+    const uint32_t L = m->hp.layers, D = m->hp.dim;
+    const size_t total = (size_t)L * S::LAYER_BYTES + S::HEAD_BYTES + kMegaTile;  // + the all-zero dummy tile
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&m->mega_stream), total);
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&m->mega_norms), ((size_t)L * 2 + 1) * D * 4);
+    if (e != hipSuccess)
+        return fail(e == hipErrorOutOfMemory ? LV_ERR_OOM : LV_ERR_HIP, "persistent weight stream of %llu bytes: %s",
+                    (unsigned long long)total, hipGetErrorString(e));
+    auto pack = [&](uint8_t *dst, int phase, int tiles, const MatView &a, const MatView &b, const MatView &cc) -> int {
+        MegaPackSrc src{};
+        src.m[0] = a; src.m[1] = b; src.m[2] = cc;
+        const size_t threads = (size_t)kMegaWGs * S::NW * tiles * 64;
+        mega_pack_kernel<S><<<dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, c->stream>>>(dst, src, phase, m->hp.vocab);
+        HIP_TRY(hipGetLastError());
+        return LV_OK;
+    };
+    const MatView none{};
+    LV_TRY(zero_async(m->mega_stream + (size_t)L * S::LAYER_BYTES + S::HEAD_BYTES, kMegaTile, c->stream));
+    for (uint32_t i = 0; i < L; i++) {
+        const LayerWeights &lw = m->layers[i];
+        uint8_t *base = m->mega_stream + (size_t)i * S::LAYER_BYTES;
+        LV_TRY(pack(base, 0, S::TA, lw.wq.view, lw.wk.view, lw.wv.view));
+        LV_TRY(pack(base + S::PHASE_A_BYTES, 1, S::TC, lw.wo.view, none, none));
+        LV_TRY(pack(base + S::PHASE_A_BYTES + S::PHASE_C_BYTES, 2, S::TD, lw.w3.view, lw.w1.view, none));
+        LV_TRY(pack(base + S::PHASE_A_BYTES + S::PHASE_C_BYTES + S::PHASE_D_BYTES, 3, S::TE, lw.w2.view, none, none));
+        HIP_TRY(hipMemcpyAsync(m->mega_norms + (size_t)i * 2 * D, lw.attn_norm, (size_t)D * 4, hipMemcpyDeviceToDevice, c->stream));
+        HIP_TRY(hipMemcpyAsync(m->mega_norms + ((size_t)i * 2 + 1) * D, lw.ffn_norm, (size_t)D * 4, hipMemcpyDeviceToDevice, c->stream));
+    }
+    LV_TRY(pack(m->mega_stream + (size_t)L * S::LAYER_BYTES, 4, kMegaHeadSlots, m->output.view, none, none));
+    HIP_TRY(hipMemcpyAsync(m->mega_norms + (size_t)L * 2 * D, m->norm, (size_t)D * 4, hipMemcpyDeviceToDevice, c->stream));
+    HIP_TRY(hipStreamSynchronize(c->stream));
+    return LV_OK;
+}
+
+static int build_mega(lv_model *m)
+{
+    const lv_hparams &hp = m->hp;
+    bool all_q4 = m->output.ftype == LV_Q4_0 && m->tok_ftype == LV_F32;
+    for (const LayerWeights &lw : m->layers)
+        for (const lv_matrix *x : {&lw.wq, &lw.wk, &lw.wv, &lw.wo, &lw.w1, &lw.w2, &lw.w3}) all_q4 = all_q4 && x->ftype == LV_Q4_0;
+    if (!all_q4 || (int)m->ctx->props.multiProcessorCount < kMegaWGs) return LV_OK;
+    if (hp.dim == Mega7B::D && hp.ff == Mega7B::F && hp.heads == Mega7B::H &&
+        (hp.vocab + kMegaWGs - 1) / kMegaWGs <= (uint32_t)(kMegaHeadSlots * Mega7B::NRD)) {
+        LV_TRY(build_mega_stream<Mega7B>(m));
+        m->mega_kind = 1;
+    }
+    return LV_OK;
+}
+
 struct Want {
     std::string name;
     uint32_t rows, cols;   // expected shape (cols == 1 for vectors)
@@ -649,7 +748,10 @@ extern "C" int lv_model_upload(lv_ctx *c, const void *base, uint64_t base_size, 
         if (rc == LV_OK && (lw.w1.ftype != lw.w3.ftype)) rc = fail(LV_ERR_ARG, "lv_model_upload: layer %u w1/w3 types differ", i);
     }
     (void)hipFree(staging);
+    if (rc == LV_OK) rc = build_mega(m);
     if (rc != LV_OK) {
+        (void)hipFree(m->mega_stream);
+        (void)hipFree(m->mega_norms);
         (void)hipFree(m->arena);
         delete m;
         return rc;
@@ -662,6 +764,8 @@ extern "C" int lv_model_destroy(lv_model *m)
 {
     if (!m) return LV_OK;
     (void)hipSetDevice(m->ctx->device);
+    (void)hipFree(m->mega_stream);
+    (void)hipFree(m->mega_norms);
     (void)hipFree(m->arena);
     delete m;
     return LV_OK;
@@ -701,8 +805,13 @@ extern "C" int lv_session_destroy(lv_session *s)
     void *dev[] = {s->kv, s->trig, s->x, s->xn, s->q, s->k, s->v, s->vo, s->ff, s->logits, s->attn_part, s->attn_counters,
                    s->cfg, s->argmax_dev, s->trace_buf};
     for (void *p : dev) (void)hipFree(p);
+    (void)hipFree(s->xchg[0]);
+    (void)hipFree(s->xchg[1]);
+    if (s->status_host) (void)hipHostFree(s->status_host);
     if (s->cfg_host) (void)hipHostFree(s->cfg_host);
     if (s->argmax_host) (void)hipHostFree(s->argmax_host);
+    if (s->ev_start) (void)hipEventDestroy(s->ev_start);
+    if (s->ev_stop) (void)hipEventDestroy(s->ev_stop);
     if (s->stream) (void)hipStreamDestroy(s->stream);
     delete s;
     return LV_OK;
@@ -725,6 +834,16 @@ static int session_alloc(lv_session *s)
     HIP_TRY(hipMalloc(reinterpret_cast<void **>(&s->argmax_dev), 4));
     HIP_TRY(hipHostMalloc(reinterpret_cast<void **>(&s->cfg_host), (1 + kMaxStepTokens) * 4, hipHostMallocDefault));
     HIP_TRY(hipHostMalloc(reinterpret_cast<void **>(&s->argmax_host), 4, hipHostMallocDefault));
+    if (s->model->mega_kind == 1) {
+        const size_t bytes = (size_t)hp.layers * Mega7B::XCHG_LAYER * 4;
+        for (int i = 0; i < 2; i++) {
+            HIP_TRY(hipMalloc(reinterpret_cast<void **>(&s->xchg[i]), bytes));
+            HIP_TRY(hipMemsetAsync(s->xchg[i], 0xff, bytes, s->stream));
+        }
+        HIP_TRY(hipHostMalloc(reinterpret_cast<void **>(&s->status_host), 4096, hipHostMallocDefault));
+        memset(s->status_host, 0, 4096);
+        HIP_TRY(hipStreamSynchronize(s->stream));
+    }
     return LV_OK;
 }
 
@@ -804,6 +923,48 @@ extern "C" int lv_session_use_graph(lv_session *s, int enable)
 {
     if (!s) return fail(LV_ERR_ARG, "lv_session_use_graph: session is null");
     s->use_graph = enable != 0;
+    return LV_OK;
+}
+
+extern "C" int lv_session_set_path(lv_session *s, int path)
+{
+    if (!s) return fail(LV_ERR_ARG, "lv_session_set_path: session is null");
+    if (path < LV_PATH_AUTO || path > LV_PATH_PERSISTENT) return fail(LV_ERR_ARG, "lv_session_set_path: path %d", path);
+    if (path == LV_PATH_PERSISTENT && s->model->mega_kind == 0)
+        return fail(LV_ERR_ARG, "lv_session_set_path: this model has no persistent-kernel form (shape or types not covered)");
+    s->path = path;
+    return LV_OK;
+}
+
+extern "C" int lv_session_path(const lv_session *s, int *path)
+{
+    if (!s || !path) return fail(LV_ERR_ARG, "lv_session_path: null argument");
+    *path = s->path != LV_PATH_AUTO ? s->path
+            : s->model->mega_kind   ? LV_PATH_PERSISTENT
+            : s->use_graph          ? LV_PATH_GRAPH
+                                    : LV_PATH_KERNELS;
+    return LV_OK;
+}
+
+// One token through the persistent kernel.
+static int launch_mega(lv_session *s, uint32_t pos, uint32_t token)
+{
+    const lv_model *m = s->model;
+    MegaArgs a{};
+    a.wstream = m->mega_stream;
+    a.norms = m->mega_norms;
+    a.tok_f32 = m->tok_f32;
+    a.kv = s->kv;
+    a.trig = s->trig;
+    a.xchg = s->xchg[s->xchg_turn & 1];
+    a.xchg_rearm = s->xchg[(s->xchg_turn + 1) & 1];
+    a.logits = s->logits;
+    a.status = s->status_host;
+    a.layers = m->hp.layers; a.vocab = m->hp.vocab; a.backlog = s->backlog; a.pos = pos; a.token = token;
+    s->xchg_turn++;
+    void *params[] = {&a};
+    HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<const void *>(&mega_decode_kernel<Mega7B>), dim3(kMegaWGs),
+                                       dim3((Mega7B::NW + kMegaServiceWaves) * 64), params, 0, s->stream));
     return LV_OK;
 }
 
@@ -888,7 +1049,11 @@ extern "C" int lv_step_begin(lv_session *s, const uint32_t *tokens, uint32_t n, 
     HIP_TRY(hipMemcpyAsync(s->cfg, s->cfg_host, (size_t)(1 + n) * 4, hipMemcpyHostToDevice, s->stream));
     s->have_logits = false;
 
-    if (n == 1 && s->use_graph && !s->trace) {
+    int path = LV_PATH_AUTO;
+    (void)lv_session_path(s, &path);
+    if (n == 1 && path == LV_PATH_PERSISTENT && !s->trace) {
+        LV_TRY(launch_mega(s, pos, tokens[0]));
+    } else if (n == 1 && (path == LV_PATH_GRAPH || (path == LV_PATH_PERSISTENT && s->use_graph)) && !s->trace) {
         if (!s->graph_exec) {
             HIP_TRY(hipStreamBeginCapture(s->stream, hipStreamCaptureModeThreadLocal));
             int rc = record_token(s, 0, true);
@@ -918,6 +1083,10 @@ extern "C" int lv_step_wait(lv_session *s)
     if (!s) return fail(LV_ERR_ARG, "lv_step_wait: session is null");
     HIP_TRY(hipStreamSynchronize(s->stream));
     s->in_flight = false;
+    if (s->status_host && *s->status_host) {
+        *s->status_host = 0;
+        return fail(LV_ERR_HIP, "persistent decode kernel: a hand-over wait expired (workgroups not co-resident?)");
+    }
     return LV_OK;
 }
 
@@ -938,6 +1107,20 @@ extern "C" int lv_argmax(lv_session *s, uint32_t *token)
     HIP_TRY(hipMemcpyAsync(s->argmax_host, s->argmax_dev, 4, hipMemcpyDeviceToHost, s->stream));
     LV_TRY(lv_step_wait(s));
     *token = *s->argmax_host;
+    return LV_OK;
+}
+
+extern "C" int lv_session_timer_start(lv_session *s)
+{
+    if (!s) return fail(LV_ERR_ARG, "lv_session_timer_start: session is null");
+    return timer_start(&s->ev_start, &s->ev_stop, s->stream);
+}
+
+extern "C" int lv_session_timer_stop(lv_session *s, float *ms)
+{
+    if (!s || !ms) return fail(LV_ERR_ARG, "lv_session_timer_stop: null argument");
+    LV_TRY(timer_stop(s->ev_start, s->ev_stop, s->stream, ms));
+    s->in_flight = false;
     return LV_OK;
 }
 
@@ -999,3 +1182,13 @@ extern "C" int lv_trace_read(lv_session *s, uint32_t layer, int which, float *ds
     s->in_flight = false;
     return LV_OK;
 }
+
+#ifdef LV_MEGA_TIMING
+// debugging aid of timing builds only: the persistent kernel's phase timestamps
+extern "C" int lv_debug_status_words(lv_session *s, uint32_t *dst, uint32_t n)
+{
+    if (!s || !s->status_host || n > 1024) return LV_ERR_ARG;
+    memcpy(dst, s->status_host, (size_t)n * 4);
+    return LV_OK;
+}
+#endif

@@ -45,6 +45,28 @@ __device__ __forceinline__ float wave_sum(float v)
     v += __shfl_xor(v, 32, kWave);
     return v;
 }
+// Four per-lane partials (one per matrix row) -> every lane of 16-lane row j holds the total of partial
+// kRowOfLaneGroup[j]: two v_permlane32_swap + one v_permlane16_swap fold the 64 lanes down to 16 per partial,
+// then DPP adds finish inside the rows.
+__device__ __forceinline__ float quad_partials_sum(float p0, float p1, float p2, float p3)
+{
+    // swap32(a, b): a' = [a.lo32 | b.lo32], b' = [a.hi32 | b.hi32]
+    auto s01 = __builtin_amdgcn_permlane32_swap(__float_as_uint(p0), __float_as_uint(p1), false, false);
+    auto s23 = __builtin_amdgcn_permlane32_swap(__float_as_uint(p2), __float_as_uint(p3), false, false);
+    const float a = __uint_as_float(s01[0]) + __uint_as_float(s01[1]);  // lanes 0-31: p0 pairs, 32-63: p1 pairs
+    const float b = __uint_as_float(s23[0]) + __uint_as_float(s23[1]);  // lanes 0-31: p2 pairs, 32-63: p3 pairs
+    // swap16(a, b): a' = [a.r0 b.r0 a.r2 b.r2], b' = [a.r1 b.r1 a.r3 b.r3]
+    auto t = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    const float c = __uint_as_float(t[0]) + __uint_as_float(t[1]);      // rows of 16 lanes hold p0, p2, p1, p3
+    return group16_sum(c);
+}
+// which of the four partials ends up in 16-lane row j of the result above
+__device__ __forceinline__ int quad_partial_of_lane(int lane)
+{
+    const int j = lane >> 4;
+    return ((j & 1) << 1) | (j >> 1);
+}
+
 template <int Lanes>
 __device__ __forceinline__ float group_sum(float v)
 {
@@ -75,6 +97,13 @@ __device__ __forceinline__ float ubyte_to_float(uint32_t v)
 
 // Sum over one q4_0 block of code*x with the codes left unsigned (0..15); the caller subtracts 8*sum(x).
 // GGML order (llava_buffer.cpp:361-369): byte j holds element j in its low nibble, element j+16 in its high one.
+//
+// Nibble -> float without a per-element extract: a byte 0x0q read as an OCP fp8 E4M3 number is exactly
+// q * 2^-9 for every q in 0..15 (q < 8 are the subnormals m * 2^-9, q >= 8 have exponent field 1 and value
+// (8 + m) * 2^-9).  v_cvt_pk_f32_fp8 converts two such bytes per instruction, so eight codes cost two masks,
+// one shift and four converts.  The factor 2^9 is applied once per block (exact).
+typedef float lv_float2 __attribute__((ext_vector_type(2)));
+
 __device__ __forceinline__ float q4_block_dot(const uint4 &q, const float (&x)[32])
 {
     const uint32_t w[4] = {q.x, q.y, q.z, q.w};
@@ -83,16 +112,18 @@ __device__ __forceinline__ float q4_block_dot(const uint4 &q, const float (&x)[3
     for (int i = 0; i < 4; i++) {
         const uint32_t lo = w[i] & 0x0f0f0f0fu;
         const uint32_t hi = (w[i] >> 4) & 0x0f0f0f0fu;
-        acc = fmaf(ubyte_to_float<0>(lo), x[4 * i + 0], acc);
-        acc = fmaf(ubyte_to_float<1>(lo), x[4 * i + 1], acc);
-        acc = fmaf(ubyte_to_float<2>(lo), x[4 * i + 2], acc);
-        acc = fmaf(ubyte_to_float<3>(lo), x[4 * i + 3], acc);
-        acc = fmaf(ubyte_to_float<0>(hi), x[16 + 4 * i + 0], acc);
-        acc = fmaf(ubyte_to_float<1>(hi), x[16 + 4 * i + 1], acc);
-        acc = fmaf(ubyte_to_float<2>(hi), x[16 + 4 * i + 2], acc);
-        acc = fmaf(ubyte_to_float<3>(hi), x[16 + 4 * i + 3], acc);
+        const lv_float2 l01 = __builtin_amdgcn_cvt_pk_f32_fp8(lo, false), l23 = __builtin_amdgcn_cvt_pk_f32_fp8(lo, true);
+        const lv_float2 h01 = __builtin_amdgcn_cvt_pk_f32_fp8(hi, false), h23 = __builtin_amdgcn_cvt_pk_f32_fp8(hi, true);
+        acc = fmaf(l01.x, x[4 * i + 0], acc);
+        acc = fmaf(l01.y, x[4 * i + 1], acc);
+        acc = fmaf(l23.x, x[4 * i + 2], acc);
+        acc = fmaf(l23.y, x[4 * i + 3], acc);
+        acc = fmaf(h01.x, x[16 + 4 * i + 0], acc);
+        acc = fmaf(h01.y, x[16 + 4 * i + 1], acc);
+        acc = fmaf(h23.x, x[16 + 4 * i + 2], acc);
+        acc = fmaf(h23.y, x[16 + 4 * i + 3], acc);
     }
-    return acc;
+    return acc * 512.f;
 }
 
 // Sum over one q8_0 block of (code+128)*x: codes are biased to unsigned by flipping the sign bit so the byte

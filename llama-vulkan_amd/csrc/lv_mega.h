@@ -1,0 +1,692 @@
+// lv_mega.h — the whole decode step of one token as ONE persistent kernel (gfx950, 256 CUs).
+//
+// Why: at batch 1 a layer is five tiny dependent GEMVs (1-6 us of HBM time each).  Launched one by one
+// they spend more time draining, launching and refilling the memory pipeline than streaming weights.
+// Here one workgroup per CU stays resident for the whole token; every wavefront walks its own contiguous
+// weight stream with a 12-deep register queue of 128-bit loads that keeps running across the phase
+// boundaries, so HBM stays busy while the workgroups exchange the small activation vectors.
+//
+// Phases of a layer (llava_layer.cpp:53-73), each separated by a data hand-over through HBM/L2:
+//   A  norm + [Wq;Wk;Wv] x        -> q, new K/V row (fp16 into the cache)
+//   B  single-query attention, 8 (or 6) position chunks per head -> partial numerators / denominators
+//   B' combine the chunks         -> o
+//   C  x += Wo o                  -> x1
+//   D  norm + (W3 x1)*silu(W1 x1) -> ff
+//   E  x1 += W2 ff                -> x2 (next layer's x)
+// then norm + output matrix -> logits.
+//
+// Hand-over without barriers: every exchanged float lives in a buffer that holds the bit pattern
+// 0xFFFFFFFF ("not written yet") until its producer stores the value with a device-scope write-through
+// store; consumers poll the data itself with device-scope loads.  No flag, no fence, no wait for store
+// acknowledgement.  Two buffer sets alternate between tokens; each token re-arms the other set.
+// Every poll loop is bounded: on expiry the kernel raises *status and carries on to its end.
+//
+// Weight stream: for each (layer, phase, workgroup, wave) the tiles that wave will consume, in order.
+// A tile is one matrix row restricted to the wave's 64-block column slab: 64 x 16 B codes + 64 x fp16
+// scales (1152 B).  Lane l of the wave always owns block column 64*slab + l, so the 32 activations of
+// that column sit in registers for the whole phase.
+#pragma once
+
+#include "lv_device.h"
+
+namespace lv {
+
+constexpr uint32_t kNotReady = 0xFFFFFFFFu;
+constexpr int kMegaWGs = 256;
+constexpr int kMegaDepth = 8;           // tiles in flight per wave
+constexpr int kMegaTile = 1152;         // bytes per q4_0 tile
+constexpr int kMegaHeadSlots = 24;      // head tiles per wave (static upper bound)
+constexpr uint32_t kSpinLimit = 1u << 20;
+
+__device__ __forceinline__ uint32_t ld_dev(const uint32_t *p)
+{
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void st_dev(float *p, float v)
+{
+    __hip_atomic_store(reinterpret_cast<uint32_t *>(p), __float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Workgroup barrier that orders LDS traffic only: global loads of the weight queue stay in flight across it
+// (__syncthreads would wait for vmcnt(0) and drain the queue at every phase step).
+__device__ __forceinline__ void lds_barrier()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+constexpr int cdiv(int a, int b) { return (a + b - 1) / b; }
+constexpr int round_up(int a, int b) { return cdiv(a, b) * b; }
+
+// Static shape of one model class.  NW = wavefronts per workgroup.
+template <int D_, int F_, int H_, int NW_>
+struct MegaShape {
+    static constexpr int D = D_, F = F_, H = H_, NW = NW_, R = 128;
+    static constexpr int NBD = D / 32, NBF = F / 32;            // blocks per row
+    static constexpr int NSD = cdiv(NBD, 64), NSF = cdiv(NBF, 64);  // column slabs
+    static constexpr int NRD = NW / NSD, NRF = NW / NSF;        // row sets (waves sharing a slab split the rows)
+    static constexpr int ROWS_A = 3 * D / kMegaWGs, ROWS_C = D / kMegaWGs, ROWS_D = 2 * F / kMegaWGs, ROWS_E = D / kMegaWGs;
+    static constexpr int TA = cdiv(ROWS_A, NRD), TC = cdiv(ROWS_C, NRD), TD = cdiv(ROWS_D, NRD), TE = cdiv(ROWS_E, NRF);
+    static constexpr int SEQ_A = 0, SEQ_C = TA, SEQ_D = TA + TC, SEQ_E = TA + TC + TD;
+    static constexpr int PER_LAYER = round_up(TA + TC + TD + TE, kMegaDepth);
+    static constexpr int CPH = kMegaWGs / H;                    // position chunks per head
+    static constexpr int PART = R + 4;                          // floats per partial (128 numerators, denominator, pad)
+    // floats of one layer's hand-over buffers
+    static constexpr int OFF_QKV = 0, OFF_PART = 3 * D, OFF_O = OFF_PART + H * CPH * PART, OFF_X1 = OFF_O + D,
+                         OFF_FF = OFF_X1 + D, OFF_X2 = OFF_FF + F, XCHG_LAYER = OFF_X2 + D;
+    static_assert((3 * D) % kMegaWGs == 0 && (2 * F) % kMegaWGs == 0 && D % kMegaWGs == 0, "rows must split over 256 workgroups");
+    static_assert(H * R == D && CPH >= 1 && NRD >= 1 && NRF >= 1, "shape");
+    // bytes of the weight stream of one layer
+    static constexpr size_t PHASE_A_BYTES = (size_t)kMegaWGs * NW * TA * kMegaTile, PHASE_C_BYTES = (size_t)kMegaWGs * NW * TC * kMegaTile,
+                            PHASE_D_BYTES = (size_t)kMegaWGs * NW * TD * kMegaTile, PHASE_E_BYTES = (size_t)kMegaWGs * NW * TE * kMegaTile;
+    static constexpr size_t LAYER_BYTES = PHASE_A_BYTES + PHASE_C_BYTES + PHASE_D_BYTES + PHASE_E_BYTES;
+    static constexpr size_t HEAD_BYTES = (size_t)kMegaWGs * NW * kMegaHeadSlots * kMegaTile;
+};
+
+struct MegaArgs {
+    const uint8_t *wstream;    // [layers] x LAYER_BYTES, then HEAD_BYTES, then one all-zero tile
+    const float *norms;        // [layers][2][D] (attention_norm, ffn_norm), then the final norm [D]
+    const float *tok_f32;      // embedding table [vocab][D] (fp32)
+    uint16_t *kv;              // [layers][2][backlog][D] fp16
+    const float2 *trig;        // [backlog][64]
+    float *xchg;               // this token's hand-over buffers: [layers] x XCHG_LAYER floats, all kNotReady
+    float *xchg_rearm;         // the other set, re-armed to kNotReady during this token
+    float *logits;             // [vocab]
+    uint32_t *status;          // host-visible; set non-zero when a poll loop expired
+    uint32_t layers, vocab, backlog, pos, token;
+};
+
+// Optional phase timestamps (built only with -DLV_MEGA_TIMING): workgroup 0 records the 100 MHz wall clock at
+// every phase boundary of layers 0..3 into status[16 + ...].
+#ifdef LV_MEGA_TIMING
+#define MEGA_STAMP(idx)                                                                                        \
+    do {                                                                                                       \
+        if (blockIdx.x == LV_MEGA_TIMING_WG && st == 0 && layer < 4)                                  \
+            status[16 + layer * 16 + (idx)] = (uint32_t)wall_clock64();                                        \
+    } while (0)
+#else
+#define MEGA_STAMP(idx) do { } while (0)
+#endif
+
+struct MegaTile {
+    uint4 c;
+    uint16_t d;
+};
+
+// ---- polling helpers ----------------------------------------------------------------------------------------
+// N values strided by `stride` elements starting at p; spins until none of them is the not-ready pattern.
+template <int N>
+__device__ __forceinline__ void poll_values(float (&v)[N], const float *p, int stride, const bool (&want)[N], uint32_t *status)
+{
+    uint32_t spins = 0;
+    bool pending;
+    do {
+        pending = false;
+#pragma unroll
+        for (int j = 0; j < N; j++) {
+            uint32_t u = 0;
+            if (want[j]) u = ld_dev(reinterpret_cast<const uint32_t *>(p) + (size_t)j * stride);
+            v[j] = __uint_as_float(u);
+            pending |= (u == kNotReady);
+        }
+    } while (pending && ++spins < kSpinLimit);
+    if (pending) *status = 1u;
+}
+
+// the 32 activations of this lane's block column, from LDS
+__device__ __forceinline__ void load_slab(float (&xr)[32], float &xsum, const float *xs, int block, bool have)
+{
+    const float4 *src = reinterpret_cast<const float4 *>(xs + (have ? block : 0) * 32);
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        float4 v = src[j];
+        if (!have) v = make_float4(0.f, 0.f, 0.f, 0.f);
+        xr[4 * j] = v.x; xr[4 * j + 1] = v.y; xr[4 * j + 2] = v.z; xr[4 * j + 3] = v.w;
+        s += (v.x + v.y) + (v.z + v.w);
+    }
+    xsum = s;
+}
+
+// Everything a wave needs to find its tiles.
+template <class S>
+struct MegaWave {
+    const uint8_t *wstream, *dummy /* one all-zero tile after the head */;
+    uint32_t layers, vocab_rows /* head rows per workgroup */, vocab;
+    int b, w, lane;
+    // per phase geometry (column slab, row set, whether the wave works in the phase, whether the lane has a column)
+    int sD, rD, sF, rF;
+    bool actD, actF, laneD, laneF;
+
+    __device__ __forceinline__ void init(const MegaArgs &a)
+    {
+        wstream = a.wstream; layers = a.layers; vocab = a.vocab;
+        dummy = a.wstream + (size_t)a.layers * S::LAYER_BYTES + S::HEAD_BYTES;
+        vocab_rows = (a.vocab + kMegaWGs - 1) / kMegaWGs;
+        // the wave index is uniform: telling the compiler so keeps every tile address in scalar registers
+        b = blockIdx.x; w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); lane = threadIdx.x & 63;
+        sD = w % S::NSD; rD = w / S::NSD; actD = rD < S::NRD; laneD = sD * 64 + lane < S::NBD;
+        sF = w % S::NSF; rF = w / S::NSF; actF = rF < S::NRF; laneF = sF * 64 + lane < S::NBF;
+    }
+
+    // Loads sequence slot k (relative to the start of `layer`; k >= PER_LAYER runs into the next layer, or into
+    // the head after the last layer).  k is a compile-time constant after unrolling, so whether a slot loads at
+    // all is static; every runtime condition (row past the end, lane without a column, last layer) only selects
+    // the address: an invalid tile reads the all-zero dummy tile at the end of the stream.  Straight-line loads
+    // let the compiler count outstanding loads exactly and wait with vmcnt(N > 0).
+    __device__ __forceinline__ void fetch(MegaTile &t, int k, uint32_t layer) const
+    {
+        const bool wrapped = k >= S::PER_LAYER;
+        if (wrapped) { k -= S::PER_LAYER; layer += 1; }
+        const bool into_head = wrapped && layer >= layers;  // uniform, runtime
+        int i = 0, tiles = 0, rows = 0, rset = 0;
+        bool act = false, lane_ok = false, real = true;
+        size_t off = 0;
+        if (k < S::SEQ_C) { i = k; tiles = S::TA; rows = S::ROWS_A; act = actD; lane_ok = laneD; rset = rD; }
+        else if (k < S::SEQ_D) { i = k - S::SEQ_C; tiles = S::TC; rows = S::ROWS_C; act = actD; lane_ok = laneD; rset = rD; off = S::PHASE_A_BYTES; }
+        else if (k < S::SEQ_E) { i = k - S::SEQ_D; tiles = S::TD; rows = S::ROWS_D; act = actD; lane_ok = laneD; rset = rD; off = S::PHASE_A_BYTES + S::PHASE_C_BYTES; }
+        else if (k < S::SEQ_E + S::TE) { i = k - S::SEQ_E; tiles = S::TE; rows = S::ROWS_E; act = actF; lane_ok = laneF; rset = rF; off = S::PHASE_A_BYTES + S::PHASE_C_BYTES + S::PHASE_D_BYTES; }
+        else real = false;                                   // padding slot of the layer sequence
+        const bool head_slot = wrapped && k < kMegaHeadSlots;  // static
+        if (!real && !head_slot) return;                     // static: this slot never loads
+        const uint8_t *p = dummy;
+        if (real) {
+            const bool ok = !into_head && act && lane_ok && rset * tiles + i < rows;
+            const uint8_t *q = wstream + (size_t)layer * S::LAYER_BYTES + off + ((size_t)(b * S::NW + w) * tiles + i) * kMegaTile;
+            p = ok ? q : p;
+        }
+        if (head_slot) {
+            const uint8_t *q = head_tile(k);
+            p = (into_head && q) ? q : p;
+        }
+        t.c = *reinterpret_cast<const uint4 *>(p + lane * 16);
+        t.d = *reinterpret_cast<const uint16_t *>(p + 1024 + lane * 2);
+    }
+
+    // address of head tile k of this wave, or null when the wave/lane/row has none
+    __device__ __forceinline__ const uint8_t *head_tile(int k) const
+    {
+        const int rows = (int)vocab_rows, per_set = (rows + S::NRD - 1) / S::NRD;
+        const int j = rD * per_set + k;
+        const bool ok = actD && laneD && k < per_set && j < rows && (uint32_t)(b * rows + j) < vocab;
+        return ok ? wstream + (size_t)layers * S::LAYER_BYTES + ((size_t)(b * S::NW + w) * kMegaHeadSlots + k) * kMegaTile : nullptr;
+    }
+
+    // head phase: slot k of the head sequence (static k)
+    __device__ __forceinline__ void fetch_head(MegaTile &t, int k) const
+    {
+        if (k >= kMegaHeadSlots) return;
+        const uint8_t *q = head_tile(k);
+        const uint8_t *p = q ? q : dummy;
+        t.c = *reinterpret_cast<const uint4 *>(p + lane * 16);
+        t.d = *reinterpret_cast<const uint16_t *>(p + 1024 + lane * 2);
+    }
+};
+
+// One GEMV phase of one wave: consumes NT queue slots starting at sequence index SEQ0, refills each consumed
+// slot with the tile kMegaDepth further down the sequence, leaves per-row sums in red[row*NS + slab].
+template <class S, int SEQ0, int NT, int NS>
+__device__ __forceinline__ void gemv_phase(MegaTile (&q)[kMegaDepth], const MegaWave<S> &mw, uint32_t layer, const float (&xr)[32],
+                                           float xsum, int slab, int rset, bool active, int rows, float *red)
+{
+    constexpr int NT4 = round_up(NT, 4);
+    float p[4];
+#pragma unroll
+    for (int i = 0; i < NT4; i++) {
+        if (i < NT) {
+            const int slot = (SEQ0 + i) % kMegaDepth;
+            const MegaTile t = q[slot];
+            p[i & 3] = (q4_block_dot(t.c, xr) - 8.f * xsum) * half_bits_to_float(t.d);
+            mw.fetch(q[slot], SEQ0 + i + kMegaDepth, layer);
+        } else {
+            p[i & 3] = 0.f;
+        }
+        if ((i & 3) == 3) {
+            const float s = quad_partials_sum(p[0], p[1], p[2], p[3]);
+            const int ii = (i - 3) + quad_partial_of_lane(mw.lane);
+            const int row = rset * NT + ii;
+            if (active && (mw.lane & 15) == 0 && row < rows && ii < NT) red[row * NS + slab] = s;
+        }
+    }
+}
+
+template <int NS>
+__device__ __forceinline__ float red_row(const float *red, int row)
+{
+    float t = 0.f;
+#pragma unroll
+    for (int s = 0; s < NS; s++) t += red[row * NS + s];
+    return t;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Roles.  A wavefront's vector-memory operations complete in order, so a wave that polls a hand-over buffer
+// (or loads K/V rows) cannot see its answer before every weight tile it requested earlier has arrived: a
+// polling wave drains its own prefetch queue.  Therefore the workgroup is split:
+//   * S::NW  "stream" waves own the weight queues and do nothing but tiles; they meet the others only at LDS
+//     barriers, which leave global loads in flight;
+//   * kMegaServiceWaves "service" waves poll the hand-over buffers, normalise, run the attention and write
+//     every result.  They issue no weight loads.
+// Both roles execute the same sequence of barriers.
+// ---------------------------------------------------------------------------------------------------------
+constexpr int kMegaServiceWaves = 4;
+constexpr int kMegaServiceThreads = kMegaServiceWaves * 64;
+
+// LDS of the kernel, shared by both roles.
+template <class S>
+struct MegaLds {
+    static constexpr int XS = S::F > S::D ? S::F : S::D;
+    static constexpr int RED_ROWS = S::ROWS_D > kMegaHeadSlots * S::NRD ? S::ROWS_D : kMegaHeadSlots * S::NRD;
+    static constexpr int RED_COLS = S::NSF > S::NSD ? S::NSF : S::NSD;
+    float xs[XS];                    // the phase's input vector (during attention: exp(score) of the chunk)
+    float red[RED_ROWS * RED_COLS];  // per-row partial sums, one column per slab
+    float xown[S::ROWS_C];           // this workgroup's rows of the residual stream
+    float scratch[8];
+    float attn_red[kMegaServiceWaves * (S::R + 1)];
+};
+
+// Service waves: bring the N-float vector at `src` into LDS, optionally normalised (normalize.comp:34-64: mean,
+// then mean-centred variance, no epsilon).  Barriers: 3 when NORM, else 1; the stream waves run the same count.
+template <int N, bool NORM>
+__device__ __forceinline__ void service_acquire(int st, float *xs, const float *src, const float *w, float *scratch, uint32_t *status)
+{
+    constexpr int T = kMegaServiceThreads, PER = cdiv(N, T);
+    float v[PER];
+    bool want[PER];
+#pragma unroll
+    for (int j = 0; j < PER; j++) want[j] = st + j * T < N;
+    poll_values<PER>(v, src + st, T, want, status);
+    if constexpr (NORM) {
+        const int sw = st >> 6;
+        float s = 0.f;
+#pragma unroll
+        for (int j = 0; j < PER; j++) s += want[j] ? v[j] : 0.f;
+        s = wave_sum(s);
+        if ((st & 63) == 0) scratch[sw] = s;
+        lds_barrier();
+        const float mean = ((scratch[0] + scratch[1]) + (scratch[2] + scratch[3])) / (float)N;
+        float q = 0.f;
+#pragma unroll
+        for (int j = 0; j < PER; j++) {
+            const float c = want[j] ? v[j] - mean : 0.f;
+            q = fmaf(c, c, q);
+        }
+        q = wave_sum(q);
+        if ((st & 63) == 0) scratch[4 + sw] = q;
+        lds_barrier();
+        const float inv = rsqrtf(((scratch[4] + scratch[5]) + (scratch[6] + scratch[7])) / (float)N);
+#pragma unroll
+        for (int j = 0; j < PER; j++)
+            if (want[j]) xs[st + j * T] = (v[j] * w[st + j * T]) * inv;
+    } else {
+#pragma unroll
+        for (int j = 0; j < PER; j++)
+            if (want[j]) xs[st + j * T] = v[j];
+    }
+    lds_barrier();
+}
+
+template <bool NORM>
+__device__ __forceinline__ void stream_await_vector()
+{
+    if constexpr (NORM) { lds_barrier(); lds_barrier(); }
+    lds_barrier();
+}
+
+// ---- the stream role: weight tiles only -----------------------------------------------------------------------
+template <class S>
+__device__ __forceinline__ void mega_stream_role(const MegaArgs &a, const MegaWave<S> &mw, MegaLds<S> &l)
+{
+    const int lane = mw.lane;
+    MegaTile q[kMegaDepth];
+#pragma unroll
+    for (int k = 0; k < kMegaDepth; k++) mw.fetch(q[k], k, 0);
+    float xr[32];
+    float xsum;
+    for (uint32_t layer = 0; layer < a.layers; layer++) {
+        // A
+        stream_await_vector<true>();
+        load_slab(xr, xsum, l.xs, mw.sD * 64 + lane, mw.laneD);
+        gemv_phase<S, S::SEQ_A, S::TA, S::NSD>(q, mw, layer, xr, xsum, mw.sD, mw.rD, mw.actD, S::ROWS_A, l.red);
+        lds_barrier();
+        // B: attention runs on the service waves (two barriers of theirs)
+        lds_barrier();
+        lds_barrier();
+        // C
+        stream_await_vector<false>();
+        load_slab(xr, xsum, l.xs, mw.sD * 64 + lane, mw.laneD);
+        gemv_phase<S, S::SEQ_C, S::TC, S::NSD>(q, mw, layer, xr, xsum, mw.sD, mw.rD, mw.actD, S::ROWS_C, l.red);
+        lds_barrier();
+        // D
+        stream_await_vector<true>();
+        load_slab(xr, xsum, l.xs, mw.sD * 64 + lane, mw.laneD);
+        gemv_phase<S, S::SEQ_D, S::TD, S::NSD>(q, mw, layer, xr, xsum, mw.sD, mw.rD, mw.actD, S::ROWS_D, l.red);
+        lds_barrier();
+        // E
+        stream_await_vector<false>();
+        load_slab(xr, xsum, l.xs, mw.sF * 64 + lane, mw.laneF);
+        gemv_phase<S, S::SEQ_E, S::TE, S::NSF>(q, mw, layer, xr, xsum, mw.sF, mw.rF, mw.actF, S::ROWS_E, l.red);
+        // padding slots of the layer's sequence carry no tile, but the slot kMegaDepth ahead of them does
+#pragma unroll
+        for (int k = S::SEQ_E + S::TE; k < S::PER_LAYER; k++) mw.fetch(q[k % kMegaDepth], k + kMegaDepth, layer);
+        lds_barrier();
+    }
+    // head
+    stream_await_vector<true>();
+    load_slab(xr, xsum, l.xs, mw.sD * 64 + lane, mw.laneD);
+    const int rows = (int)mw.vocab_rows, per_set = (rows + S::NRD - 1) / S::NRD;
+    float p[4];
+#pragma unroll
+    for (int i = 0; i < kMegaHeadSlots; i++) {
+        const int slot = i % kMegaDepth;
+        const MegaTile t = q[slot];
+        p[i & 3] = (q4_block_dot(t.c, xr) - 8.f * xsum) * half_bits_to_float(t.d);
+        mw.fetch_head(q[slot], i + kMegaDepth);
+        if ((i & 3) == 3) {
+            const float s = quad_partials_sum(p[0], p[1], p[2], p[3]);
+            const int ii = (i - 3) + quad_partial_of_lane(lane);
+            const int row = mw.rD * per_set + ii;
+            if (mw.actD && (lane & 15) == 0 && ii < per_set && row < rows) l.red[row * S::NSD + mw.sD] = s;
+        }
+    }
+    lds_barrier();
+}
+
+// ---- the service role: hand-over polling, normalisation, attention, every store -------------------------------
+template <class S>
+__device__ __forceinline__ void mega_service_role(const MegaArgs &a, const MegaWave<S> &mw, MegaLds<S> &l)
+{
+    constexpr int D = S::D, F = S::F, H = S::H, R = S::R, NSV = kMegaServiceWaves;
+    const int b = mw.b, lane = mw.lane;
+    const int st = (int)threadIdx.x - S::NW * 64, sw = mw.w - S::NW;
+    uint32_t *status = a.status;
+    float *xs = l.xs, *red = l.red, *xown = l.xown;
+
+    // re-arm the other buffer set for the next token
+#ifndef LV_MEGA_NOWAIT   // (experiment builds leave stale, "ready" data in place to time the kernel without hand-over waits)
+    {
+        const size_t n4 = (size_t)a.layers * S::XCHG_LAYER / 4;
+        uint4 *dst = reinterpret_cast<uint4 *>(a.xchg_rearm);
+        for (size_t i = (size_t)b * kMegaServiceThreads + st; i < n4; i += (size_t)kMegaWGs * kMegaServiceThreads)
+            dst[i] = make_uint4(kNotReady, kNotReady, kNotReady, kNotReady);
+    }
+#endif
+    const uint32_t pos = a.pos;
+    const float *x_src = a.tok_f32 + (size_t)a.token * D;  // layer 0 reads the embedding row directly (constant data)
+    if (st < S::ROWS_C) xown[st] = x_src[b * S::ROWS_C + st];
+
+    for (uint32_t layer = 0; layer < a.layers; layer++) {
+        float *xc = a.xchg + (size_t)layer * S::XCHG_LAYER;
+        const float *norm_w = a.norms + (size_t)layer * 2 * D;
+        uint16_t *kc = a.kv + (size_t)layer * 2 * a.backlog * D, *vc = kc + (size_t)a.backlog * D;
+
+        // ================= A: norm + QKV ====================================================================
+        MEGA_STAMP(0);
+        service_acquire<D, true>(st, xs, x_src, norm_w, l.scratch, status);
+        MEGA_STAMP(1);
+        lds_barrier();  // the stream waves have filled `red`
+        if (st < S::ROWS_A) {
+            const float v = red_row<S::NSD>(red, st);
+            const int g = b * S::ROWS_A + st, which = g / D, col = g % D;
+            if (which == 0) {
+                st_dev(xc + S::OFF_QKV + col, v);
+            } else {
+                // copy_to_cache.comp:35: the cache keeps fp16; attention of this very step reads the rounded value too
+                const uint16_t hbits = float_to_half_bits(v);
+                (which == 1 ? kc : vc)[(size_t)pos * D + col] = hbits;
+                st_dev(xc + S::OFF_QKV + which * D + col, half_bits_to_float(hbits));
+            }
+        }
+
+        // ================= B: attention chunk (head h, chunk c) ================================================
+        MEGA_STAMP(2);
+        {
+            const int h = b / S::CPH, c = b % S::CPH;
+            const bool att = h < H;
+            const uint32_t n_valid = pos + 1;
+            uint32_t chunk = (n_valid + S::CPH - 1) / S::CPH;
+            chunk = (chunk + 3) & ~3u;
+            const uint32_t p_begin = min((uint32_t)c * chunk, n_valid), p_end = min(p_begin + chunk, n_valid);
+            const int sub = lane & 15, rsel = sw * 4 + (lane >> 4);
+            float *e_lds = xs;            // chunk <= backlog/CPH + 3 floats; xs is free between phases A and C
+            constexpr int RPR = NSV * 4;  // cache rows per round of the service waves
+            constexpr int PRE = 4;        // rounds whose K and V rows are requested before the query arrives
+            const size_t row_off = (size_t)h * R + sub * 8;
+            const bool want8[8] = {true, true, true, true, true, true, true, true};
+            auto unpack8 = [](float (&f)[8], const uint4 &raw) {
+                const uint32_t wv[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    f[2 * i] = half_bits_to_float((uint16_t)(wv[i] & 0xffffu));
+                    f[2 * i + 1] = half_bits_to_float((uint16_t)(wv[i] >> 16));
+                }
+            };
+            uint4 vpre[PRE];
+            float den = 0.f;
+            if (att) {
+                // Rows older than this token do not depend on it: ask for them first, then wait for q.
+                uint4 kpre[PRE];
+#pragma unroll
+                for (int r = 0; r < PRE; r++) {
+                    const uint32_t p = p_begin + r * RPR + rsel;
+                    const uint32_t pc = (p < p_end && p != pos) ? p : 0;  // any valid row; unused when masked
+                    kpre[r] = *reinterpret_cast<const uint4 *>(kc + (size_t)pc * D + row_off);
+                    vpre[r] = *reinterpret_cast<const uint4 *>(vc + (size_t)pc * D + row_off);
+                }
+                float qv[8];
+                poll_values<8>(qv, xc + S::OFF_QKV + h * R + sub * 8, 1, want8, status);
+                MEGA_STAMP(3);
+                const float scale = rsqrtf((float)R);
+                auto score_round = [&](uint32_t p, const uint4 &kraw) {
+                    float s = 0.f;
+                    if (p < p_end) {
+                        float kf[8];
+                        if (p == pos) poll_values<8>(kf, xc + S::OFF_QKV + D + h * R + sub * 8, 1, want8, status);
+                        else unpack8(kf, kraw);
+                        const float4 *tp = reinterpret_cast<const float4 *>(a.trig + (size_t)(pos - p) * (R / 2) + sub * 4);
+                        const float4 t0 = tp[0], t1 = tp[1];
+                        const float ct[4] = {t0.x, t0.z, t1.x, t1.z}, stn[4] = {t0.y, t0.w, t1.y, t1.w};
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            const float kx = kf[2 * i], ky = kf[2 * i + 1], qx = qv[2 * i], qy = qv[2 * i + 1];
+                            const float dotp = fmaf(qy, ky, qx * kx);
+                            const float crs = fmaf(qx, ky, -(qy * kx));
+                            s = fmaf(ct[i], dotp, s);
+                            s = fmaf(stn[i], crs, s);
+                        }
+                    }
+                    s = group16_sum(s);
+                    float e = 0.f;
+                    if (p < p_end) {
+                        e = __expf(s * scale);
+                        if (sub == 0) e_lds[p - p_begin] = e;
+                    }
+                    den += (sub == 0) ? e : 0.f;
+                };
+#pragma unroll
+                for (int r = 0; r < PRE; r++) score_round(p_begin + r * RPR + rsel, kpre[r]);
+                for (uint32_t p0 = p_begin + PRE * RPR; p0 < p_end; p0 += RPR) {
+                    const uint32_t p = p0 + rsel;
+                    const uint32_t pc = (p < p_end && p != pos) ? p : 0;
+                    score_round(p, *reinterpret_cast<const uint4 *>(kc + (size_t)pc * D + row_off));
+                }
+            }
+            lds_barrier();
+            if (att) {
+                float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                auto pv_round = [&](uint32_t p, const uint4 &vraw) {
+                    if (p < p_end) {
+                        float vf[8];
+                        if (p == pos) poll_values<8>(vf, xc + S::OFF_QKV + 2 * D + h * R + sub * 8, 1, want8, status);
+                        else unpack8(vf, vraw);
+                        const float e = e_lds[p - p_begin];
+#pragma unroll
+                        for (int i = 0; i < 8; i++) acc[i] = fmaf(e, vf[i], acc[i]);
+                    }
+                };
+#pragma unroll
+                for (int r = 0; r < PRE; r++) pv_round(p_begin + r * RPR + rsel, vpre[r]);
+                for (uint32_t p0 = p_begin + PRE * RPR; p0 < p_end; p0 += RPR) {
+                    const uint32_t p = p0 + rsel;
+                    const uint32_t pc = (p < p_end && p != pos) ? p : 0;
+                    pv_round(p, *reinterpret_cast<const uint4 *>(vc + (size_t)pc * D + row_off));
+                }
+#pragma unroll
+                for (int off = 16; off < 64; off <<= 1) {
+#pragma unroll
+                    for (int i = 0; i < 8; i++) acc[i] += __shfl_xor(acc[i], off, kWave);
+                    den += __shfl_xor(den, off, kWave);
+                }
+                if (lane < 16) {
+#pragma unroll
+                    for (int i = 0; i < 8; i++) l.attn_red[sw * (R + 1) + lane * 8 + i] = acc[i];
+                    if (lane == 0) l.attn_red[sw * (R + 1) + R] = den;
+                }
+            }
+            lds_barrier();
+            if (att && st <= R) {
+                float t = 0.f;
+#pragma unroll
+                for (int i = 0; i < NSV; i++) t += l.attn_red[i * (R + 1) + st];
+                st_dev(xc + S::OFF_PART + (h * S::CPH + c) * S::PART + st, t);
+            }
+        }
+
+        // ================= B': combine the chunks of head b =====================================================
+        MEGA_STAMP(4);
+        if (b < H && st < R) {
+            float num[S::CPH], dn[S::CPH];
+            bool want[S::CPH];
+#pragma unroll
+            for (int c = 0; c < S::CPH; c++) want[c] = true;
+            const float *hp = xc + S::OFF_PART + (size_t)b * S::CPH * S::PART;
+            poll_values<S::CPH>(num, hp + st, S::PART, want, status);
+            poll_values<S::CPH>(dn, hp + R, S::PART, want, status);
+            float n = 0.f, d = 0.f;
+#pragma unroll
+            for (int c = 0; c < S::CPH; c++) { n += num[c]; d += dn[c]; }
+            st_dev(xc + S::OFF_O + b * R + st, n / d);
+        }
+
+        // ================= C: x += Wo o ============================================================================
+        MEGA_STAMP(5);
+        service_acquire<D, false>(st, xs, xc + S::OFF_O, nullptr, l.scratch, status);
+        MEGA_STAMP(6);
+        lds_barrier();
+        if (st < S::ROWS_C) {
+            const float v = xown[st] + red_row<S::NSD>(red, st);
+            xown[st] = v;
+            st_dev(xc + S::OFF_X1 + b * S::ROWS_C + st, v);
+        }
+
+        // ================= D: norm + SwiGLU ========================================================================
+        MEGA_STAMP(7);
+        service_acquire<D, true>(st, xs, xc + S::OFF_X1, norm_w + D, l.scratch, status);
+        MEGA_STAMP(8);
+        lds_barrier();
+        if (st < S::ROWS_D / 2) {
+            // rows alternate W3 row k, W1 row k (matmul_silu_ff.comp:96: result1 * result2 / (exp(-result2) + 1))
+            const float r1 = red_row<S::NSD>(red, 2 * st), r2 = red_row<S::NSD>(red, 2 * st + 1);
+            st_dev(xc + S::OFF_FF + b * (S::ROWS_D / 2) + st, r1 * r2 / (__expf(-r2) + 1.f));
+        }
+
+        // ================= E: x += W2 ff ===========================================================================
+        MEGA_STAMP(9);
+        service_acquire<F, false>(st, xs, xc + S::OFF_FF, nullptr, l.scratch, status);
+        MEGA_STAMP(10);
+        lds_barrier();
+        if (st < S::ROWS_E) {
+            const float v = xown[st] + red_row<S::NSF>(red, st);
+            xown[st] = v;
+            st_dev(xc + S::OFF_X2 + b * S::ROWS_E + st, v);
+        }
+        MEGA_STAMP(11);
+        x_src = xc + S::OFF_X2;
+    }
+
+    // ================= head: norm + output matrix ====================================================================
+    service_acquire<D, true>(st, xs, x_src, a.norms + (size_t)a.layers * 2 * D, l.scratch, status);
+    lds_barrier();
+    const int rows = (int)mw.vocab_rows;
+    for (int j = st; j < rows; j += kMegaServiceThreads) {
+        const uint32_t n = (uint32_t)b * rows + j;
+        if (n < a.vocab) a.logits[n] = red_row<S::NSD>(red, j);
+    }
+}
+
+template <class S>
+__global__ __launch_bounds__((S::NW + kMegaServiceWaves) * 64, 1) void mega_decode_kernel(MegaArgs a)
+{
+    __shared__ __attribute__((aligned(16))) MegaLds<S> lds;
+#ifdef LV_MEGA_TIMING
+    const uint64_t clk0 = clock64(), wall0 = wall_clock64();
+#endif
+    MegaWave<S> mw;
+    mw.init(a);
+    if (mw.w < S::NW) mega_stream_role<S>(a, mw, lds);
+    else mega_service_role<S>(a, mw, lds);
+#ifdef LV_MEGA_TIMING
+    if (blockIdx.x == LV_MEGA_TIMING_WG && threadIdx.x == S::NW * 64) {
+        a.status[8] = (uint32_t)(clock64() - clk0);
+        a.status[9] = (uint32_t)(wall_clock64() - wall0);
+    }
+#endif
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Builds the weight stream from the row-major split layout (runs once at upload).
+// One thread per (tile, lane).  phase: 0 A, 1 C, 2 D, 3 E, 4 head.
+// ---------------------------------------------------------------------------------------------------------
+struct MegaPackSrc {
+    MatView m[3];  // A: wq, wk, wv;  C: wo;  D: w3, w1;  E: w2;  head: output
+};
+
+template <class S>
+__global__ void mega_pack_kernel(uint8_t *dst /* start of the phase region */, MegaPackSrc src, int phase, uint32_t vocab)
+{
+    const int tiles = phase == 0 ? S::TA : phase == 1 ? S::TC : phase == 2 ? S::TD : phase == 3 ? S::TE : kMegaHeadSlots;
+    const int ns = phase == 3 ? S::NSF : S::NSD, nr = phase == 3 ? S::NRF : S::NRD, nb = phase == 3 ? S::NBF : S::NBD;
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t total = (size_t)kMegaWGs * S::NW * tiles * 64;
+    if (idx >= total) return;
+    const int lane = idx % 64;
+    const size_t tile = idx / 64;
+    const int i = tile % tiles;
+    const int w = (tile / tiles) % S::NW;
+    const int b = tile / tiles / S::NW;
+    const int slab = w % ns, rset = w / ns;
+    uint8_t *out = dst + tile * kMegaTile;
+    uint4 codes = make_uint4(0, 0, 0, 0);
+    uint16_t scale = 0;
+    const int blk = slab * 64 + lane;
+    bool ok = rset < nr && blk < nb;
+    const MatView *mv = nullptr;
+    uint32_t row = 0;
+    if (ok) {
+        if (phase == 4) {
+            const int rows = (vocab + kMegaWGs - 1) / kMegaWGs, per_set = (rows + nr - 1) / nr;
+            const int j = rset * per_set + i;
+            ok = i < per_set && j < rows && (uint32_t)(b * rows + j) < vocab;
+            row = b * rows + j;
+            mv = &src.m[0];
+        } else {
+            const int rows = phase == 0 ? S::ROWS_A : phase == 1 ? S::ROWS_C : phase == 2 ? S::ROWS_D : S::ROWS_E;
+            const int j = rset * tiles + i;
+            ok = j < rows;
+            const int g = b * rows + j;
+            if (phase == 0) { mv = &src.m[g / S::D]; row = g % S::D; }
+            else if (phase == 2) { mv = &src.m[g & 1]; row = g >> 1; }
+            else { mv = &src.m[0]; row = g; }
+        }
+    }
+    if (ok) {
+        const size_t sb = (size_t)row * nb + blk;
+        codes = mv->codes[sb];
+        scale = mv->scales[sb];
+    }
+    *reinterpret_cast<uint4 *>(out + lane * 16) = codes;
+    *reinterpret_cast<uint16_t *>(out + 1024 + lane * 2) = scale;
+}
+
+}  // namespace lv
