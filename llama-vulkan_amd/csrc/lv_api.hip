@@ -964,7 +964,7 @@ static int launch_mega(lv_session *s, uint32_t pos, uint32_t token)
     s->xchg_turn++;
     void *params[] = {&a};
     HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<const void *>(&mega_decode_kernel<Mega7B>), dim3(kMegaWGs),
-                                       dim3((Mega7B::NW + kMegaServiceWaves) * 64), params, 0, s->stream));
+                                       dim3(Mega7B::NW * 64), params, 0, s->stream));
     return LV_OK;
 }
 

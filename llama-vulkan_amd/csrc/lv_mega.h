@@ -33,7 +33,7 @@ namespace lv {
 
 constexpr uint32_t kNotReady = 0xFFFFFFFFu;
 constexpr int kMegaWGs = 256;
-constexpr int kMegaDepth = 8;           // tiles in flight per wave
+constexpr int kMegaDepth = 4;           // tiles in flight per wave
 constexpr int kMegaTile = 1152;         // bytes per q4_0 tile
 constexpr int kMegaHeadSlots = 24;      // head tiles per wave (static upper bound)
 constexpr uint32_t kSpinLimit = 1u << 20;
@@ -51,6 +51,9 @@ __device__ __forceinline__ void st_dev(float *p, float v)
 // (__syncthreads would wait for vmcnt(0) and drain the queue at every phase step).
 __device__ __forceinline__ void lds_barrier()
 {
+#ifdef LV_MEGA_FREERUN   // experiment: no synchronisation at all, to time the bare weight stream + tile arithmetic
+    return;
+#endif
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
@@ -102,11 +105,17 @@ struct MegaArgs {
 #ifdef LV_MEGA_TIMING
 #define MEGA_STAMP(idx)                                                                                        \
     do {                                                                                                       \
-        if (blockIdx.x == LV_MEGA_TIMING_WG && st == 0 && layer < 4)                                  \
+        if (blockIdx.x == LV_MEGA_TIMING_WG && threadIdx.x == 0 && layer < 4)                                  \
             status[16 + layer * 16 + (idx)] = (uint32_t)wall_clock64();                                        \
+    } while (0)
+#define MEGA_STREAM_STAMP(idx)                                                                                 \
+    do {                                                                                                       \
+        if (blockIdx.x == LV_MEGA_TIMING_WG && threadIdx.x == 0 && layer < 4)                                  \
+            a.status[16 + layer * 16 + (idx)] = (uint32_t)wall_clock64();                                      \
     } while (0)
 #else
 #define MEGA_STAMP(idx) do { } while (0)
+#define MEGA_STREAM_STAMP(idx) do { } while (0)
 #endif
 
 struct MegaTile {
@@ -117,7 +126,8 @@ struct MegaTile {
 // ---- polling helpers ----------------------------------------------------------------------------------------
 // N values strided by `stride` elements starting at p; spins until none of them is the not-ready pattern.
 template <int N>
-__device__ __forceinline__ void poll_values(float (&v)[N], const float *p, int stride, const bool (&want)[N], uint32_t *status)
+__device__ __forceinline__ void poll_values(float (&v)[N], const float *p, int stride, const bool (&want)[N], uint32_t *status,
+                                            int group_stride = 0 /* when non-zero: element j lives at p[(j/8)*8*group_stride + j%8] */)
 {
     uint32_t spins = 0;
     bool pending;
@@ -126,7 +136,8 @@ __device__ __forceinline__ void poll_values(float (&v)[N], const float *p, int s
 #pragma unroll
         for (int j = 0; j < N; j++) {
             uint32_t u = 0;
-            if (want[j]) u = ld_dev(reinterpret_cast<const uint32_t *>(p) + (size_t)j * stride);
+            const size_t off = group_stride ? (size_t)(j / 8) * 8 * group_stride + (j % 8) : (size_t)j * stride;
+            if (want[j]) u = ld_dev(reinterpret_cast<const uint32_t *>(p) + off);
             v[j] = __uint_as_float(u);
             pending |= (u == kNotReady);
         }
@@ -260,20 +271,7 @@ __device__ __forceinline__ float red_row(const float *red, int row)
     return t;
 }
 
-// ---------------------------------------------------------------------------------------------------------
-// Roles.  A wavefront's vector-memory operations complete in order, so a wave that polls a hand-over buffer
-// (or loads K/V rows) cannot see its answer before every weight tile it requested earlier has arrived: a
-// polling wave drains its own prefetch queue.  Therefore the workgroup is split:
-//   * S::NW  "stream" waves own the weight queues and do nothing but tiles; they meet the others only at LDS
-//     barriers, which leave global loads in flight;
-//   * kMegaServiceWaves "service" waves poll the hand-over buffers, normalise, run the attention and write
-//     every result.  They issue no weight loads.
-// Both roles execute the same sequence of barriers.
-// ---------------------------------------------------------------------------------------------------------
-constexpr int kMegaServiceWaves = 4;
-constexpr int kMegaServiceThreads = kMegaServiceWaves * 64;
-
-// LDS of the kernel, shared by both roles.
+// LDS of the kernel.
 template <class S>
 struct MegaLds {
     static constexpr int XS = S::F > S::D ? S::F : S::D;
@@ -282,139 +280,99 @@ struct MegaLds {
     float xs[XS];                    // the phase's input vector (during attention: exp(score) of the chunk)
     float red[RED_ROWS * RED_COLS];  // per-row partial sums, one column per slab
     float xown[S::ROWS_C];           // this workgroup's rows of the residual stream
-    float scratch[8];
-    float attn_red[kMegaServiceWaves * (S::R + 1)];
+    float scratch[S::NW];
+    float attn_red[S::NW * (S::R + 1)];
 };
 
-// Service waves: bring the N-float vector at `src` into LDS, optionally normalised (normalize.comp:34-64: mean,
-// then mean-centred variance, no epsilon).  Barriers: 3 when NORM, else 1; the stream waves run the same count.
-template <int N, bool NORM>
-__device__ __forceinline__ void service_acquire(int st, float *xs, const float *src, const float *w, float *scratch, uint32_t *status)
+template <int NW>
+__device__ __forceinline__ float block_sum(float v, float *scratch /* NW floats */)
 {
-    constexpr int T = kMegaServiceThreads, PER = cdiv(N, T);
+    v = wave_sum(v);
+    lds_barrier();
+    if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = v;
+    lds_barrier();
+    float t = 0.f;
+#pragma unroll
+    for (int i = 0; i < NW; i++) t += scratch[i];
+    return t;
+}
+
+// Brings the N-float vector at `src` (being produced by other workgroups) into LDS, optionally normalised
+// (normalize.comp:34-64: mean, then mean-centred variance, no epsilon) with weights w.  One round trip to
+// memory when the data is there: the norm weights are requested before the wait, not after it.
+template <int N, int NW, bool NORM>
+__device__ __forceinline__ void acquire_vector(float *xs, const float *src, const float *w, float *scratch, uint32_t *status)
+{
+    constexpr int T = NW * 64, PER = cdiv(N, T);
     float v[PER];
     bool want[PER];
 #pragma unroll
-    for (int j = 0; j < PER; j++) want[j] = st + j * T < N;
-    poll_values<PER>(v, src + st, T, want, status);
+    for (int j = 0; j < PER; j++) want[j] = (int)threadIdx.x + j * T < N;
+    float wn[NORM ? PER : 1];
     if constexpr (NORM) {
-        const int sw = st >> 6;
+#pragma unroll
+        for (int j = 0; j < PER; j++) wn[j] = want[j] ? w[threadIdx.x + j * T] : 0.f;
+    }
+    poll_values<PER>(v, src + threadIdx.x, T, want, status);
+    if constexpr (NORM) {
         float s = 0.f;
 #pragma unroll
         for (int j = 0; j < PER; j++) s += want[j] ? v[j] : 0.f;
-        s = wave_sum(s);
-        if ((st & 63) == 0) scratch[sw] = s;
-        lds_barrier();
-        const float mean = ((scratch[0] + scratch[1]) + (scratch[2] + scratch[3])) / (float)N;
+        const float mean = block_sum<NW>(s, scratch) / (float)N;
         float q = 0.f;
 #pragma unroll
         for (int j = 0; j < PER; j++) {
             const float c = want[j] ? v[j] - mean : 0.f;
             q = fmaf(c, c, q);
         }
-        q = wave_sum(q);
-        if ((st & 63) == 0) scratch[4 + sw] = q;
-        lds_barrier();
-        const float inv = rsqrtf(((scratch[4] + scratch[5]) + (scratch[6] + scratch[7])) / (float)N);
+        const float inv = rsqrtf(block_sum<NW>(q, scratch) / (float)N);
 #pragma unroll
         for (int j = 0; j < PER; j++)
-            if (want[j]) xs[st + j * T] = (v[j] * w[st + j * T]) * inv;
+            if (want[j]) xs[threadIdx.x + j * T] = (v[j] * wn[j]) * inv;
     } else {
 #pragma unroll
         for (int j = 0; j < PER; j++)
-            if (want[j]) xs[st + j * T] = v[j];
+            if (want[j]) xs[threadIdx.x + j * T] = v[j];
     }
     lds_barrier();
 }
 
-template <bool NORM>
-__device__ __forceinline__ void stream_await_vector()
-{
-    if constexpr (NORM) { lds_barrier(); lds_barrier(); }
-    lds_barrier();
-}
-
-// ---- the stream role: weight tiles only -----------------------------------------------------------------------
 template <class S>
-__device__ __forceinline__ void mega_stream_role(const MegaArgs &a, const MegaWave<S> &mw, MegaLds<S> &l)
+__global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
 {
-    const int lane = mw.lane;
+    constexpr int D = S::D, F = S::F, H = S::H, R = S::R, NW = S::NW, T = NW * 64;
+    __shared__ __attribute__((aligned(16))) MegaLds<S> l;
+    float *xs = l.xs, *red = l.red, *xown = l.xown, *scratch = l.scratch;
+#ifdef LV_MEGA_TIMING
+    const uint64_t clk0 = clock64(), wall0 = wall_clock64();
+#endif
+    MegaWave<S> mw;
+    mw.init(a);
+    const int b = mw.b, w = mw.w, lane = mw.lane;
+    const int st = threadIdx.x;
+    uint32_t *status = a.status;
+
+    // ---- start the weight stream ------------------------------------------------------------------------------
     MegaTile q[kMegaDepth];
 #pragma unroll
     for (int k = 0; k < kMegaDepth; k++) mw.fetch(q[k], k, 0);
-    float xr[32];
-    float xsum;
-    for (uint32_t layer = 0; layer < a.layers; layer++) {
-        // A
-        stream_await_vector<true>();
-        load_slab(xr, xsum, l.xs, mw.sD * 64 + lane, mw.laneD);
-        gemv_phase<S, S::SEQ_A, S::TA, S::NSD>(q, mw, layer, xr, xsum, mw.sD, mw.rD, mw.actD, S::ROWS_A, l.red);
-        lds_barrier();
-        // B: attention runs on the service waves (two barriers of theirs)
-        lds_barrier();
-        lds_barrier();
-        // C
-        stream_await_vector<false>();
-        load_slab(xr, xsum, l.xs, mw.sD * 64 + lane, mw.laneD);
-        gemv_phase<S, S::SEQ_C, S::TC, S::NSD>(q, mw, layer, xr, xsum, mw.sD, mw.rD, mw.actD, S::ROWS_C, l.red);
-        lds_barrier();
-        // D
-        stream_await_vector<true>();
-        load_slab(xr, xsum, l.xs, mw.sD * 64 + lane, mw.laneD);
-        gemv_phase<S, S::SEQ_D, S::TD, S::NSD>(q, mw, layer, xr, xsum, mw.sD, mw.rD, mw.actD, S::ROWS_D, l.red);
-        lds_barrier();
-        // E
-        stream_await_vector<false>();
-        load_slab(xr, xsum, l.xs, mw.sF * 64 + lane, mw.laneF);
-        gemv_phase<S, S::SEQ_E, S::TE, S::NSF>(q, mw, layer, xr, xsum, mw.sF, mw.rF, mw.actF, S::ROWS_E, l.red);
-        // padding slots of the layer's sequence carry no tile, but the slot kMegaDepth ahead of them does
-#pragma unroll
-        for (int k = S::SEQ_E + S::TE; k < S::PER_LAYER; k++) mw.fetch(q[k % kMegaDepth], k + kMegaDepth, layer);
-        lds_barrier();
-    }
-    // head
-    stream_await_vector<true>();
-    load_slab(xr, xsum, l.xs, mw.sD * 64 + lane, mw.laneD);
-    const int rows = (int)mw.vocab_rows, per_set = (rows + S::NRD - 1) / S::NRD;
-    float p[4];
-#pragma unroll
-    for (int i = 0; i < kMegaHeadSlots; i++) {
-        const int slot = i % kMegaDepth;
-        const MegaTile t = q[slot];
-        p[i & 3] = (q4_block_dot(t.c, xr) - 8.f * xsum) * half_bits_to_float(t.d);
-        mw.fetch_head(q[slot], i + kMegaDepth);
-        if ((i & 3) == 3) {
-            const float s = quad_partials_sum(p[0], p[1], p[2], p[3]);
-            const int ii = (i - 3) + quad_partial_of_lane(lane);
-            const int row = mw.rD * per_set + ii;
-            if (mw.actD && (lane & 15) == 0 && ii < per_set && row < rows) l.red[row * S::NSD + mw.sD] = s;
-        }
-    }
-    lds_barrier();
-}
 
-// ---- the service role: hand-over polling, normalisation, attention, every store -------------------------------
-template <class S>
-__device__ __forceinline__ void mega_service_role(const MegaArgs &a, const MegaWave<S> &mw, MegaLds<S> &l)
-{
-    constexpr int D = S::D, F = S::F, H = S::H, R = S::R, NSV = kMegaServiceWaves;
-    const int b = mw.b, lane = mw.lane;
-    const int st = (int)threadIdx.x - S::NW * 64, sw = mw.w - S::NW;
-    uint32_t *status = a.status;
-    float *xs = l.xs, *red = l.red, *xown = l.xown;
-
-    // re-arm the other buffer set for the next token
+    // ---- re-arm the other buffer set for the next token ---------------------------------------------------------
 #ifndef LV_MEGA_NOWAIT   // (experiment builds leave stale, "ready" data in place to time the kernel without hand-over waits)
     {
         const size_t n4 = (size_t)a.layers * S::XCHG_LAYER / 4;
         uint4 *dst = reinterpret_cast<uint4 *>(a.xchg_rearm);
-        for (size_t i = (size_t)b * kMegaServiceThreads + st; i < n4; i += (size_t)kMegaWGs * kMegaServiceThreads)
+        for (size_t i = (size_t)b * T + threadIdx.x; i < n4; i += (size_t)kMegaWGs * T)
             dst[i] = make_uint4(kNotReady, kNotReady, kNotReady, kNotReady);
     }
 #endif
+
     const uint32_t pos = a.pos;
     const float *x_src = a.tok_f32 + (size_t)a.token * D;  // layer 0 reads the embedding row directly (constant data)
-    if (st < S::ROWS_C) xown[st] = x_src[b * S::ROWS_C + st];
+    if (threadIdx.x < S::ROWS_C) xown[threadIdx.x] = x_src[b * S::ROWS_C + threadIdx.x];
+
+    float xr[32];
+    float xsum;
 
     for (uint32_t layer = 0; layer < a.layers; layer++) {
         float *xc = a.xchg + (size_t)layer * S::XCHG_LAYER;
@@ -423,12 +381,14 @@ __device__ __forceinline__ void mega_service_role(const MegaArgs &a, const MegaW
 
         // ================= A: norm + QKV ====================================================================
         MEGA_STAMP(0);
-        service_acquire<D, true>(st, xs, x_src, norm_w, l.scratch, status);
+        acquire_vector<D, NW, true>(xs, x_src, norm_w, scratch, status);
         MEGA_STAMP(1);
-        lds_barrier();  // the stream waves have filled `red`
-        if (st < S::ROWS_A) {
-            const float v = red_row<S::NSD>(red, st);
-            const int g = b * S::ROWS_A + st, which = g / D, col = g % D;
+        load_slab(xr, xsum, xs, mw.sD * 64 + lane, mw.laneD);
+        gemv_phase<S, S::SEQ_A, S::TA, S::NSD>(q, mw, layer, xr, xsum, mw.sD, mw.rD, mw.actD, S::ROWS_A, red);
+        lds_barrier();
+        if (threadIdx.x < S::ROWS_A) {
+            const float v = red_row<S::NSD>(red, threadIdx.x);
+            const int g = b * S::ROWS_A + threadIdx.x, which = g / D, col = g % D;
             if (which == 0) {
                 st_dev(xc + S::OFF_QKV + col, v);
             } else {
@@ -443,53 +403,62 @@ __device__ __forceinline__ void mega_service_role(const MegaArgs &a, const MegaW
         MEGA_STAMP(2);
         {
             const int h = b / S::CPH, c = b % S::CPH;
-            const bool att = h < H;
-            const uint32_t n_valid = pos + 1;
-            uint32_t chunk = (n_valid + S::CPH - 1) / S::CPH;
-            chunk = (chunk + 3) & ~3u;
-            const uint32_t p_begin = min((uint32_t)c * chunk, n_valid), p_end = min(p_begin + chunk, n_valid);
-            const int sub = lane & 15, rsel = sw * 4 + (lane >> 4);
-            float *e_lds = xs;            // chunk <= backlog/CPH + 3 floats; xs is free between phases A and C
-            constexpr int RPR = NSV * 4;  // cache rows per round of the service waves
-            constexpr int PRE = 4;        // rounds whose K and V rows are requested before the query arrives
-            const size_t row_off = (size_t)h * R + sub * 8;
-            const bool want8[8] = {true, true, true, true, true, true, true, true};
-            auto unpack8 = [](float (&f)[8], const uint4 &raw) {
-                const uint32_t wv[4] = {raw.x, raw.y, raw.z, raw.w};
+            if (h < H) {
+                const uint32_t n_valid = pos + 1;
+                uint32_t chunk = (n_valid + S::CPH - 1) / S::CPH;
+                chunk = (chunk + 3) & ~3u;
+                const uint32_t p_begin = min((uint32_t)c * chunk, n_valid), p_end = min(p_begin + chunk, n_valid);
+                const int sub = lane & 15, rsel = w * 4 + (lane >> 4);
+                float *e_lds = xs;            // chunk <= backlog/CPH + 3 floats; xs is free between phases A and C
+                constexpr int RPR = NW * 4;   // cache rows per round of the workgroup
+                constexpr int PRE = 2;        // rounds whose K, V and rotation rows are requested before the query arrives
+                const size_t row_off = (size_t)h * R + sub * 8;
+                auto unpack8 = [](float (&f)[8], const uint4 &raw) {
+                    const uint32_t wv[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    f[2 * i] = half_bits_to_float((uint16_t)(wv[i] & 0xffffu));
-                    f[2 * i + 1] = half_bits_to_float((uint16_t)(wv[i] >> 16));
-                }
-            };
-            uint4 vpre[PRE];
-            float den = 0.f;
-            if (att) {
+                    for (int i = 0; i < 4; i++) {
+                        f[2 * i] = half_bits_to_float((uint16_t)(wv[i] & 0xffffu));
+                        f[2 * i + 1] = half_bits_to_float((uint16_t)(wv[i] >> 16));
+                    }
+                };
                 // Rows older than this token do not depend on it: ask for them first, then wait for q.
-                uint4 kpre[PRE];
+                uint4 kpre[PRE], vpre[PRE];
+                float4 tpre[PRE][2];
 #pragma unroll
                 for (int r = 0; r < PRE; r++) {
                     const uint32_t p = p_begin + r * RPR + rsel;
                     const uint32_t pc = (p < p_end && p != pos) ? p : 0;  // any valid row; unused when masked
                     kpre[r] = *reinterpret_cast<const uint4 *>(kc + (size_t)pc * D + row_off);
                     vpre[r] = *reinterpret_cast<const uint4 *>(vc + (size_t)pc * D + row_off);
+                    const float4 *tp = reinterpret_cast<const float4 *>(a.trig + (size_t)(p < p_end ? pos - p : 0) * (R / 2) + sub * 4);
+                    tpre[r][0] = tp[0];
+                    tpre[r][1] = tp[1];
                 }
-                float qv[8];
-                poll_values<8>(qv, xc + S::OFF_QKV + h * R + sub * 8, 1, want8, status);
+                // one wait for the query and, in the lanes that own the newest position, its K and V row
+                const bool newest = (pos >= p_begin && pos < p_end) && ((pos - p_begin) % RPR) == (uint32_t)rsel;
+                float qkv[24];
+                {
+                    bool want24[24];
+#pragma unroll
+                    for (int i = 0; i < 24; i++) want24[i] = i < 8 || newest;
+                    poll_values<24>(qkv, xc + S::OFF_QKV + h * R + sub * 8, 1, want24, status, D / 8);
+                }
                 MEGA_STAMP(3);
                 const float scale = rsqrtf((float)R);
-                auto score_round = [&](uint32_t p, const uint4 &kraw) {
+                float den = 0.f;
+                auto score_round = [&](uint32_t p, const uint4 &kraw, const float4 &t0, const float4 &t1) {
                     float s = 0.f;
                     if (p < p_end) {
                         float kf[8];
-                        if (p == pos) poll_values<8>(kf, xc + S::OFF_QKV + D + h * R + sub * 8, 1, want8, status);
-                        else unpack8(kf, kraw);
-                        const float4 *tp = reinterpret_cast<const float4 *>(a.trig + (size_t)(pos - p) * (R / 2) + sub * 4);
-                        const float4 t0 = tp[0], t1 = tp[1];
+                        unpack8(kf, kraw);
+                        if (p == pos) {
+#pragma unroll
+                            for (int i = 0; i < 8; i++) kf[i] = qkv[8 + i];
+                        }
                         const float ct[4] = {t0.x, t0.z, t1.x, t1.z}, stn[4] = {t0.y, t0.w, t1.y, t1.w};
 #pragma unroll
                         for (int i = 0; i < 4; i++) {
-                            const float kx = kf[2 * i], ky = kf[2 * i + 1], qx = qv[2 * i], qy = qv[2 * i + 1];
+                            const float kx = kf[2 * i], ky = kf[2 * i + 1], qx = qkv[2 * i], qy = qkv[2 * i + 1];
                             const float dotp = fmaf(qy, ky, qx * kx);
                             const float crs = fmaf(qx, ky, -(qy * kx));
                             s = fmaf(ct[i], dotp, s);
@@ -505,21 +474,23 @@ __device__ __forceinline__ void mega_service_role(const MegaArgs &a, const MegaW
                     den += (sub == 0) ? e : 0.f;
                 };
 #pragma unroll
-                for (int r = 0; r < PRE; r++) score_round(p_begin + r * RPR + rsel, kpre[r]);
+                for (int r = 0; r < PRE; r++) score_round(p_begin + r * RPR + rsel, kpre[r], tpre[r][0], tpre[r][1]);
                 for (uint32_t p0 = p_begin + PRE * RPR; p0 < p_end; p0 += RPR) {
                     const uint32_t p = p0 + rsel;
                     const uint32_t pc = (p < p_end && p != pos) ? p : 0;
-                    score_round(p, *reinterpret_cast<const uint4 *>(kc + (size_t)pc * D + row_off));
+                    const float4 *tp = reinterpret_cast<const float4 *>(a.trig + (size_t)(p < p_end ? pos - p : 0) * (R / 2) + sub * 4);
+                    score_round(p, *reinterpret_cast<const uint4 *>(kc + (size_t)pc * D + row_off), tp[0], tp[1]);
                 }
-            }
-            lds_barrier();
-            if (att) {
+                lds_barrier();
                 float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
                 auto pv_round = [&](uint32_t p, const uint4 &vraw) {
                     if (p < p_end) {
                         float vf[8];
-                        if (p == pos) poll_values<8>(vf, xc + S::OFF_QKV + 2 * D + h * R + sub * 8, 1, want8, status);
-                        else unpack8(vf, vraw);
+                        unpack8(vf, vraw);
+                        if (p == pos) {
+#pragma unroll
+                            for (int i = 0; i < 8; i++) vf[i] = qkv[16 + i];
+                        }
                         const float e = e_lds[p - p_begin];
 #pragma unroll
                         for (int i = 0; i < 8; i++) acc[i] = fmaf(e, vf[i], acc[i]);
@@ -540,39 +511,54 @@ __device__ __forceinline__ void mega_service_role(const MegaArgs &a, const MegaW
                 }
                 if (lane < 16) {
 #pragma unroll
-                    for (int i = 0; i < 8; i++) l.attn_red[sw * (R + 1) + lane * 8 + i] = acc[i];
-                    if (lane == 0) l.attn_red[sw * (R + 1) + R] = den;
+                    for (int i = 0; i < 8; i++) l.attn_red[w * (R + 1) + lane * 8 + i] = acc[i];
+                    if (lane == 0) l.attn_red[w * (R + 1) + R] = den;
                 }
-            }
-            lds_barrier();
-            if (att && st <= R) {
-                float t = 0.f;
+                lds_barrier();
+                if (st <= R) {
+                    float t = 0.f;
 #pragma unroll
-                for (int i = 0; i < NSV; i++) t += l.attn_red[i * (R + 1) + st];
-                st_dev(xc + S::OFF_PART + (h * S::CPH + c) * S::PART + st, t);
+                    for (int i = 0; i < NW; i++) t += l.attn_red[i * (R + 1) + st];
+                    st_dev(xc + S::OFF_PART + (h * S::CPH + c) * S::PART + st, t);
+                }
             }
         }
 
-        // ================= B': combine the chunks of head b =====================================================
+        // ================= B': combine the chunks of head b (one wait for numerators and denominators) ==========
         MEGA_STAMP(4);
         if (b < H && st < R) {
-            float num[S::CPH], dn[S::CPH];
-            bool want[S::CPH];
+            float nd[2 * S::CPH];
+            bool want[2 * S::CPH];
 #pragma unroll
-            for (int c = 0; c < S::CPH; c++) want[c] = true;
+            for (int c = 0; c < 2 * S::CPH; c++) want[c] = true;
             const float *hp = xc + S::OFF_PART + (size_t)b * S::CPH * S::PART;
-            poll_values<S::CPH>(num, hp + st, S::PART, want, status);
-            poll_values<S::CPH>(dn, hp + R, S::PART, want, status);
+            uint32_t spins = 0;
+            bool pending;
+            do {
+                pending = false;
+#pragma unroll
+                for (int c = 0; c < S::CPH; c++) {
+                    const uint32_t un = ld_dev(reinterpret_cast<const uint32_t *>(hp + c * S::PART + st));
+                    const uint32_t ud = ld_dev(reinterpret_cast<const uint32_t *>(hp + c * S::PART + R));
+                    nd[c] = __uint_as_float(un);
+                    nd[S::CPH + c] = __uint_as_float(ud);
+                    pending |= (un == kNotReady) | (ud == kNotReady);
+                }
+            } while (pending && ++spins < kSpinLimit);
+            if (pending) *status = 1u;
             float n = 0.f, d = 0.f;
 #pragma unroll
-            for (int c = 0; c < S::CPH; c++) { n += num[c]; d += dn[c]; }
+            for (int c = 0; c < S::CPH; c++) { n += nd[c]; d += nd[S::CPH + c]; }
             st_dev(xc + S::OFF_O + b * R + st, n / d);
         }
+        lds_barrier();  // xs (attention scratch) is about to be overwritten
 
         // ================= C: x += Wo o ============================================================================
         MEGA_STAMP(5);
-        service_acquire<D, false>(st, xs, xc + S::OFF_O, nullptr, l.scratch, status);
+        acquire_vector<D, NW, false>(xs, xc + S::OFF_O, nullptr, scratch, status);
         MEGA_STAMP(6);
+        load_slab(xr, xsum, xs, mw.sD * 64 + lane, mw.laneD);
+        gemv_phase<S, S::SEQ_C, S::TC, S::NSD>(q, mw, layer, xr, xsum, mw.sD, mw.rD, mw.actD, S::ROWS_C, red);
         lds_barrier();
         if (st < S::ROWS_C) {
             const float v = xown[st] + red_row<S::NSD>(red, st);
@@ -582,8 +568,10 @@ __device__ __forceinline__ void mega_service_role(const MegaArgs &a, const MegaW
 
         // ================= D: norm + SwiGLU ========================================================================
         MEGA_STAMP(7);
-        service_acquire<D, true>(st, xs, xc + S::OFF_X1, norm_w + D, l.scratch, status);
+        acquire_vector<D, NW, true>(xs, xc + S::OFF_X1, norm_w + D, scratch, status);
         MEGA_STAMP(8);
+        load_slab(xr, xsum, xs, mw.sD * 64 + lane, mw.laneD);
+        gemv_phase<S, S::SEQ_D, S::TD, S::NSD>(q, mw, layer, xr, xsum, mw.sD, mw.rD, mw.actD, S::ROWS_D, red);
         lds_barrier();
         if (st < S::ROWS_D / 2) {
             // rows alternate W3 row k, W1 row k (matmul_silu_ff.comp:96: result1 * result2 / (exp(-result2) + 1))
@@ -593,8 +581,13 @@ __device__ __forceinline__ void mega_service_role(const MegaArgs &a, const MegaW
 
         // ================= E: x += W2 ff ===========================================================================
         MEGA_STAMP(9);
-        service_acquire<F, false>(st, xs, xc + S::OFF_FF, nullptr, l.scratch, status);
+        acquire_vector<F, NW, false>(xs, xc + S::OFF_FF, nullptr, scratch, status);
         MEGA_STAMP(10);
+        load_slab(xr, xsum, xs, mw.sF * 64 + lane, mw.laneF);
+        gemv_phase<S, S::SEQ_E, S::TE, S::NSF>(q, mw, layer, xr, xsum, mw.sF, mw.rF, mw.actF, S::ROWS_E, red);
+        // padding slots of the layer's sequence carry no tile, but the slot kMegaDepth ahead of them does
+#pragma unroll
+        for (int k = S::SEQ_E + S::TE; k < S::PER_LAYER; k++) mw.fetch(q[k % kMegaDepth], k + kMegaDepth, layer);
         lds_barrier();
         if (st < S::ROWS_E) {
             const float v = xown[st] + red_row<S::NSF>(red, st);
@@ -606,28 +599,33 @@ __device__ __forceinline__ void mega_service_role(const MegaArgs &a, const MegaW
     }
 
     // ================= head: norm + output matrix ====================================================================
-    service_acquire<D, true>(st, xs, x_src, a.norms + (size_t)a.layers * 2 * D, l.scratch, status);
-    lds_barrier();
-    const int rows = (int)mw.vocab_rows;
-    for (int j = st; j < rows; j += kMegaServiceThreads) {
-        const uint32_t n = (uint32_t)b * rows + j;
-        if (n < a.vocab) a.logits[n] = red_row<S::NSD>(red, j);
+    {
+        acquire_vector<D, NW, true>(xs, x_src, a.norms + (size_t)a.layers * 2 * D, scratch, status);
+        load_slab(xr, xsum, xs, mw.sD * 64 + lane, mw.laneD);
+        const int rows = (int)mw.vocab_rows, per_set = (rows + S::NRD - 1) / S::NRD;
+        // the head's slots are numbered from 0; tiles beyond per_set read the dummy tile
+        float p[4];
+#pragma unroll
+        for (int i = 0; i < kMegaHeadSlots; i++) {
+            const int slot = i % kMegaDepth;
+            const MegaTile t = q[slot];
+            p[i & 3] = (q4_block_dot(t.c, xr) - 8.f * xsum) * half_bits_to_float(t.d);
+            mw.fetch_head(q[slot], i + kMegaDepth);
+            if ((i & 3) == 3) {
+                const float s = quad_partials_sum(p[0], p[1], p[2], p[3]);
+                const int ii = (i - 3) + quad_partial_of_lane(lane);
+                const int row = mw.rD * per_set + ii;
+                if (mw.actD && (lane & 15) == 0 && ii < per_set && row < rows) red[row * S::NSD + mw.sD] = s;
+            }
+        }
+        lds_barrier();
+        for (int j = st; j < rows; j += T) {
+            const uint32_t n = (uint32_t)b * rows + j;
+            if (n < a.vocab) a.logits[n] = red_row<S::NSD>(red, j);
+        }
     }
-}
-
-template <class S>
-__global__ __launch_bounds__((S::NW + kMegaServiceWaves) * 64, 1) void mega_decode_kernel(MegaArgs a)
-{
-    __shared__ __attribute__((aligned(16))) MegaLds<S> lds;
 #ifdef LV_MEGA_TIMING
-    const uint64_t clk0 = clock64(), wall0 = wall_clock64();
-#endif
-    MegaWave<S> mw;
-    mw.init(a);
-    if (mw.w < S::NW) mega_stream_role<S>(a, mw, lds);
-    else mega_service_role<S>(a, mw, lds);
-#ifdef LV_MEGA_TIMING
-    if (blockIdx.x == LV_MEGA_TIMING_WG && threadIdx.x == S::NW * 64) {
+    if (blockIdx.x == LV_MEGA_TIMING_WG && threadIdx.x == 0) {
         a.status[8] = (uint32_t)(clock64() - clk0);
         a.status[9] = (uint32_t)(wall_clock64() - wall0);
     }

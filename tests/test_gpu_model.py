@@ -145,3 +145,74 @@ def test_step_api_state_errors(lva, ctx, tiny_models):
     assert lib.lv_session_reserve(s.h, 256) == -4                                  # in flight
     assert lib.lv_step_wait(s.h) == 0
     s.close(); model.close()
+
+
+@pytest.fixture(scope="module")
+def wide_model(lva, tmp_path_factory):
+    """LLaMA-7B layer shape (dim 4096, 32 heads, ff 11008) with 2 layers and a small vocabulary: the shape class
+    the persistent decode kernel is built for."""
+    p = str(tmp_path_factory.mktemp("wide") / "wide_q4.ggml")
+    lva.write_model(p, wtype=lva.LV_Q4_0, seed=9, vocab=2048, dim=4096, heads=32, layers=2, ff=11008)
+    return p
+
+
+def test_persistent_kernel_matches_oracle_and_operator_path(lva, orc, ctx, wide_model):
+    om = orc.Model(wide_model)
+    osess = orc.Session(om, 128)
+    model = lva.Model(ctx, wide_model)
+    pk, ops = lva.Session(model, 128), lva.Session(model, 128)
+    assert pk.path() == lva.PATH_PERSISTENT          # chosen automatically for this shape
+    ops.set_path(lva.PATH_KERNELS)
+    prompt = lva.synth_tokens(8, 3, 2048, seed=1)
+    want = osess.eval(prompt)
+    pk.begin(prompt, 0)                               # prompts go through the operator path in both sessions
+    ops.begin(prompt, 0)
+    got_pk, got_ops = pk.logits(), ops.logits()
+    _check_logits(got_pk, want)
+    pos = len(prompt)
+    for step in range(24):
+        tok = orc.greedy(want)
+        assert pk.argmax() == tok == ops.argmax(), f"step {step}"
+        want = osess.eval([tok])
+        pk.begin([tok], pos)
+        ops.begin([tok], pos)
+        got_pk, got_ops = pk.logits(), ops.logits()
+        _check_logits(got_pk, want)
+        _check_logits(got_ops, want)
+        assert np.max(np.abs(got_pk - got_ops)) <= 1e-4 * np.max(np.abs(want))
+        pos += 1
+    # both paths left the same cache behind (up to fp16 rounding of differently ordered fp32 sums)
+    for layer in range(2):
+        for which in (0, 1):
+            a, b = pk.kv(layer, which, pos), ops.kv(layer, which, pos)
+            af, bf = a.view(np.float16).astype(np.float32), b.view(np.float16).astype(np.float32)
+            assert np.max(np.abs(af - bf)) <= np.max(np.abs(bf)) * 2.0 ** -9
+    pk.close(); ops.close(); model.close(); osess.close(); om.close()
+
+
+def test_persistent_kernel_is_deterministic_and_rearms(lva, ctx, wide_model):
+    """Same tokens twice from scratch give bit-identical logits (fixed summation order, hand-over buffers re-armed
+    between tokens), also when another session's steps are interleaved."""
+    model = lva.Model(ctx, wide_model)
+    a, b = lva.Session(model, 128), lva.Session(model, 128)
+    toks = lva.synth_tokens(20, 3, 2048, seed=2)
+    la, lb = [], []
+    for i, t in enumerate(toks):
+        a.begin([t], i)
+        la.append(a.logits())
+        b.begin([t], i)
+        lb.append(b.logits())
+    assert all(np.array_equal(x, y) for x, y in zip(la, lb))
+    # rewind: decode the last 5 tokens again over the same cache rows
+    for i in range(15, 20):
+        a.begin([toks[i]], i)
+        assert np.array_equal(a.logits(), la[i])
+    a.close(); b.close(); model.close()
+
+
+def test_persistent_kernel_refused_for_other_shapes(lva, ctx, tiny_models):
+    model = lva.Model(ctx, tiny_models["tiny_q4"])
+    s = lva.Session(model, 128)
+    assert s.path() == lva.PATH_GRAPH
+    assert ctx.lib.lv_session_set_path(s.h, lva.PATH_PERSISTENT) == -1
+    s.close(); model.close()
