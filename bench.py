@@ -1,0 +1,170 @@
+#!/usr/bin/env python3
+"""Decode benchmark: LLaMA-7B-shaped q4_0, batch 1, greedy, ending at a 512-token context, on one MI355X.
+
+A "step" is one decode token through the C-ABI (lv_step_begin -> lv_argmax), inputs already resident in HBM.
+Prints ONE JSON line:
+
+  value      tokens/s over the K timed steps (wall clock, host sampling included)
+  roofline   the persistent decode kernel (one launch = one token): algorithmic bytes per launch / average launch
+             duration measured with HIP events on the session's stream, against the 8 TB/s HBM peak
+  cpu_baseline  the CPU checker (oracle/) timed on a few decode steps of the same model at the same positions, on
+             this box's host cores; reported beside the GPU number, never the target
+
+Weights and prompt are synthetic (seeded writer, llama-vulkan_amd/mkggml.c).
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+CONTEXT = 512
+HBM_PEAK_GBS = 8000.0
+SHAPE = dict(vocab=32000, dim=4096, heads=32, layers=32, ff=11008)
+
+
+def algorithmic_bytes(pos):
+    """HBM bytes one decode step at cache position `pos` has to move: GGML storage cost of every weight
+    (18 B / 32 weights), fp32 norm vectors, the fp16 K/V rows 0..pos of all layers, the new K/V row, the embedding
+    row in and the logits out."""
+    D, F, V, L = SHAPE["dim"], SHAPE["ff"], SHAPE["vocab"], SHAPE["layers"]
+    per_layer = (4 * D * D + 3 * D * F) // 32 * 18
+    weights = L * per_layer + V * D // 32 * 18
+    norms = (2 * L + 1) * D * 4
+    kv_read = L * 2 * D * 2 * (pos + 1)
+    kv_write = L * 2 * D * 2
+    return weights + norms + kv_read + kv_write + V * 4 + D * 4
+
+
+def model_path():
+    base = "/dev/shm" if os.access("/dev/shm", os.W_OK) else "/tmp"
+    return os.path.join(base, "llava_bench_7b_q4_0_seed0.ggml")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--cpu-steps", type=int, default=3, help="decode steps the CPU checker is timed on (0 = skip)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs the decode path on ONE GPU (batch-1 decode has nothing to shard in this "
+                 "round); run it with --gpus 1")
+    if args.steps < 1 or args.warmup < 0 or args.steps + args.warmup >= CONTEXT:
+        sys.exit(f"bench.py: need 1 <= steps and steps + warmup < {CONTEXT}")
+
+    lva = importlib.import_module("llama-vulkan_amd")
+    ctx = lva.Context(0)
+    device, cus, _ = ctx.info()
+
+    path = model_path()
+    if not os.path.exists(path):
+        lva.write_model(path + ".tmp", wtype=lva.LV_Q4_0, seed=0, **SHAPE)
+        os.replace(path + ".tmp", path)
+    model = lva.Model(ctx, path)
+    sess = lva.Session(model, CONTEXT)
+    path_kind = {lva.PATH_KERNELS: "kernels", lva.PATH_GRAPH: "graph", lva.PATH_PERSISTENT: "persistent"}[sess.path()]
+
+    # fill the cache up to the first warm-up position with a seeded prompt, then decode greedily
+    first = CONTEXT - args.steps - args.warmup
+    prompt = lva.synth_tokens(first, 3, SHAPE["vocab"], seed=0)
+    sess.begin(prompt, 0)
+    tok = sess.argmax()
+    pos = first
+    for _ in range(args.warmup):
+        sess.begin([tok], pos)
+        tok = sess.argmax()
+        pos += 1
+
+    # ---- timed region: K steps, synchronised on both sides -------------------------------------------------
+    timed_first = pos
+    tokens = [tok]
+    sess.wait()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        sess.begin([tok], pos)
+        tok = sess.argmax()          # device argmax + 4-byte read back: the sampler is inside the step
+        tokens.append(tok)
+        pos += 1
+    sess.wait()
+    dt = time.perf_counter() - t0
+    tok_s = args.steps / dt
+
+    # ---- the dominant kernel by itself: same steps again (same cache rows, same tokens), one event pair each ----
+    kern_ms = []
+    for i in range(args.steps):
+        sess.timer_start()
+        sess.begin([tokens[i]], timed_first + i)
+        kern_ms.append(sess.timer_stop())
+    avg_ms = sum(kern_ms) / len(kern_ms)
+    avg_bytes = sum(algorithmic_bytes(timed_first + i) for i in range(args.steps)) / args.steps
+    achieved = avg_bytes / (avg_ms * 1e-3) / 1e9
+
+    # ---- CPU baseline: the checker on the same model, cache restored from the GPU session, last positions ------
+    cpu = None
+    if args.cpu_steps > 0:
+        import numpy as np
+        import oracle
+        n_cpu = min(args.cpu_steps, args.steps)
+        start = pos - n_cpu
+        om = oracle.Model(path)
+        osess = oracle.Session(om, CONTEXT)
+        for layer in range(SHAPE["layers"]):
+            for which in (0, 1):
+                osess.kv_load(layer, which, sess.kv(layer, which, start))
+        osess.set_pos(start)
+        worst = 0.0
+        t1 = time.perf_counter()
+        for i in range(n_cpu):
+            want = osess.eval([tokens[start - timed_first + i]])
+            tok_cpu = oracle.greedy(want)
+            if tok_cpu != tokens[start - timed_first + i + 1]:
+                raise SystemExit(f"bench.py: greedy token at position {start + i} differs from the CPU checker "
+                                 f"({tokens[start - timed_first + i + 1]} vs {tok_cpu})")
+        cpu_dt = time.perf_counter() - t1
+        # logits of the last step, GPU against checker
+        sess.begin([tokens[pos - 1 - timed_first]], pos - 1)
+        worst = float(np.max(np.abs(sess.logits() - want)))
+        if not worst <= min(1e-2, 1e-3 * float(np.max(np.abs(want)))):
+            raise SystemExit(f"bench.py: logits differ from the CPU checker by {worst}")
+        cpu = {"value": round(n_cpu / cpu_dt, 3), "unit": "tok/s", "cores": oracle.num_threads(), "kind": "port",
+               "sample": f"{n_cpu} greedy decode steps of the same model at positions {start}..{pos - 1} "
+                         f"(cache restored from the GPU run; tokens identical, max |dlogit| {worst:.1e})"}
+        osess.close()
+        om.close()
+
+    out = {
+        "metric": "decode tok/s LLaMA-7B q4_0 bs1 on 1 MI355X; achieved HBM GB/s vs peak",
+        "value": round(tok_s, 2),
+        "unit": "tok/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(dt / args.steps * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": f"LLaMA-7B-shaped q4_0 GGJT (dim 4096, 32 layers, 32 heads, ff 11008, vocab 32000, seed 0), "
+                               f"batch 1 greedy decode, cache positions {timed_first}..{pos - 1} of a {CONTEXT}-token context",
+                   "decode_path": path_kind, "device": device, "compute_units": cus},
+        "roofline": {"bound": "hbm", "kernel": "mega_decode_kernel (one launch per token)" if path_kind == "persistent" else "decode step (all launches)",
+                     "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "algorithmic_bytes_per_launch": int(avg_bytes), "avg_launch_ms": round(avg_ms, 4), "traffic": None},
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(out), flush=True)
+    sess.close()
+    model.close()
+    ctx.close()
+
+
+if __name__ == "__main__":
+    main()

@@ -80,6 +80,9 @@ def lib():
         L.orc_session_kv.restype = vp
         L.orc_session_trace.argtypes = [vp, u32, C.c_int, C.POINTER(u32)]
         L.orc_session_trace.restype = vp
+        L.orc_session_kv_load.argtypes = [vp, u32, C.c_int, vp, u32]
+        L.orc_session_set_pos.argtypes = [vp, u32]
+        L.orc_num_threads.argtypes = []
         _lib = L
     return _lib
 
@@ -180,6 +183,10 @@ def attention(kcache, vcache, q, pos, heads, rot):
     return kqv(vcache, softmax(mhsa(kcache, q, pos, heads, rot), pos, rot), heads, rot)
 
 
+def num_threads():
+    return int(lib().orc_num_threads())
+
+
 def greedy(logits):
     logits = _f32(logits)
     return int(lib().orc_sample_greedy(_p(logits), logits.shape[0]))
@@ -243,6 +250,15 @@ class Session:
         D = self.model.hp["dim"]
         full = np.ctypeslib.as_array(C.cast(addr, C.POINTER(C.c_uint16)), shape=(self.backlog, D))
         return full[:n_tokens].copy()
+
+    def kv_load(self, layer, which, rows):
+        rows = np.ascontiguousarray(rows, dtype=np.uint16)
+        if lib().orc_session_kv_load(self.h, layer, which, _p(rows), rows.shape[0]):
+            raise ValueError("orc_session_kv_load refused the arguments")
+
+    def set_pos(self, pos):
+        if lib().orc_session_set_pos(self.h, pos):
+            raise ValueError("position beyond the backlog")
 
     def trace(self, layer, which):
         n = C.c_uint32()

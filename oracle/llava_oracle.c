@@ -713,6 +713,31 @@ const uint16_t *orc_session_kv(const orc_session *s, uint32_t layer, int which)
     return which ? s->vc[layer] : s->kc[layer];
 }
 
+/* llava_layer_session_data.cpp:174-181 (restore_kv_cache) + llava_session.cpp:586-588: load n rows of one plane
+ * and continue from position n (call for every layer and both planes, then orc_session_set_pos). */
+int orc_session_kv_load(orc_session *s, uint32_t layer, int which, const uint16_t *rows, uint32_t n)
+{
+    if (layer >= s->m->hp.layers || n > s->backlog)
+        return -1;
+    memcpy(which ? s->vc[layer] : s->kc[layer], rows, (size_t)n * s->m->hp.dim * 2);
+    return 0;
+}
+
+int orc_session_set_pos(orc_session *s, uint32_t pos)
+{
+    if (pos > s->backlog)
+        return -1;
+    s->pos = pos;
+    return 0;
+}
+
+#ifdef _OPENMP
+#include <omp.h>
+int orc_num_threads(void) { return omp_get_max_threads(); }
+#else
+int orc_num_threads(void) { return 1; }
+#endif
+
 const float *orc_session_trace(const orc_session *s, uint32_t layer, int which, uint32_t *count)
 {
     if (layer >= s->m->hp.layers || which < 0 || which >= TR_COUNT)

@@ -88,6 +88,11 @@ void         orc_session_rewind(orc_session *s, uint32_t pos);
 int orc_session_eval(orc_session *s, const uint32_t *tokens, uint32_t n, float *logits_last, float *logits_all);
 /* raw fp16 cache rows [backlog][dim] of one layer (which: 0 = K, 1 = V) */
 const uint16_t *orc_session_kv(const orc_session *s, uint32_t layer, int which);
+/* restore n cache rows of one plane / set the position to continue from (snapshot restore) */
+int orc_session_kv_load(orc_session *s, uint32_t layer, int which, const uint16_t *rows, uint32_t n);
+int orc_session_set_pos(orc_session *s, uint32_t pos);
+/* threads the checker's row loops run on */
+int orc_num_threads(void);
 /* per-layer intermediates of the LAST row of the last eval (trace); returns dim or ff floats */
 const float *orc_session_trace(const orc_session *s, uint32_t layer, int which, uint32_t *count);
 
