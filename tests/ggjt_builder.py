@@ -1,0 +1,81 @@
+"""Builds small GGJT (v1/v3) files byte by byte from Python, independently of the C model writer, so that parser
+and tokenizer tests control every field (vocabulary pieces, scores, duplicate pieces, record order, padding)."""
+import struct
+
+import numpy as np
+
+F32, F16, Q4_0, Q8_0 = 0, 1, 2, 8
+MAGIC = 0x67676A74
+
+
+def payload_bytes(ftype, n, version=3):
+    return {F32: n * 4, F16: n * 2, Q4_0: n // 32 * (20 if version == 1 else 18), Q8_0: n // 32 * (36 if version == 1 else 34)}[ftype]
+
+
+def build(path, vocab, tensors, dim=64, heads=2, layers=1, multiple_of=256, version=3, ftype=2, tail=b""):
+    """vocab: list of (bytes, score); tensors: list of (name, ftype, shape tuple (rows, cols) or (n,), payload bytes or None
+    for a seeded fill).  Returns {name: (offset, size)}."""
+    out = bytearray()
+    out += struct.pack("<9I", MAGIC, version, len(vocab), dim, multiple_of, heads, layers, dim // heads, ftype)
+    for piece, score in vocab:
+        out += struct.pack("<i", len(piece)) + piece + struct.pack("<f", score)
+    where = {}
+    rng = np.random.default_rng(1234)
+    for name, ft, shape, data in tensors:
+        nm = name.encode()
+        if len(shape) == 2:
+            rows, cols = shape
+            out += struct.pack("<5I", 2, len(nm), ft, cols, rows)   # ne0 = columns is written first
+            n = rows * cols
+        else:
+            out += struct.pack("<4I", 1, len(nm), ft, shape[0])
+            n = shape[0]
+        out += nm
+        out += b"\0" * ((-len(out)) % 32)
+        size = payload_bytes(ft, n, version)
+        if data is None:
+            data = rng.integers(0, 256, size, dtype=np.uint8).tobytes() if ft != F32 else rng.standard_normal(n).astype(np.float32).tobytes()
+        assert len(data) == size, (name, len(data), size)
+        where[name] = (len(out), size)
+        out += data
+    out += tail
+    with open(path, "wb") as f:
+        f.write(out)
+    return where
+
+
+def minimal_tensors(dim=64, ff=96, vocab=None, wtype=Q4_0):
+    """the smallest tensor set every parser here accepts (it needs layers.0.feed_forward.w1 to learn the ff size)"""
+    t = [("tok_embeddings.weight", F32, (vocab or 8, dim), None), ("norm.weight", F32, (dim,), None), ("output.weight", wtype, (vocab or 8, dim), None)]
+    p = "layers.0."
+    for nm, shape in [("attention.wq", (dim, dim)), ("attention.wk", (dim, dim)), ("attention.wv", (dim, dim)), ("attention.wo", (dim, dim)),
+                      ("feed_forward.w1", (ff, dim)), ("feed_forward.w2", (dim, ff)), ("feed_forward.w3", (ff, dim))]:
+        t.append((p + nm + ".weight", wtype, shape, None))
+    t.append((p + "attention_norm.weight", F32, (dim,), None))
+    t.append((p + "ffn_norm.weight", F32, (dim,), None))
+    return t
+
+
+def tokenizer_vocab():
+    """A vocabulary that exercises the merge rules: byte tokens at ids 3..258, multi-byte pieces with distinct and with
+    equal scores, a piece that occurs twice (the lower id must win), UTF-8 pieces and a piece only reachable through
+    an intermediate merge."""
+    v = [(b"<unk>", 0.0), (b"<s>", 0.0), (b"</s>", 0.0)]
+    v += [(bytes([b]), -100.0 - b) for b in range(256)]            # ids 3..258
+    extra = [
+        (b"he", -1.0), (b"ll", -2.0), (b"lo", -2.0),                # 259, 260, 261: "ll" and "lo" tie on score
+        (b"hell", -3.0), (b"hello", -4.0), (b"llo", -2.5),          # 262, 263, 264
+        (b" w", -1.5), (b"or", -1.2), (b"ld", -1.1), (b"wor", -5.0), (b"world", -6.0), (b" world", -0.5),   # 265..270
+        (b"ab", -7.0), (b"ab", -0.1),                               # 271, 272: same piece twice, the first id wins and ITS score counts
+        (b"abab", -8.0),                                            # 273
+        ("é".encode(), -9.0), ("日本".encode(), -9.5), ("日".encode(), -9.6), ("本".encode(), -9.7),  # 274..277
+        (b"aa", -3.0), (b"aaa", -2.0), (b"aaaa", -1.0),             # 278..280
+        (b"xyz", -0.2),                                             # 281: no "xy" or "yz" piece, so it can never be formed
+    ]
+    return v + extra
+
+
+TOKENIZER_TEXTS = [
+    "", "h", "hello", "hello world", "hellohello", " world", "world", "ab", "abab", "ababab", "aaaaaaa", "aaaa", "xyz", "xy",
+    "é", "日本", "日本語", "héllo wörld", "\x00\x01\xff", "a" * 33, "llo", "lllo", "hell", "hel", "\xe6\x97",
+]
