@@ -1,0 +1,259 @@
+"""llava_session / llava_context (the C++ host classes in llama-vulkan_amd/host, mirroring the reference's
+llava_session.cpp and llava_context.cpp) on the GPU, against the oracle: text in, greedy tokens out, cache reuse
+between prompts, rewind, growth of the backlog, the snapshot and frame file formats and the seeded sampler."""
+import importlib
+import os
+import struct
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+PROMPT = b"The quick brown fox"
+
+
+@pytest.fixture(scope="module")
+def hl():
+    return importlib.import_module("llama-vulkan_amd.hostlib")
+
+
+@pytest.fixture(scope="module")
+def loaded(hl, tiny_models):
+    c = hl.LlavaContext()
+    assert c.load_model(tiny_models["tiny_q4"]), c.error()
+    f = hl.GgmlFile(tiny_models["tiny_q4"])
+    yield c, f, tiny_models["tiny_q4"]
+    f.close()
+    c.close()
+
+
+def oracle_greedy(orc, path, tokens, steps, backlog=128):
+    om = orc.Model(path)
+    s = orc.Session(om, backlog)
+    logits = s.eval(np.array(tokens, dtype=np.uint32))
+    out, rows = [], [logits]
+    for _ in range(steps):
+        nxt = orc.greedy(logits)
+        out.append(nxt)
+        logits = s.eval(np.array([nxt], dtype=np.uint32))
+        rows.append(logits)
+    s.close(); om.close()
+    return out, rows
+
+
+def test_greedy_text_decode_matches_oracle(hl, orc, loaded):
+    c, f, path = loaded
+    s = hl.LlavaSession(c)
+    assert s.good()
+    assert s.set_text(PROMPT)
+    toks = f.tokenize(PROMPT, True)
+    assert s.tokens() == toks and toks[0] == 1
+    want, rows = oracle_greedy(orc, path, toks, 24)
+    got = []
+    nxt = s.predict(True)
+    for i in range(24):
+        assert np.max(np.abs(s.logits() - rows[i])) <= 1e-2 + 1e-3 * np.max(np.abs(rows[i]))
+        got.append(nxt)
+        assert s.push_token(nxt)
+        assert s.start()                       # asynchronous submit ...
+        nxt = s.finish(True)                   # ... and the only wait
+    assert got == want
+    assert s.tokens_in_gpu() == len(toks) + 24
+    s.close()
+
+
+def test_set_text_reuses_the_common_prefix_and_rewind_drops_the_tail(hl, orc, loaded):
+    c, f, path = loaded
+    s = hl.LlavaSession(c)
+    assert s.set_text(PROMPT + b" jumps")
+    first = s.predict(True)
+    n_full = s.token_count()
+    assert s.tokens_in_gpu() == n_full
+    # a new text that shares a prefix keeps those cache rows (the reference compares text lengths only:
+    # llava_session.cpp:243-277; here the tokens themselves are compared)
+    assert s.set_text(PROMPT + b" sleeps")
+    shared = 0
+    a, b = f.tokenize(PROMPT + b" jumps", True), f.tokenize(PROMPT + b" sleeps", True)
+    while shared < min(len(a), len(b)) and a[shared] == b[shared]:
+        shared += 1
+    assert s.tokens_in_gpu() == shared and 0 < shared < len(b)
+    got = s.predict(True)
+    want, _ = oracle_greedy(orc, path, b, 1)
+    assert got == want[0]
+    # rewind to the first prompt's prefix and decode it again: same answer as the first time
+    s.rewind(shared)
+    assert s.token_count() == shared and s.tokens_in_gpu() == shared
+    for t in a[shared:]:
+        assert s.push_token(t)
+    assert s.predict(True) == first
+    s.rewind(10_000)                            # beyond the end: nothing happens (llava_session.cpp:390-395)
+    assert s.token_count() == len(a)
+    s.close()
+
+
+def test_add_text_appends_through_the_detokenised_text(hl, loaded):
+    c, f, _ = loaded
+    s = hl.LlavaSession(c)
+    assert s.set_text(b"abc")
+    before = s.tokens()
+    assert s.add_text(b"def")
+    # llava_session.cpp:279-282: the whole token list is turned back into text (BOS prints as "<s>") and re-tokenised
+    assert s.tokens() == f.tokenize(f.detokenize(before) + b"def", True)
+    s.close()
+
+
+def test_backlog_doubles_and_stops_at_2048(hl, orc, loaded):
+    c, f, path = loaded
+    s = hl.LlavaSession(c)
+    assert s.backlog() == 128 and s.spevars()["backlog"] == 128 and s.spevars()["backlog_bits"] == 7
+    rng = np.random.default_rng(0)
+    toks = [1] + [int(t) for t in rng.integers(3, 512, 139)]
+    for t in toks[:128]:
+        assert s.push_token(t)
+    assert s.backlog() == 128
+    first = s.predict(True)                     # 128 rows are in the cache now
+    for t in toks[128:]:
+        assert s.push_token(t)                  # grows to 256 and keeps the cached rows
+    assert s.backlog() == 256 and s.spevars()["backlog"] == 256 and s.tokens_in_gpu() == 128
+    got = s.predict(True)
+    om = orc.Model(path)
+    o = orc.Session(om, 256)
+    assert orc.greedy(o.eval(np.array(toks[:128], dtype=np.uint32))) == first
+    want = o.eval(np.array(toks[128:], dtype=np.uint32))
+    assert got == orc.greedy(want)
+    assert np.max(np.abs(s.logits() - want)) <= 1e-2 + 1e-3 * np.max(np.abs(want))
+    o.close(); om.close()
+    assert not s.push_token(1 << 20)            # not a token of this vocabulary
+    assert s.set_text(b"x" * 300)               # 301 tokens: 512 rows
+    assert s.backlog() == 512
+    assert not s.set_text(b"y" * 3000)          # would need more than 2048 rows (llava_session.cpp:253-262)
+    assert s.backlog() == 512 and s.token_count() == 301
+    s.close()
+
+
+def test_snapshot_file_format_and_restore(hl, orc, loaded, tmp_path):
+    c, f, path = loaded
+    s = hl.LlavaSession(c)
+    assert s.set_text(PROMPT)
+    first = s.predict(True)
+    toks = s.tokens()
+    n = len(toks)
+    snap = str(tmp_path / "snap.bin")
+    assert s.snapshot(snap) == hl.RC_OK
+    raw = open(snap, "rb").read()
+    dim, layers = 256, 2
+    # llava_session.cpp:447-520: u32 n, the tokens, then per layer the K rows followed by the V rows, fp16
+    assert len(raw) == 4 + 4 * n + layers * 2 * n * dim * 2
+    assert struct.unpack_from("<I", raw)[0] == n
+    assert list(struct.unpack_from(f"<{n}I", raw, 4)) == toks
+    om = orc.Model(path)
+    o = orc.Session(om, 128)
+    o.eval(np.array(toks, dtype=np.uint32))
+    body = np.frombuffer(raw, dtype=np.uint16, offset=4 + 4 * n).reshape(layers, 2, n, dim)
+    for layer in range(layers):
+        for which in range(2):
+            want = o.kv(layer, which, n)
+            diff = np.abs(body[layer, which].view(np.float16).astype(np.float32) - want.view(np.float16).astype(np.float32))
+            assert np.mean(body[layer, which] != want) < 1e-2 and np.max(diff) <= 2e-3 * max(1.0, np.max(np.abs(want.view(np.float16).astype(np.float32))))
+    o.close(); om.close()
+
+    # a fresh session restored from the file continues exactly like the one that wrote it
+    t = hl.LlavaSession(c)
+    assert t.restore(snap) == hl.RC_OK
+    assert t.tokens() == toks and t.tokens_in_gpu() == n
+    assert s.push_token(first) and t.push_token(first)
+    a, b = s.predict(True), t.predict(True)
+    assert a == b and np.array_equal(s.logits(), t.logits())
+
+    # malformed snapshot files are refused and leave the session as it was (llava_session.cpp:522-603)
+    before = t.tokens()
+    open(str(tmp_path / "short.bin"), "wb").write(b"\x01\x00")
+    assert t.restore(str(tmp_path / "short.bin")) == hl.RC_NOK
+    open(str(tmp_path / "cut.bin"), "wb").write(raw[:-2])
+    assert t.restore(str(tmp_path / "cut.bin")) == hl.RC_NOK
+    open(str(tmp_path / "huge.bin"), "wb").write(struct.pack("<I", 1 << 30) + raw[4:])
+    assert t.restore(str(tmp_path / "huge.bin")) == hl.RC_NOK
+    assert t.restore(str(tmp_path / "absent.bin")) == hl.RC_NOK
+    assert t.restore(str(tmp_path)) == hl.RC_NOK
+    assert t.tokens() == before
+    s.close(); t.close()
+
+
+def test_save_frame_needs_tracing_and_writes_named_buffers(hl, orc, loaded, tmp_path):
+    c, f, path = loaded
+    s = hl.LlavaSession(c)
+    frame = str(tmp_path / "frame.bin")
+    assert not s.is_tracing()
+    assert s.save_frame(frame) == hl.RC_NOT_TRACING
+    assert s.set_options(1) == hl.RC_OK and s.is_tracing()
+    assert s.set_text(PROMPT)
+    s.predict(True)
+    assert s.save_frame(frame) == hl.RC_OK
+    raw = open(frame, "rb").read()
+    om = orc.Model(path)
+    o = orc.Session(om, 128)
+    o.eval(np.array(s.tokens(), dtype=np.uint32))
+    which = {"normalized_input_logit": 0, "post_attn_logit": 1, "post_attn_norm_logit": 2, "ff_result": 3, "output_logit": 4}
+    cur, seen = 0, []
+    while cur < len(raw):
+        # llava_buffer.cpp:497-522: two shape words, the type, the name, zeros up to a multiple of 32, the values
+        count, rows, ftype = struct.unpack_from("<3I", raw, cur)
+        name = raw[cur + 12:raw.index(b"\0", cur + 12)].decode()
+        head = (12 + len(name) + 1 + 31) // 32 * 32
+        vals = np.frombuffer(raw, dtype=np.float32, count=count * rows, offset=cur + head)
+        cur += head + 4 * count * rows
+        assert ftype == 0 and rows == 1
+        _, layer, slot = name.split(".")
+        want = o.trace(int(layer), which[slot])
+        assert vals.shape == want.shape and np.max(np.abs(vals - want)) <= 1e-4 * max(1.0, np.max(np.abs(want))), name
+        seen.append(name)
+    assert cur == len(raw) and len(seen) == 2 * 5 and seen[0] == "layer.0.ff_result"
+    o.close(); om.close()
+    assert s.set_options(0) == hl.RC_OK and not s.is_tracing()
+    s.close()
+
+
+def test_seeded_sampler_is_reproducible_and_picks_plausible_tokens(hl, loaded):
+    c, f, _ = loaded
+    runs = []
+    for seed in (7, 7, 8):
+        s = hl.LlavaSession(c)
+        s.seed(seed)
+        assert s.set_text(PROMPT)
+        out = []
+        for _ in range(16):
+            t = s.predict(False)
+            assert t != 0xFFFFFFFF
+            # the sampler keeps tokens that are at least 2^-mu likely at temperature 0.8 (llava_session.cpp:169-195);
+            # whatever mu is, the pick can never be less likely than 2^-64
+            p = np.exp(s.logits().astype(np.float64) / 0.8)
+            assert p[t] / p.sum() > 2.0 ** -64
+            out.append(t)
+            assert s.push_token(t)
+        runs.append(out)
+        s.close()
+    assert runs[0] == runs[1]
+    assert len(set(runs[0])) > 1
+
+
+def test_cli_prints_the_greedy_continuation(hl, orc, loaded):
+    c, f, path = loaded
+    exe = os.path.join(os.path.dirname(hl.__file__), "bin", "llava")
+    assert os.path.exists(exe), "llama-vulkan_amd/bin/llava is not built"
+    toks = f.tokenize(PROMPT, True)
+    want, _ = oracle_greedy(orc, path, toks, 12)
+    text = PROMPT
+    for t in want:
+        if t == 2:
+            break
+        text += f.token(t)[0]
+    r = subprocess.run([exe, "-m", path, "--greedy", "-n", "12", PROMPT.decode()], capture_output=True, timeout=120)
+    assert r.returncode == 0, r.stderr.decode(errors="replace")
+    assert r.stdout.rstrip(b"\n") == text.rstrip(b"\n")
+    r = subprocess.run([exe, "-m", path, "-s", "x"], capture_output=True, timeout=60)
+    assert r.returncode != 0                       # the server mode is not part of this build
+    r = subprocess.run([exe, "-m", path + ".absent", "hi"], capture_output=True, timeout=60)
+    assert r.returncode != 0 and b"absent" in r.stderr
