@@ -179,7 +179,10 @@ extern "C" int lv_ctx_destroy(lv_ctx *c)
 extern "C" int lv_ctx_info(const lv_ctx *c, char *name, size_t cap, uint32_t *cus, uint64_t *hbm)
 {
     if (!c) return fail(LV_ERR_ARG, "lv_ctx_info: ctx is null");
-    if (name && cap) snprintf(name, cap, "%s (%s)", c->props.name, c->props.gcnArchName);
+    if (name && cap) {
+        if (c->props.name[0]) snprintf(name, cap, "%s (%s)", c->props.name, c->props.gcnArchName);
+        else snprintf(name, cap, "%s", c->props.gcnArchName);  // some driver set-ups report no marketing name
+    }
     if (cus) *cus = (uint32_t)c->props.multiProcessorCount;
     if (hbm) *hbm = (uint64_t)c->props.totalGlobalMem;
     return LV_OK;

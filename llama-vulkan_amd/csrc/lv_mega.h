@@ -3,7 +3,7 @@
 // Why: at batch 1 a layer is five tiny dependent GEMVs (1-6 us of HBM time each).  Launched one by one
 // they spend more time draining, launching and refilling the memory pipeline than streaming weights.
 // Here one workgroup per CU stays resident for the whole token; every wavefront walks its own contiguous
-// weight stream with a 12-deep register queue of 128-bit loads that keeps running across the phase
+// weight stream with a kMegaDepth-deep (4) register queue of 128-bit loads that keeps running across the phase
 // boundaries, so HBM stays busy while the workgroups exchange the small activation vectors.
 //
 // Phases of a layer (llava_layer.cpp:53-73), each separated by a data hand-over through HBM/L2:
