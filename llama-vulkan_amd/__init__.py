@@ -110,6 +110,7 @@ _HIP_SIGS = {
     "lv_matrix_bytes": [_VP, C.POINTER(_U64)],
     "lv_kernel_dequant": [_VP, _VP, _U32, _U32, _VP],
     "lv_kernel_gemv": [_VP, _VP, _VP, _VP, _U32, _I],
+    "lv_kernel_gemm": [_VP, _VP, _VP, _VP, _U32, _I],
     "lv_kernel_gemv_silu": [_VP, _VP, _VP, _VP, _VP, _U32],
     "lv_kernel_normalize": [_VP, _VP, _VP, _VP, _U32, _U32],
     "lv_kernel_kv_append": [_VP, _VP, _VP, _U32, _U32, _U32, _U32],

@@ -19,6 +19,7 @@
 
 #include "lv_kernels.h"
 #include "lv_mega.h"
+#include "lv_gemm.h"
 
 using namespace lv;
 
@@ -121,6 +122,12 @@ struct lv_session {
     hipGraphExec_t graph_exec = nullptr;
     bool use_graph = true;
     int path = LV_PATH_AUTO;
+    // workspace of the batched prompt path, allocated at first use: activations for pf_cap tokens
+    uint32_t pf_cap = 0, pf_backlog = 0;
+    float *pf_x = nullptr, *pf_xn = nullptr, *pf_q = nullptr, *pf_k = nullptr, *pf_v = nullptr, *pf_vo = nullptr, *pf_g1 = nullptr, *pf_g2 = nullptr;
+    uint16_t *pf_xh = nullptr, *pf_xl = nullptr;
+    float *pf_part = nullptr;
+    uint32_t *pf_counters = nullptr;
     float *xchg[2] = {nullptr, nullptr};  // hand-over buffer sets of the persistent kernel
     uint32_t xchg_turn = 0;
     uint32_t *status_host = nullptr;      // pinned, written by the persistent kernel when a poll expires
@@ -514,6 +521,52 @@ extern "C" int lv_kernel_gemv_silu(lv_ctx *c, float *out, const lv_matrix *w3, c
     return launch_gemv(c->stream, out, *w3, w1, x, batch, kGemvSilu);
 }
 
+// out[n][ldo] (+)= x[n][K] * W^T on the matrix cores; xh/xl = workspace for the fp16 halves of x, n_pad rows
+static int launch_gemm_presplit(hipStream_t st, float *out, uint32_t ldo, const lv_matrix &w, uint32_t n, const uint16_t *xh, const uint16_t *xl,
+                                bool accumulate);
+
+static int launch_gemm(hipStream_t st, float *out, uint32_t ldo, const lv_matrix &w, const float *x, uint32_t n, uint16_t *xh, uint16_t *xl,
+                       bool accumulate)
+{
+    const uint32_t K = w.view.cols, n_pad = (n + kGemmTile - 1) / kGemmTile * kGemmTile;
+    if (K % 32) return fail(LV_ERR_ARG, "gemm: %u columns", K);
+    split_half_kernel<<<dim3((K / 4 + 255) / 256, n_pad), dim3(256), 0, st>>>(xh, xl, x, n, K);
+    HIP_TRY(hipGetLastError());
+    return launch_gemm_presplit(st, out, ldo, w, n, xh, xl, accumulate);
+}
+
+// the same with the activations already split (one split serves wq, wk, wv or w3, w1)
+static int launch_gemm_presplit(hipStream_t st, float *out, uint32_t ldo, const lv_matrix &w, uint32_t n, const uint16_t *xh, const uint16_t *xl,
+                                bool accumulate)
+{
+    const uint32_t n_pad = (n + kGemmTile - 1) / kGemmTile * kGemmTile;
+    GemmArgs a{};
+    a.out = out; a.xh = xh; a.xl = xl; a.w = w.view; a.n = n; a.ldo = ldo; a.accumulate = accumulate ? 1 : 0;
+    const dim3 grid((w.view.rows + kGemmTile - 1) / kGemmTile, n_pad / kGemmTile);
+    if (w.ftype == LV_Q4_0) gemm_kernel<4><<<grid, dim3(256), 0, st>>>(a);
+    else if (w.ftype == LV_Q8_0) gemm_kernel<8><<<grid, dim3(256), 0, st>>>(a);
+    else return fail(LV_ERR_ARG, "gemm: matrix type %u", w.ftype);
+    HIP_TRY(hipGetLastError());
+    return LV_OK;
+}
+
+extern "C" int lv_kernel_gemm(lv_ctx *c, float *out, const lv_matrix *w, const float *x, uint32_t batch, int accumulate)
+{
+    if (!c || !out || !w || !x) return fail(LV_ERR_ARG, "lv_kernel_gemm: null argument");
+    if (batch == 0) return LV_OK;
+    if (batch > kMaxStepTokens) return fail(LV_ERR_RANGE, "lv_kernel_gemm: batch %u (limit %u)", batch, kMaxStepTokens);
+    HIP_TRY(hipSetDevice(c->device));
+    const size_t n_pad = (batch + kGemmTile - 1) / kGemmTile * kGemmTile, halfs = n_pad * w->view.cols;
+    uint16_t *xh = nullptr, *xl = nullptr;
+    HIP_TRY(hipMalloc(reinterpret_cast<void **>(&xh), halfs * 2));
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&xl), halfs * 2);
+    int rc = e == hipSuccess ? launch_gemm(c->stream, out, w->view.rows, *w, x, batch, xh, xl, accumulate != 0) : fail(LV_ERR_OOM, "lv_kernel_gemm: workspace");
+    (void)hipStreamSynchronize(c->stream);
+    (void)hipFree(xh);
+    (void)hipFree(xl);
+    return rc;
+}
+
 extern "C" int lv_kernel_normalize(lv_ctx *c, float *out, const float *x, const float *w, uint32_t dim, uint32_t batch)
 {
     if (!c || !out || !x || !w) return fail(LV_ERR_ARG, "lv_kernel_normalize: null argument");
@@ -806,7 +859,8 @@ extern "C" int lv_session_destroy(lv_session *s)
     if (s->stream) (void)hipStreamSynchronize(s->stream);
     drop_graph(s);
     void *dev[] = {s->kv, s->trig, s->x, s->xn, s->q, s->k, s->v, s->vo, s->ff, s->logits, s->attn_part, s->attn_counters,
-                   s->cfg, s->argmax_dev, s->trace_buf};
+                   s->cfg, s->argmax_dev, s->trace_buf, s->pf_x, s->pf_xn, s->pf_q, s->pf_k, s->pf_v, s->pf_vo, s->pf_g1, s->pf_g2,
+                   s->pf_xh, s->pf_xl, s->pf_part, s->pf_counters};
     for (void *p : dev) (void)hipFree(p);
     (void)hipFree(s->xchg[0]);
     (void)hipFree(s->xchg[1]);
@@ -1034,6 +1088,97 @@ static int record_token(lv_session *s, uint32_t idx, bool with_head)
     return LV_OK;
 }
 
+// ---- batched prompt evaluation -----------------------------------------------------------------------------
+constexpr uint32_t kPrefillChunk = 512;    // tokens evaluated together (bounds the workspace)
+constexpr uint32_t kPrefillMin = 16;       // below this the rows go through the one-token kernels
+
+static int prefill_reserve(lv_session *s, uint32_t n)
+{
+    const lv_hparams &hp = s->model->hp;
+    const size_t D = hp.dim, F = hp.ff;
+    const uint32_t cap = (n + kGemmTile - 1) / kGemmTile * kGemmTile;
+    if (cap > s->pf_cap) {
+        HIP_TRY(hipStreamSynchronize(s->stream));
+        void **bufs[] = {(void **)&s->pf_x, (void **)&s->pf_xn, (void **)&s->pf_q, (void **)&s->pf_k, (void **)&s->pf_v, (void **)&s->pf_vo,
+                         (void **)&s->pf_g1, (void **)&s->pf_g2, (void **)&s->pf_xh, (void **)&s->pf_xl};
+        const size_t sizes[] = {D * 4, D * 4, D * 4, D * 4, D * 4, D * 4, F * 4, F * 4, (F > D ? F : D) * 2, (F > D ? F : D) * 2};
+        s->pf_cap = 0;
+        for (int i = 0; i < 10; i++) {
+            (void)hipFree(*bufs[i]);
+            *bufs[i] = nullptr;
+            hipError_t e = hipMalloc(bufs[i], sizes[i] * cap);
+            if (e != hipSuccess) return fail(e == hipErrorOutOfMemory ? LV_ERR_OOM : LV_ERR_HIP, "prompt workspace: %s", hipGetErrorString(e));
+        }
+        s->pf_cap = cap;
+        s->pf_backlog = 0;
+    }
+    if (s->pf_backlog != s->backlog) {
+        HIP_TRY(hipStreamSynchronize(s->stream));
+        (void)hipFree(s->pf_part);
+        (void)hipFree(s->pf_counters);
+        s->pf_part = nullptr; s->pf_counters = nullptr; s->pf_backlog = 0;
+        const uint32_t splits = (s->backlog + kAttnChunk - 1) / kAttnChunk;
+        HIP_TRY(hipMalloc(reinterpret_cast<void **>(&s->pf_part), attn_part_floats(s->pf_cap, hp.heads, splits, hp.rot) * sizeof(float)));
+        HIP_TRY(hipMalloc(reinterpret_cast<void **>(&s->pf_counters), (size_t)s->pf_cap * hp.heads * 4));
+        LV_TRY(zero_async(s->pf_counters, (size_t)s->pf_cap * hp.heads * 4, s->stream));
+        s->pf_backlog = s->backlog;
+    }
+    return LV_OK;
+}
+
+// Rows idx0 .. idx0+n-1 of the step at once (llava_layer.cpp:39-75 with batch > 1).  Row z sees cache rows
+// 0..pos+z: all K/V rows of the chunk are appended before any row attends, rows above its own are masked.
+static int record_prefill(lv_session *s, uint32_t idx0, uint32_t n, bool with_head)
+{
+    const lv_model *m = s->model;
+    const lv_hparams &hp = m->hp;
+    const uint32_t D = hp.dim, F = hp.ff;
+    hipStream_t st = s->stream;
+    const uint32_t *pos_ptr = s->cfg, *tok_ptr = s->cfg + 1 + idx0;
+    LV_TRY(prefill_reserve(s, n));
+
+    if (m->tok_ftype == LV_F32)
+        embed_f32_kernel<<<dim3((D + 255) / 256, n), dim3(256), 0, st>>>(s->pf_x, m->tok_f32, tok_ptr, D);
+    else if (m->tok_ftype == LV_Q4_0)
+        embed_quant_kernel<4><<<dim3((D / 32 + 63) / 64, n), dim3(64), 0, st>>>(s->pf_x, m->tok_quant.view, tok_ptr);
+    else
+        embed_quant_kernel<8><<<dim3((D / 32 + 63) / 64, n), dim3(64), 0, st>>>(s->pf_x, m->tok_quant.view, tok_ptr);
+    HIP_TRY(hipGetLastError());
+
+    const dim3 kv_grid((D + 255) / 256, n);
+    for (uint32_t li = 0; li < hp.layers; li++) {
+        const LayerWeights &lw = m->layers[li];
+        normalize_kernel<<<dim3(n), dim3(256), 0, st>>>(s->pf_xn, s->pf_x, lw.attn_norm, D);
+        HIP_TRY(hipGetLastError());
+        split_half_kernel<<<dim3((D / 4 + 255) / 256, (n + kGemmTile - 1) / kGemmTile * kGemmTile), dim3(256), 0, st>>>(s->pf_xh, s->pf_xl, s->pf_xn, n, D);
+        LV_TRY(launch_gemm_presplit(st, s->pf_q, D, lw.wq, n, s->pf_xh, s->pf_xl, false));
+        LV_TRY(launch_gemm_presplit(st, s->pf_k, D, lw.wk, n, s->pf_xh, s->pf_xl, false));
+        LV_TRY(launch_gemm_presplit(st, s->pf_v, D, lw.wv, n, s->pf_xh, s->pf_xl, false));
+        kv_append_kernel<<<kv_grid, dim3(256), 0, st>>>(kv_ptr(s, li, 0), s->pf_k, pos_ptr, idx0, D, s->backlog);
+        kv_append_kernel<<<kv_grid, dim3(256), 0, st>>>(kv_ptr(s, li, 1), s->pf_v, pos_ptr, idx0, D, s->backlog);
+        HIP_TRY(hipGetLastError());
+        LV_TRY(launch_attention(st, s->pf_vo, kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->pf_q, s->trig, s->pf_part, s->pf_counters, pos_ptr, idx0,
+                                s->backlog, hp.heads, hp.rot, n));
+        LV_TRY(launch_gemm(st, s->pf_x, D, lw.wo, s->pf_vo, n, s->pf_xh, s->pf_xl, true));
+        normalize_kernel<<<dim3(n), dim3(256), 0, st>>>(s->pf_xn, s->pf_x, lw.ffn_norm, D);
+        HIP_TRY(hipGetLastError());
+        split_half_kernel<<<dim3((D / 4 + 255) / 256, (n + kGemmTile - 1) / kGemmTile * kGemmTile), dim3(256), 0, st>>>(s->pf_xh, s->pf_xl, s->pf_xn, n, D);
+        LV_TRY(launch_gemm_presplit(st, s->pf_g1, F, lw.w3, n, s->pf_xh, s->pf_xl, false));
+        LV_TRY(launch_gemm_presplit(st, s->pf_g2, F, lw.w1, n, s->pf_xh, s->pf_xl, false));
+        const size_t count = (size_t)n * F;
+        silu_mul_kernel<<<dim3((unsigned)((count + 255) / 256)), dim3(256), 0, st>>>(s->pf_g1, s->pf_g1, s->pf_g2, count);
+        HIP_TRY(hipGetLastError());
+        LV_TRY(launch_gemm(st, s->pf_x, D, lw.w2, s->pf_g1, n, s->pf_xh, s->pf_xl, true));
+    }
+    if (with_head) {
+        // only the last row's logits are ever read (llava_session.cpp:131-139)
+        normalize_kernel<<<dim3(1), dim3(256), 0, st>>>(s->xn, s->pf_x + (size_t)(n - 1) * D, m->norm, D);
+        HIP_TRY(hipGetLastError());
+        LV_TRY(launch_gemv(st, s->logits, m->output, nullptr, s->xn, 1, kGemvStore));
+    }
+    return LV_OK;
+}
+
 extern "C" int lv_step_begin(lv_session *s, const uint32_t *tokens, uint32_t n, uint32_t pos)
 {
     if (!s || !tokens) return fail(LV_ERR_ARG, "lv_step_begin: null argument");
@@ -1074,7 +1219,14 @@ extern "C" int lv_step_begin(lv_session *s, const uint32_t *tokens, uint32_t n, 
     } else {
         // rows are evaluated one after the other: row z sees cache rows 0..pos+z, which is what the batched
         // shaders compute (every row's K/V is appended before any row attends, and rows above are masked)
-        for (uint32_t i = 0; i < n; i++) LV_TRY(record_token(s, i, i + 1 == n));
+        if (n >= kPrefillMin && !s->trace) {
+            for (uint32_t i = 0; i < n; i += kPrefillChunk) {
+                const uint32_t m = n - i < kPrefillChunk ? n - i : kPrefillChunk;
+                LV_TRY(record_prefill(s, i, m, i + m == n));
+            }
+        } else {
+            for (uint32_t i = 0; i < n; i++) LV_TRY(record_token(s, i, i + 1 == n));
+        }
     }
     s->in_flight = true;
     s->have_logits = true;

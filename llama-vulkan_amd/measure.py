@@ -1,0 +1,149 @@
+#!/usr/bin/env python3
+"""Measurements of the decode path beyond the headline bench: one JSON line per case.
+
+    python llama-vulkan_amd/measure.py gemv          isolated dequant-fused GEMVs at the 7B shapes, q4_0 and q8_0
+    python llama-vulkan_amd/measure.py decode-q8     7B q8_0, cache positions 1920..2047 (128 greedy steps)
+    python llama-vulkan_amd/measure.py decode-13b    13B q4_0, 32-token prompt + 256 greedy steps
+    python llama-vulkan_amd/measure.py prefill-13b   13B q8_0, 512-token prompt evaluated in one lv_step_begin
+    python llama-vulkan_amd/measure.py all
+
+Every figure is algorithmic bytes (weights as stored in the GGML file, 18 B / 34 B per 32 weights, plus vectors and the
+fp16 cache rows a step reads) divided by the time measured with HIP events on the stream that runs the kernels.
+Models are seeded synthetic GGJT files written to /dev/shm (or /tmp) on first use."""
+import importlib
+import json
+import os
+import sys
+import time
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.dirname(HERE))
+lva = importlib.import_module("llama-vulkan_amd")
+HBM_PEAK_GBS = 8000.0
+SHAPES = {"7b": dict(vocab=32000, dim=4096, heads=32, layers=32, ff=11008), "13b": dict(vocab=32000, dim=5120, heads=40, layers=40, ff=13824)}
+
+
+def emit(**kw):
+    print(json.dumps(kw), flush=True)
+
+
+def block_bytes(ftype):
+    return 18 if ftype == lva.LV_Q4_0 else 34
+
+
+def gemv_cases(ctx):
+    """reference: matmul.glsl / matmul_q8.glsl / matmul_silu_ff.comp at the three layer shapes and the output matrix"""
+    for ftype, tname in ((lva.LV_Q4_0, "q4_0"), (lva.LV_Q8_0, "q8_0")):
+        for rows, cols, mode in ((4096, 4096, "store"), (11008, 4096, "silu"), (4096, 11008, "add"), (32000, 4096, "store")):
+            nbytes = rows * cols // 32 * block_bytes(ftype) * (2 if mode == "silu" else 1) + 4 * cols + 4 * rows * (2 if mode == "add" else 1)
+            # enough distinct matrices that the working set exceeds the 256 MB last-level cache
+            nmat = max(2, min(12, int(1.5e9 // nbytes)))
+            mats = []
+            for i in range(nmat * (2 if mode == "silu" else 1)):
+                mats.append(ctx.matrix(lva.synth_quant(ftype, rows, cols, seed=100 + i), ftype, rows, cols))
+            x = ctx.to_device(lva.synth_normal(1, cols, seed=1))
+            out = ctx.zeros(rows * 4)
+
+            def run(i):
+                if mode == "silu":
+                    lva.check(ctx.lib.lv_kernel_gemv_silu(ctx.h, out, mats[2 * i], mats[2 * i + 1], x, 1))
+                else:
+                    lva.check(ctx.lib.lv_kernel_gemv(ctx.h, out, mats[i], x, 1, 1 if mode == "add" else 0))
+            for i in range(nmat):
+                run(i)
+            ctx.sync()
+            iters = 20
+            ctx.timer_start()
+            for _ in range(iters):
+                for i in range(nmat):
+                    run(i)
+            us = ctx.timer_stop() * 1e3 / (iters * nmat)
+            emit(case="gemv", wtype=tname, rows=rows, cols=cols, mode=mode, us=round(us, 2), algorithmic_bytes=nbytes,
+                 GBps=round(nbytes / us / 1e3, 1), frac_of_peak=round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4))
+            for m in mats:
+                ctx.matrix_free(m)
+            ctx.free(x)
+            ctx.free(out)
+
+
+def model_file(preset, wtype, seed):
+    base = "/dev/shm" if os.access("/dev/shm", os.W_OK) else "/tmp"
+    path = os.path.join(base, f"llava_measure_{preset}_{'q4_0' if wtype == lva.LV_Q4_0 else 'q8_0'}_seed{seed}.ggml")
+    if not os.path.exists(path):
+        lva.write_model(path + ".tmp", wtype=wtype, seed=seed, **SHAPES[preset])
+        os.replace(path + ".tmp", path)
+    return path
+
+
+def step_bytes(shape, wtype, pos):
+    D, F, V, L = shape["dim"], shape["ff"], shape["vocab"], shape["layers"]
+    per_layer = (4 * D * D + 3 * D * F) // 32 * block_bytes(wtype)
+    return L * per_layer + V * D // 32 * block_bytes(wtype) + (2 * L + 1) * D * 4 + L * 2 * D * 2 * (pos + 2) + V * 4 + D * 4
+
+
+def decode_case(ctx, name, preset, wtype, seed, backlog, first, steps):
+    shape = SHAPES[preset]
+    path = model_file(preset, wtype, seed)
+    model = lva.Model(ctx, path)
+    s = lva.Session(model, backlog)
+    kind = {lva.PATH_KERNELS: "kernels", lva.PATH_GRAPH: "graph", lva.PATH_PERSISTENT: "persistent"}[s.path()]
+    prompt = lva.synth_tokens(first, 3, shape["vocab"], seed=seed)
+    t0 = time.perf_counter()
+    s.begin(prompt, 0)
+    tok = s.argmax()
+    prefill_s = time.perf_counter() - t0
+    pos = first
+    for _ in range(4):
+        s.begin([tok], pos)
+        tok = s.argmax()
+        pos += 1
+    t0 = time.perf_counter()
+    total = 0
+    for _ in range(steps):
+        s.begin([tok], pos)
+        tok = s.argmax()
+        total += step_bytes(shape, wtype, pos)
+        pos += 1
+    dt = time.perf_counter() - t0
+    emit(case=name, model=preset, wtype="q4_0" if wtype == lva.LV_Q4_0 else "q8_0", path=kind, positions=[first + 4, pos - 1], steps=steps,
+         tok_s=round(steps / dt, 1), ms_per_token=round(dt / steps * 1e3, 4), GBps=round(total / dt / 1e9, 1),
+         frac_of_peak=round(total / dt / 1e9 / HBM_PEAK_GBS, 4), prompt_tokens=first, prompt_s=round(prefill_s, 3))
+    s.close()
+    model.close()
+
+
+def prefill_case(ctx):
+    shape, wtype = SHAPES["13b"], lva.LV_Q8_0
+    path = model_file("13b", wtype, 3)
+    model = lva.Model(ctx, path)
+    s = lva.Session(model, 512)
+    prompt = lva.synth_tokens(512, 3, shape["vocab"], seed=3)
+    s.begin(prompt[:8], 0)
+    s.wait()
+    s.timer_start()
+    s.begin(prompt, 0)
+    ms = s.timer_stop()
+    D, F, V, L = shape["dim"], shape["ff"], shape["vocab"], shape["layers"]
+    flops = 2.0 * 512 * (L * (4 * D * D + 3 * D * F) + V * D)
+    emit(case="prefill-13b", model="13b", wtype="q8_0", tokens=512, ms=round(ms, 2), tok_s=round(512 / ms * 1e3, 1), TFLOPs=round(flops / ms / 1e9, 2))
+    s.close()
+    model.close()
+
+
+def main():
+    which = sys.argv[1] if len(sys.argv) > 1 else "all"
+    ctx = lva.Context(0)
+    name, cus, hbm = ctx.info()
+    emit(case="device", name=name, compute_units=cus, hbm_GiB=hbm >> 30)
+    if which in ("gemv", "all"):
+        gemv_cases(ctx)
+    if which in ("decode-q8", "all"):
+        decode_case(ctx, "decode-q8", "7b", lva.LV_Q8_0, 1, 2048, 1916, 128)
+    if which in ("decode-13b", "all"):
+        decode_case(ctx, "decode-13b", "13b", lva.LV_Q4_0, 2, 512, 32, 256)
+    if which in ("prefill-13b", "all"):
+        prefill_case(ctx)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,117 @@
+"""Batched prompt path: the matrix-core GEMM (lv_kernel_gemm) against the oracle's fp32 GEMV at the same bound the
+one-token GEMV is held to, and whole prompts evaluated as one batch against the oracle and against token-by-token
+evaluation (reference: the *_batch shader variants and llava_session.cpp:197-229 with several pending tokens)."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def _abs_dot_bound(orc, blocks, ftype, rows, cols, x):
+    w = np.abs(orc.dequant(blocks, ftype, rows * cols).reshape(rows, cols).astype(np.float64))
+    return (w @ np.abs(x.astype(np.float64)).T).T      # [batch][rows]
+
+
+@pytest.mark.parametrize("ftype_name", ["q4_0", "q8_0"])
+@pytest.mark.parametrize("rows,cols,batch,accumulate", [
+    (128, 64, 128, False),       # exactly one tile, one K step
+    (256, 4096, 130, False),     # a second, almost empty token tile
+    (704, 256, 17, True),        # rows not a multiple of the tile, residual add
+    (96, 1376, 200, False),      # K = 43 blocks: a half K step at the end, fewer rows than a tile
+    (4096, 4096, 512, True),     # the 7B attention shape at the batch of BASELINE's prompt case
+])
+def test_gemm_matches_oracle(lva, orc, ctx, ftype_name, rows, cols, batch, accumulate):
+    ftype = lva.LV_Q4_0 if ftype_name == "q4_0" else lva.LV_Q8_0
+    blocks = lva.synth_quant(ftype, rows, cols, seed=61)
+    x = lva.synth_normal(batch, cols, seed=62)
+    x[0, :4] = [0.0, 1.0, -1000.25, 1e-7]              # zero, one, a large and a tiny activation
+    prev = lva.synth_normal(batch, rows, seed=63)
+    m = ctx.matrix(blocks, ftype, rows, cols)
+    dx, dout = ctx.to_device(x), ctx.to_device(prev)
+    lva.check(ctx.lib.lv_kernel_gemm(ctx.h, dout, m, dx, batch, int(accumulate)))
+    got = ctx.to_host(dout, (batch, rows), np.float32)
+    want = orc.gemv(blocks, ftype, rows, cols, x, out=prev if accumulate else None, accumulate=accumulate)
+    bound = 1e-5 * _abs_dot_bound(orc, blocks, ftype, rows, cols, x) + 1e-7
+    ratio = float(np.max(np.abs(got.astype(np.float64) - want) / bound))
+    assert ratio <= 1.0, ratio
+    # the one-token kernel on the same rows: each is within the bound of the oracle, so within 1.5 bounds of each other
+    # (the fp16 halves carry 22 bits of an activation, fp32 carries 24)
+    dout2 = ctx.to_device(prev)
+    nb = min(batch, 64)
+    lva.check(ctx.lib.lv_kernel_gemv(ctx.h, dout2, m, dx, nb, int(accumulate)))
+    one = ctx.to_host(dout2, (batch, rows), np.float32)[:nb]
+    assert float(np.max(np.abs(one.astype(np.float64) - got[:nb]) / bound[:nb])) <= 1.5
+    for p in (dx, dout, dout2):
+        ctx.free(p)
+    ctx.matrix_free(m)
+
+
+def test_gemm_special_inputs(lva, orc, ctx):
+    """all codes 8 -> exact zeros; one-hot activations -> exact dequantised columns"""
+    rows, cols, batch = 128, 128, 128
+    blocks = lva.synth_quant(lva.LV_Q4_0, rows, cols, seed=64)
+    m = ctx.matrix(blocks, lva.LV_Q4_0, rows, cols)
+    x = np.zeros((batch, cols), dtype=np.float32)
+    x[np.arange(batch), np.arange(batch)] = 1.0
+    dx, dout = ctx.to_device(x), ctx.alloc(batch * rows * 4)
+    lva.check(ctx.lib.lv_kernel_gemm(ctx.h, dout, m, dx, batch, 0))
+    got = ctx.to_host(dout, (batch, rows), np.float32)
+    w = orc.dequant(blocks, lva.LV_Q4_0, rows * cols).reshape(rows, cols)
+    assert np.array_equal(got, w.T)                      # hi + lo halves restore every weight exactly
+    for p in (dx, dout):
+        ctx.free(p)
+    ctx.matrix_free(m)
+
+
+@pytest.mark.parametrize("name,n_prompt", [("tiny_q4", 40), ("tiny_q8", 130), ("small_q4", 77)])
+def test_prompt_as_one_batch_matches_oracle(lva, orc, ctx, tiny_models, name, n_prompt):
+    path = tiny_models[name]
+    om = orc.Model(path)
+    vocab, layers = om.hp["vocab"], om.hp["layers"]
+    osess = orc.Session(om, 256)
+    model = lva.Model(ctx, path)
+    a, b = lva.Session(model, 256), lva.Session(model, 256)
+    prompt = lva.synth_tokens(n_prompt, 3, vocab, seed=9)
+    want = osess.eval(prompt)
+    a.begin(prompt, 0)                                   # one step: the matrix-core path
+    for i, t in enumerate(prompt):                       # token by token: the one-token kernels
+        b.begin([int(t)], i)
+        b.wait()
+    la, lb = a.logits(), b.logits()
+    tol = 1e-2 + 1e-3 * np.abs(want)
+    assert np.all(np.abs(la - want) <= tol) and np.all(np.abs(lb - want) <= tol)
+    assert float(np.max(np.abs(la - lb))) <= 1e-4 * max(1.0, float(np.max(np.abs(lb))))
+    for layer in range(layers):
+        for which in (0, 1):
+            ra = a.kv(layer, which, n_prompt).view(np.float16).astype(np.float32)
+            rb = b.kv(layer, which, n_prompt).view(np.float16).astype(np.float32)
+            # different summation orders flip the last fp16 bit of some entries, never more than that
+            assert np.mean(ra != rb) < 0.5 and np.max(np.abs(ra - rb)) <= 2e-3 * float(np.max(np.abs(rb)))
+    # greedy continuation from the batched cache
+    pos, logits = n_prompt, want
+    for step in range(16):
+        tok = orc.greedy(logits)
+        assert a.argmax() == tok, step
+        logits = osess.eval(np.array([tok], dtype=np.uint32))
+        a.begin([tok], pos)
+        pos += 1
+    a.close(); b.close(); model.close(); osess.close(); om.close()
+
+
+def test_second_batch_appends_behind_the_first(lva, orc, ctx, tiny_models):
+    """two batched steps in a row (prompt, then a long addition): rows of the second see the cache of the first"""
+    path = tiny_models["tiny_q4"]
+    om = orc.Model(path)
+    osess = orc.Session(om, 256)
+    model = lva.Model(ctx, path)
+    s = lva.Session(model, 256)
+    toks = lva.synth_tokens(100, 3, om.hp["vocab"], seed=10)
+    osess.eval(toks[:60])
+    want = osess.eval(toks[60:])
+    s.begin(toks[:60], 0)
+    s.wait()
+    s.begin(toks[60:], 60)
+    got = s.logits()
+    assert np.all(np.abs(got - want) <= 1e-2 + 1e-3 * np.abs(want))
+    assert s.argmax() == orc.greedy(want)
+    s.close(); model.close(); osess.close(); om.close()
