@@ -20,6 +20,7 @@
 #include "lv_kernels.h"
 #include "lv_mega.h"
 #include "lv_gemm.h"
+#include "lv_attn_batch.h"
 
 using namespace lv;
 
@@ -123,11 +124,9 @@ struct lv_session {
     bool use_graph = true;
     int path = LV_PATH_AUTO;
     // workspace of the batched prompt path, allocated at first use: activations for pf_cap tokens
-    uint32_t pf_cap = 0, pf_backlog = 0;
+    uint32_t pf_cap = 0;
     float *pf_x = nullptr, *pf_xn = nullptr, *pf_q = nullptr, *pf_k = nullptr, *pf_v = nullptr, *pf_vo = nullptr, *pf_g1 = nullptr, *pf_g2 = nullptr;
     uint16_t *pf_xh = nullptr, *pf_xl = nullptr;
-    float *pf_part = nullptr;
-    uint32_t *pf_counters = nullptr;
     float *xchg[2] = {nullptr, nullptr};  // hand-over buffer sets of the persistent kernel
     uint32_t xchg_turn = 0;
     uint32_t *status_host = nullptr;      // pinned, written by the persistent kernel when a poll expires
@@ -456,6 +455,23 @@ static int launch_attention(hipStream_t st, float *out, const uint16_t *kc, cons
     case 32: attention_kernel<32><<<grid, dim3(256), lds, st>>>(a); break;
     case 64: attention_kernel<64><<<grid, dim3(256), lds, st>>>(a); break;
     case 128: attention_kernel<128><<<grid, dim3(256), lds, st>>>(a); break;
+    default: return fail(LV_ERR_ARG, "attention: head size %u (32, 64 and 128 are built)", rot);
+    }
+    HIP_TRY(hipGetLastError());
+    return LV_OK;
+}
+
+static int launch_attention_batch(hipStream_t st, float *out, const uint16_t *kc, const uint16_t *vc, const float *q, const float2 *trig,
+                                  const uint32_t *pos_ptr, uint32_t pos_add, uint32_t n, uint32_t backlog, uint32_t heads, uint32_t rot)
+{
+    AttnBatchArgs a{};
+    a.out = out; a.kcache = kc; a.vcache = vc; a.q = q; a.trig = trig; a.pos_ptr = pos_ptr; a.pos_add = pos_add;
+    a.n = n; a.heads = heads; a.backlog = backlog;
+    const dim3 grid(heads, (n + kAttnBatchQ - 1) / kAttnBatchQ);
+    switch (rot) {
+    case 32: attention_batch_kernel<32><<<grid, dim3(256), 0, st>>>(a); break;
+    case 64: attention_batch_kernel<64><<<grid, dim3(256), 0, st>>>(a); break;
+    case 128: attention_batch_kernel<128><<<grid, dim3(256), 0, st>>>(a); break;
     default: return fail(LV_ERR_ARG, "attention: head size %u (32, 64 and 128 are built)", rot);
     }
     HIP_TRY(hipGetLastError());
@@ -860,7 +876,7 @@ extern "C" int lv_session_destroy(lv_session *s)
     drop_graph(s);
     void *dev[] = {s->kv, s->trig, s->x, s->xn, s->q, s->k, s->v, s->vo, s->ff, s->logits, s->attn_part, s->attn_counters,
                    s->cfg, s->argmax_dev, s->trace_buf, s->pf_x, s->pf_xn, s->pf_q, s->pf_k, s->pf_v, s->pf_vo, s->pf_g1, s->pf_g2,
-                   s->pf_xh, s->pf_xl, s->pf_part, s->pf_counters};
+                   s->pf_xh, s->pf_xl};
     for (void *p : dev) (void)hipFree(p);
     (void)hipFree(s->xchg[0]);
     (void)hipFree(s->xchg[1]);
@@ -1110,18 +1126,6 @@ static int prefill_reserve(lv_session *s, uint32_t n)
             if (e != hipSuccess) return fail(e == hipErrorOutOfMemory ? LV_ERR_OOM : LV_ERR_HIP, "prompt workspace: %s", hipGetErrorString(e));
         }
         s->pf_cap = cap;
-        s->pf_backlog = 0;
-    }
-    if (s->pf_backlog != s->backlog) {
-        HIP_TRY(hipStreamSynchronize(s->stream));
-        (void)hipFree(s->pf_part);
-        (void)hipFree(s->pf_counters);
-        s->pf_part = nullptr; s->pf_counters = nullptr; s->pf_backlog = 0;
-        const uint32_t splits = (s->backlog + kAttnChunk - 1) / kAttnChunk;
-        HIP_TRY(hipMalloc(reinterpret_cast<void **>(&s->pf_part), attn_part_floats(s->pf_cap, hp.heads, splits, hp.rot) * sizeof(float)));
-        HIP_TRY(hipMalloc(reinterpret_cast<void **>(&s->pf_counters), (size_t)s->pf_cap * hp.heads * 4));
-        LV_TRY(zero_async(s->pf_counters, (size_t)s->pf_cap * hp.heads * 4, s->stream));
-        s->pf_backlog = s->backlog;
     }
     return LV_OK;
 }
@@ -1157,8 +1161,8 @@ static int record_prefill(lv_session *s, uint32_t idx0, uint32_t n, bool with_he
         kv_append_kernel<<<kv_grid, dim3(256), 0, st>>>(kv_ptr(s, li, 0), s->pf_k, pos_ptr, idx0, D, s->backlog);
         kv_append_kernel<<<kv_grid, dim3(256), 0, st>>>(kv_ptr(s, li, 1), s->pf_v, pos_ptr, idx0, D, s->backlog);
         HIP_TRY(hipGetLastError());
-        LV_TRY(launch_attention(st, s->pf_vo, kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->pf_q, s->trig, s->pf_part, s->pf_counters, pos_ptr, idx0,
-                                s->backlog, hp.heads, hp.rot, n));
+        LV_TRY(launch_attention_batch(st, s->pf_vo, kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->pf_q, s->trig, pos_ptr, idx0, n, s->backlog,
+                                      hp.heads, hp.rot));
         LV_TRY(launch_gemm(st, s->pf_x, D, lw.wo, s->pf_vo, n, s->pf_xh, s->pf_xl, true));
         normalize_kernel<<<dim3(n), dim3(256), 0, st>>>(s->pf_xn, s->pf_x, lw.ffn_norm, D);
         HIP_TRY(hipGetLastError());
