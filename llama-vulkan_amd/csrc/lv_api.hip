@@ -94,12 +94,28 @@ struct lv_model {
     const float *tok_f32 = nullptr;
     lv_matrix tok_quant;
     // persistent-kernel form of the weights (null when the model's shape has no compiled MegaShape)
-    int mega_kind = 0;              // 0 none, 1 = 7B class (4096/11008/32 heads)
+    int mega_kind = 0;              // 0 none, else a compiled shape class of the persistent kernel (mega_dispatch)
     uint8_t *mega_stream = nullptr;
     float *mega_norms = nullptr;    // [layers][2][D] + final norm [D]
 };
 
-using Mega7B = MegaShape<4096, 11008, 32, 12>;
+// Shape classes the persistent kernel is compiled for: LLaMA-7B and LLaMA-13B layer shapes, q4_0 and q8_0.
+using Mega7Bq4 = MegaShape<4096, 11008, 32, 12, 4>;
+using Mega7Bq8 = MegaShape<4096, 11008, 32, 12, 8>;
+using Mega13Bq4 = MegaShape<5120, 13824, 40, 12, 4>;
+using Mega13Bq8 = MegaShape<5120, 13824, 40, 12, 8>;
+
+template <class Fn>
+static int mega_dispatch(int kind, Fn &&fn)
+{
+    switch (kind) {
+    case 1: return fn(Mega7Bq4{});
+    case 2: return fn(Mega7Bq8{});
+    case 3: return fn(Mega13Bq4{});
+    case 4: return fn(Mega13Bq8{});
+    default: return fail(LV_ERR_STATE, "no persistent kernel for this model");
+    }
+}
 
 constexpr uint32_t kAttnChunk = 64;   // cache positions per attention workgroup
 constexpr uint32_t kMaxStepTokens = 4096;
@@ -665,7 +681,7 @@ static int build_mega_stream(lv_model *m)
 {
     lv_ctx *c = m->ctx;
     const uint32_t L = m->hp.layers, D = m->hp.dim;
-    const size_t total = (size_t)L * S::LAYER_BYTES + S::HEAD_BYTES + kMegaTile;  // + the all-zero dummy tile
+    const size_t total = (size_t)L * S::LAYER_BYTES + S::HEAD_BYTES + S::TILE;  // + the all-zero dummy tile
     hipError_t e = hipMalloc(reinterpret_cast<void **>(&m->mega_stream), total);
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&m->mega_norms), ((size_t)L * 2 + 1) * D * 4);
     if (e != hipSuccess)
@@ -680,7 +696,7 @@ static int build_mega_stream(lv_model *m)
         return LV_OK;
     };
     const MatView none{};
-    LV_TRY(zero_async(m->mega_stream + (size_t)L * S::LAYER_BYTES + S::HEAD_BYTES, kMegaTile, c->stream));
+    LV_TRY(zero_async(m->mega_stream + (size_t)L * S::LAYER_BYTES + S::HEAD_BYTES, S::TILE, c->stream));
     for (uint32_t i = 0; i < L; i++) {
         const LayerWeights &lw = m->layers[i];
         uint8_t *base = m->mega_stream + (size_t)i * S::LAYER_BYTES;
@@ -691,7 +707,7 @@ static int build_mega_stream(lv_model *m)
         HIP_TRY(hipMemcpyAsync(m->mega_norms + (size_t)i * 2 * D, lw.attn_norm, (size_t)D * 4, hipMemcpyDeviceToDevice, c->stream));
         HIP_TRY(hipMemcpyAsync(m->mega_norms + ((size_t)i * 2 + 1) * D, lw.ffn_norm, (size_t)D * 4, hipMemcpyDeviceToDevice, c->stream));
     }
-    LV_TRY(pack(m->mega_stream + (size_t)L * S::LAYER_BYTES, 4, kMegaHeadSlots, m->output.view, none, none));
+    LV_TRY(pack(m->mega_stream + (size_t)L * S::LAYER_BYTES, 4, S::HEAD, m->output.view, none, none));
     HIP_TRY(hipMemcpyAsync(m->mega_norms + (size_t)L * 2 * D, m->norm, (size_t)D * 4, hipMemcpyDeviceToDevice, c->stream));
     HIP_TRY(hipStreamSynchronize(c->stream));
     return LV_OK;
@@ -700,14 +716,23 @@ static int build_mega_stream(lv_model *m)
 static int build_mega(lv_model *m)
 {
     const lv_hparams &hp = m->hp;
-    bool all_q4 = m->output.ftype == LV_Q4_0 && m->tok_ftype == LV_F32;
+    const uint32_t ft = m->output.ftype;
+    bool uniform = (ft == LV_Q4_0 || ft == LV_Q8_0) && m->tok_ftype == LV_F32;
     for (const LayerWeights &lw : m->layers)
-        for (const lv_matrix *x : {&lw.wq, &lw.wk, &lw.wv, &lw.wo, &lw.w1, &lw.w2, &lw.w3}) all_q4 = all_q4 && x->ftype == LV_Q4_0;
-    if (!all_q4 || (int)m->ctx->props.multiProcessorCount < kMegaWGs) return LV_OK;
-    if (hp.dim == Mega7B::D && hp.ff == Mega7B::F && hp.heads == Mega7B::H &&
-        (hp.vocab + kMegaWGs - 1) / kMegaWGs <= (uint32_t)(kMegaHeadSlots * Mega7B::NRD)) {
-        LV_TRY(build_mega_stream<Mega7B>(m));
-        m->mega_kind = 1;
+        for (const lv_matrix *x : {&lw.wq, &lw.wk, &lw.wv, &lw.wo, &lw.w1, &lw.w2, &lw.w3}) uniform = uniform && x->ftype == ft;
+    if (!uniform || (int)m->ctx->props.multiProcessorCount < kMegaWGs) return LV_OK;
+    for (int kind = 1; kind <= 4; kind++) {
+        bool fits = false;
+        (void)mega_dispatch(kind, [&](auto shape) -> int {
+            using S = decltype(shape);
+            fits = hp.dim == (uint32_t)S::D && hp.ff == (uint32_t)S::F && hp.heads == (uint32_t)S::H && ft == (S::QT == 4 ? LV_Q4_0 : LV_Q8_0) &&
+                   (hp.vocab + kMegaWGs - 1) / kMegaWGs <= (uint32_t)(S::HEAD * S::NRD);
+            return LV_OK;
+        });
+        if (!fits) continue;
+        LV_TRY(mega_dispatch(kind, [&](auto shape) { return build_mega_stream<decltype(shape)>(m); }));
+        m->mega_kind = kind;
+        break;
     }
     return LV_OK;
 }
@@ -907,8 +932,12 @@ static int session_alloc(lv_session *s)
     HIP_TRY(hipMalloc(reinterpret_cast<void **>(&s->argmax_dev), 4));
     HIP_TRY(hipHostMalloc(reinterpret_cast<void **>(&s->cfg_host), (1 + kMaxStepTokens) * 4, hipHostMallocDefault));
     HIP_TRY(hipHostMalloc(reinterpret_cast<void **>(&s->argmax_host), 4, hipHostMallocDefault));
-    if (s->model->mega_kind == 1) {
-        const size_t bytes = (size_t)hp.layers * Mega7B::XCHG_LAYER * 4;
+    if (s->model->mega_kind) {
+        size_t bytes = 0;
+        LV_TRY(mega_dispatch(s->model->mega_kind, [&](auto shape) -> int {
+            bytes = (size_t)hp.layers * decltype(shape)::XCHG_LAYER * 4;
+            return LV_OK;
+        }));
         for (int i = 0; i < 2; i++) {
             HIP_TRY(hipMalloc(reinterpret_cast<void **>(&s->xchg[i]), bytes));
             HIP_TRY(hipMemsetAsync(s->xchg[i], 0xff, bytes, s->stream));
@@ -1036,9 +1065,12 @@ static int launch_mega(lv_session *s, uint32_t pos, uint32_t token)
     a.layers = m->hp.layers; a.vocab = m->hp.vocab; a.backlog = s->backlog; a.pos = pos; a.token = token;
     s->xchg_turn++;
     void *params[] = {&a};
-    HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<const void *>(&mega_decode_kernel<Mega7B>), dim3(kMegaWGs),
-                                       dim3(Mega7B::NW * 64), params, 0, s->stream));
-    return LV_OK;
+    return mega_dispatch(m->mega_kind, [&](auto shape) -> int {
+        using S = decltype(shape);
+        HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<const void *>(&mega_decode_kernel<S>), dim3(kMegaWGs), dim3(S::NW * 64), params, 0,
+                                           s->stream));
+        return LV_OK;
+    });
 }
 
 // -----------------------------------------------------------------------------------------------------------

@@ -3,7 +3,7 @@
 // Why: at batch 1 a layer is five tiny dependent GEMVs (1-6 us of HBM time each).  Launched one by one
 // they spend more time draining, launching and refilling the memory pipeline than streaming weights.
 // Here one workgroup per CU stays resident for the whole token; every wavefront walks its own contiguous
-// weight stream with a kMegaDepth-deep (4) register queue of 128-bit loads that keeps running across the phase
+// weight stream with a register queue (4 q4_0 tiles or 2 q8_0 tiles deep) of 128-bit loads that keeps running across the phase
 // boundaries, so HBM stays busy while the workgroups exchange the small activation vectors.
 //
 // Phases of a layer (llava_layer.cpp:53-73), each separated by a data hand-over through HBM/L2:
@@ -22,8 +22,8 @@
 // Every poll loop is bounded: on expiry the kernel raises *status and carries on to its end.
 //
 // Weight stream: for each (layer, phase, workgroup, wave) the tiles that wave will consume, in order.
-// A tile is one matrix row restricted to the wave's 64-block column slab: 64 x 16 B codes + 64 x fp16
-// scales (1152 B).  Lane l of the wave always owns block column 64*slab + l, so the 32 activations of
+// A tile is one matrix row restricted to the wave's 64-block column slab: 64 x 16 B (q4_0) or 64 x 32 B
+// (q8_0) of codes + 64 x fp16 scales (1152 B / 2176 B).  Lane l of the wave always owns block column 64*slab + l, so the 32 activations of
 // that column sit in registers for the whole phase.
 #pragma once
 
@@ -33,9 +33,7 @@ namespace lv {
 
 constexpr uint32_t kNotReady = 0xFFFFFFFFu;
 constexpr int kMegaWGs = 256;
-constexpr int kMegaDepth = 4;           // tiles in flight per wave
-constexpr int kMegaTile = 1152;         // bytes per q4_0 tile
-constexpr int kMegaHeadSlots = 24;      // head tiles per wave (static upper bound)
+constexpr int kMegaVocabRows = 125;     // output-matrix rows per workgroup the head phase is laid out for (32000 / 256)
 constexpr uint32_t kSpinLimit = 1u << 20;
 
 __device__ __forceinline__ uint32_t ld_dev(const uint32_t *p)
@@ -63,16 +61,21 @@ constexpr int cdiv(int a, int b) { return (a + b - 1) / b; }
 constexpr int round_up(int a, int b) { return cdiv(a, b) * b; }
 
 // Static shape of one model class.  NW = wavefronts per workgroup.
-template <int D_, int F_, int H_, int NW_>
+template <int D_, int F_, int H_, int NW_, int QT_>
 struct MegaShape {
     static constexpr int D = D_, F = F_, H = H_, NW = NW_, R = 128;
+    static constexpr int QT = QT_;                               // 4: q4_0, 8: q8_0
+    static constexpr int CODE = QT == 4 ? 16 : 32;               // bytes of codes per block
+    static constexpr int TILE = 64 * CODE + 128;                 // bytes per tile: 64 blocks of codes, 64 fp16 scales
+    static constexpr int DEPTH = QT == 4 ? 4 : 2;                // tiles in flight per wave (about 4.5 KB either way)
     static constexpr int NBD = D / 32, NBF = F / 32;            // blocks per row
     static constexpr int NSD = cdiv(NBD, 64), NSF = cdiv(NBF, 64);  // column slabs
     static constexpr int NRD = NW / NSD, NRF = NW / NSF;        // row sets (waves sharing a slab split the rows)
     static constexpr int ROWS_A = 3 * D / kMegaWGs, ROWS_C = D / kMegaWGs, ROWS_D = 2 * F / kMegaWGs, ROWS_E = D / kMegaWGs;
     static constexpr int TA = cdiv(ROWS_A, NRD), TC = cdiv(ROWS_C, NRD), TD = cdiv(ROWS_D, NRD), TE = cdiv(ROWS_E, NRF);
     static constexpr int SEQ_A = 0, SEQ_C = TA, SEQ_D = TA + TC, SEQ_E = TA + TC + TD;
-    static constexpr int PER_LAYER = round_up(TA + TC + TD + TE, kMegaDepth);
+    static constexpr int PER_LAYER = round_up(TA + TC + TD + TE, DEPTH);
+    static constexpr int HEAD = round_up(cdiv(kMegaVocabRows, NRD), 4);   // head tiles per wave (static upper bound)
     static constexpr int CPH = kMegaWGs / H;                    // position chunks per head
     static constexpr int PART = R + 4;                          // floats per partial (128 numerators, denominator, pad)
     // floats of one layer's hand-over buffers
@@ -81,10 +84,10 @@ struct MegaShape {
     static_assert((3 * D) % kMegaWGs == 0 && (2 * F) % kMegaWGs == 0 && D % kMegaWGs == 0, "rows must split over 256 workgroups");
     static_assert(H * R == D && CPH >= 1 && NRD >= 1 && NRF >= 1, "shape");
     // bytes of the weight stream of one layer
-    static constexpr size_t PHASE_A_BYTES = (size_t)kMegaWGs * NW * TA * kMegaTile, PHASE_C_BYTES = (size_t)kMegaWGs * NW * TC * kMegaTile,
-                            PHASE_D_BYTES = (size_t)kMegaWGs * NW * TD * kMegaTile, PHASE_E_BYTES = (size_t)kMegaWGs * NW * TE * kMegaTile;
+    static constexpr size_t PHASE_A_BYTES = (size_t)kMegaWGs * NW * TA * TILE, PHASE_C_BYTES = (size_t)kMegaWGs * NW * TC * TILE,
+                            PHASE_D_BYTES = (size_t)kMegaWGs * NW * TD * TILE, PHASE_E_BYTES = (size_t)kMegaWGs * NW * TE * TILE;
     static constexpr size_t LAYER_BYTES = PHASE_A_BYTES + PHASE_C_BYTES + PHASE_D_BYTES + PHASE_E_BYTES;
-    static constexpr size_t HEAD_BYTES = (size_t)kMegaWGs * NW * kMegaHeadSlots * kMegaTile;
+    static constexpr size_t HEAD_BYTES = (size_t)kMegaWGs * NW * HEAD * TILE;
 };
 
 struct MegaArgs {
@@ -119,9 +122,25 @@ struct MegaArgs {
 #endif
 
 struct MegaTile {
-    uint4 c;
+    uint4 c, c2;   // c2: second half of the codes of a q8_0 block (unused for q4_0)
     uint16_t d;
 };
+
+template <class S>
+__device__ __forceinline__ void load_tile(MegaTile &t, const uint8_t *p, int lane)
+{
+    t.c = *reinterpret_cast<const uint4 *>(p + lane * S::CODE);
+    if constexpr (S::QT == 8) t.c2 = *reinterpret_cast<const uint4 *>(p + lane * S::CODE + 16);
+    t.d = *reinterpret_cast<const uint16_t *>(p + 64 * S::CODE + lane * 2);
+}
+
+// one block column of one row: sum over 32 weights of w * x, from the raw codes
+template <class S>
+__device__ __forceinline__ float tile_dot(const MegaTile &t, const float (&xr)[32], float xsum)
+{
+    if constexpr (S::QT == 4) return (q4_block_dot(t.c, xr) - 8.f * xsum) * half_bits_to_float(t.d);
+    else return (q8_block_dot(t.c, t.c2, xr) - 128.f * xsum) * half_bits_to_float(t.d);
+}
 
 // ---- polling helpers ----------------------------------------------------------------------------------------
 // N values strided by `stride` elements starting at p; spins until none of them is the not-ready pattern.
@@ -199,20 +218,19 @@ struct MegaWave {
         else if (k < S::SEQ_E) { i = k - S::SEQ_D; tiles = S::TD; rows = S::ROWS_D; act = actD; lane_ok = laneD; rset = rD; off = S::PHASE_A_BYTES + S::PHASE_C_BYTES; }
         else if (k < S::SEQ_E + S::TE) { i = k - S::SEQ_E; tiles = S::TE; rows = S::ROWS_E; act = actF; lane_ok = laneF; rset = rF; off = S::PHASE_A_BYTES + S::PHASE_C_BYTES + S::PHASE_D_BYTES; }
         else real = false;                                   // padding slot of the layer sequence
-        const bool head_slot = wrapped && k < kMegaHeadSlots;  // static
+        const bool head_slot = wrapped && k < S::HEAD;  // static
         if (!real && !head_slot) return;                     // static: this slot never loads
         const uint8_t *p = dummy;
         if (real) {
             const bool ok = !into_head && act && lane_ok && rset * tiles + i < rows;
-            const uint8_t *q = wstream + (size_t)layer * S::LAYER_BYTES + off + ((size_t)(b * S::NW + w) * tiles + i) * kMegaTile;
+            const uint8_t *q = wstream + (size_t)layer * S::LAYER_BYTES + off + ((size_t)(b * S::NW + w) * tiles + i) * S::TILE;
             p = ok ? q : p;
         }
         if (head_slot) {
             const uint8_t *q = head_tile(k);
             p = (into_head && q) ? q : p;
         }
-        t.c = *reinterpret_cast<const uint4 *>(p + lane * 16);
-        t.d = *reinterpret_cast<const uint16_t *>(p + 1024 + lane * 2);
+        load_tile<S>(t, p, lane);
     }
 
     // address of head tile k of this wave, or null when the wave/lane/row has none
@@ -221,24 +239,23 @@ struct MegaWave {
         const int rows = (int)vocab_rows, per_set = (rows + S::NRD - 1) / S::NRD;
         const int j = rD * per_set + k;
         const bool ok = actD && laneD && k < per_set && j < rows && (uint32_t)(b * rows + j) < vocab;
-        return ok ? wstream + (size_t)layers * S::LAYER_BYTES + ((size_t)(b * S::NW + w) * kMegaHeadSlots + k) * kMegaTile : nullptr;
+        return ok ? wstream + (size_t)layers * S::LAYER_BYTES + ((size_t)(b * S::NW + w) * S::HEAD + k) * S::TILE : nullptr;
     }
 
     // head phase: slot k of the head sequence (static k)
     __device__ __forceinline__ void fetch_head(MegaTile &t, int k) const
     {
-        if (k >= kMegaHeadSlots) return;
+        if (k >= S::HEAD) return;
         const uint8_t *q = head_tile(k);
         const uint8_t *p = q ? q : dummy;
-        t.c = *reinterpret_cast<const uint4 *>(p + lane * 16);
-        t.d = *reinterpret_cast<const uint16_t *>(p + 1024 + lane * 2);
+        load_tile<S>(t, p, lane);
     }
 };
 
 // One GEMV phase of one wave: consumes NT queue slots starting at sequence index SEQ0, refills each consumed
-// slot with the tile kMegaDepth further down the sequence, leaves per-row sums in red[row*NS + slab].
+// slot with the tile S::DEPTH further down the sequence, leaves per-row sums in red[row*NS + slab].
 template <class S, int SEQ0, int NT, int NS>
-__device__ __forceinline__ void gemv_phase(MegaTile (&q)[kMegaDepth], const MegaWave<S> &mw, uint32_t layer, const float (&xr)[32],
+__device__ __forceinline__ void gemv_phase(MegaTile (&q)[S::DEPTH], const MegaWave<S> &mw, uint32_t layer, const float (&xr)[32],
                                            float xsum, int slab, int rset, bool active, int rows, float *red)
 {
     constexpr int NT4 = round_up(NT, 4);
@@ -246,10 +263,10 @@ __device__ __forceinline__ void gemv_phase(MegaTile (&q)[kMegaDepth], const Mega
 #pragma unroll
     for (int i = 0; i < NT4; i++) {
         if (i < NT) {
-            const int slot = (SEQ0 + i) % kMegaDepth;
+            const int slot = (SEQ0 + i) % S::DEPTH;
             const MegaTile t = q[slot];
-            p[i & 3] = (q4_block_dot(t.c, xr) - 8.f * xsum) * half_bits_to_float(t.d);
-            mw.fetch(q[slot], SEQ0 + i + kMegaDepth, layer);
+            p[i & 3] = tile_dot<S>(t, xr, xsum);
+            mw.fetch(q[slot], SEQ0 + i + S::DEPTH, layer);
         } else {
             p[i & 3] = 0.f;
         }
@@ -275,7 +292,7 @@ __device__ __forceinline__ float red_row(const float *red, int row)
 template <class S>
 struct MegaLds {
     static constexpr int XS = S::F > S::D ? S::F : S::D;
-    static constexpr int RED_ROWS = S::ROWS_D > kMegaHeadSlots * S::NRD ? S::ROWS_D : kMegaHeadSlots * S::NRD;
+    static constexpr int RED_ROWS = S::ROWS_D > S::HEAD * S::NRD ? S::ROWS_D : S::HEAD * S::NRD;
     static constexpr int RED_COLS = S::NSF > S::NSD ? S::NSF : S::NSD;
     float xs[XS];                    // the phase's input vector (during attention: exp(score) of the chunk)
     float red[RED_ROWS * RED_COLS];  // per-row partial sums, one column per slab
@@ -353,9 +370,9 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
     uint32_t *status = a.status;
 
     // ---- start the weight stream ------------------------------------------------------------------------------
-    MegaTile q[kMegaDepth];
+    MegaTile q[S::DEPTH];
 #pragma unroll
-    for (int k = 0; k < kMegaDepth; k++) mw.fetch(q[k], k, 0);
+    for (int k = 0; k < S::DEPTH; k++) mw.fetch(q[k], k, 0);
 
     // ---- re-arm the other buffer set for the next token ---------------------------------------------------------
 #ifndef LV_MEGA_NOWAIT   // (experiment builds leave stale, "ready" data in place to time the kernel without hand-over waits)
@@ -585,9 +602,9 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
         MEGA_STAMP(10);
         load_slab(xr, xsum, xs, mw.sF * 64 + lane, mw.laneF);
         gemv_phase<S, S::SEQ_E, S::TE, S::NSF>(q, mw, layer, xr, xsum, mw.sF, mw.rF, mw.actF, S::ROWS_E, red);
-        // padding slots of the layer's sequence carry no tile, but the slot kMegaDepth ahead of them does
+        // padding slots of the layer's sequence carry no tile, but the slot S::DEPTH ahead of them does
 #pragma unroll
-        for (int k = S::SEQ_E + S::TE; k < S::PER_LAYER; k++) mw.fetch(q[k % kMegaDepth], k + kMegaDepth, layer);
+        for (int k = S::SEQ_E + S::TE; k < S::PER_LAYER; k++) mw.fetch(q[k % S::DEPTH], k + S::DEPTH, layer);
         lds_barrier();
         if (st < S::ROWS_E) {
             const float v = xown[st] + red_row<S::NSF>(red, st);
@@ -606,11 +623,11 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
         // the head's slots are numbered from 0; tiles beyond per_set read the dummy tile
         float p[4];
 #pragma unroll
-        for (int i = 0; i < kMegaHeadSlots; i++) {
-            const int slot = i % kMegaDepth;
+        for (int i = 0; i < S::HEAD; i++) {
+            const int slot = i % S::DEPTH;
             const MegaTile t = q[slot];
-            p[i & 3] = (q4_block_dot(t.c, xr) - 8.f * xsum) * half_bits_to_float(t.d);
-            mw.fetch_head(q[slot], i + kMegaDepth);
+            p[i & 3] = tile_dot<S>(t, xr, xsum);
+            mw.fetch_head(q[slot], i + S::DEPTH);
             if ((i & 3) == 3) {
                 const float s = quad_partials_sum(p[0], p[1], p[2], p[3]);
                 const int ii = (i - 3) + quad_partial_of_lane(lane);
@@ -643,7 +660,7 @@ struct MegaPackSrc {
 template <class S>
 __global__ void mega_pack_kernel(uint8_t *dst /* start of the phase region */, MegaPackSrc src, int phase, uint32_t vocab)
 {
-    const int tiles = phase == 0 ? S::TA : phase == 1 ? S::TC : phase == 2 ? S::TD : phase == 3 ? S::TE : kMegaHeadSlots;
+    const int tiles = phase == 0 ? S::TA : phase == 1 ? S::TC : phase == 2 ? S::TD : phase == 3 ? S::TE : S::HEAD;
     const int ns = phase == 3 ? S::NSF : S::NSD, nr = phase == 3 ? S::NRF : S::NRD, nb = phase == 3 ? S::NBF : S::NBD;
     const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t total = (size_t)kMegaWGs * S::NW * tiles * 64;
@@ -654,8 +671,8 @@ __global__ void mega_pack_kernel(uint8_t *dst /* start of the phase region */, M
     const int w = (tile / tiles) % S::NW;
     const int b = tile / tiles / S::NW;
     const int slab = w % ns, rset = w / ns;
-    uint8_t *out = dst + tile * kMegaTile;
-    uint4 codes = make_uint4(0, 0, 0, 0);
+    uint8_t *out = dst + tile * S::TILE;
+    uint4 codes = make_uint4(0, 0, 0, 0), codes2 = codes;
     uint16_t scale = 0;
     const int blk = slab * 64 + lane;
     bool ok = rset < nr && blk < nb;
@@ -680,11 +697,17 @@ __global__ void mega_pack_kernel(uint8_t *dst /* start of the phase region */, M
     }
     if (ok) {
         const size_t sb = (size_t)row * nb + blk;
-        codes = mv->codes[sb];
+        if constexpr (S::QT == 4) {
+            codes = mv->codes[sb];
+        } else {
+            codes = mv->codes[2 * sb];
+            codes2 = mv->codes[2 * sb + 1];
+        }
         scale = mv->scales[sb];
     }
-    *reinterpret_cast<uint4 *>(out + lane * 16) = codes;
-    *reinterpret_cast<uint16_t *>(out + 1024 + lane * 2) = scale;
+    *reinterpret_cast<uint4 *>(out + lane * S::CODE) = codes;
+    if constexpr (S::QT == 8) *reinterpret_cast<uint4 *>(out + lane * S::CODE + 16) = codes2;
+    *reinterpret_cast<uint16_t *>(out + 64 * S::CODE + lane * 2) = scale;
 }
 
 }  // namespace lv

@@ -147,12 +147,21 @@ def test_step_api_state_errors(lva, ctx, tiny_models):
     s.close(); model.close()
 
 
-@pytest.fixture(scope="module")
-def wide_model(lva, tmp_path_factory):
-    """LLaMA-7B layer shape (dim 4096, 32 heads, ff 11008) with 2 layers and a small vocabulary: the shape class
-    the persistent decode kernel is built for."""
-    p = str(tmp_path_factory.mktemp("wide") / "wide_q4.ggml")
-    lva.write_model(p, wtype=lva.LV_Q4_0, seed=9, vocab=2048, dim=4096, heads=32, layers=2, ff=11008)
+WIDE_SHAPES = {   # the shape classes the persistent decode kernel is compiled for, cut down to 2 layers and a small vocabulary
+    "7b_q4_0": dict(wtype="q4_0", dim=4096, heads=32, ff=11008),
+    "7b_q8_0": dict(wtype="q8_0", dim=4096, heads=32, ff=11008),
+    "13b_q4_0": dict(wtype="q4_0", dim=5120, heads=40, ff=13824),
+    "13b_q8_0": dict(wtype="q8_0", dim=5120, heads=40, ff=13824),
+}
+
+
+@pytest.fixture(scope="module", params=list(WIDE_SHAPES))
+def wide_model(request, lva, tmp_path_factory):
+    """LLaMA-7B / 13B layer shapes with 2 layers and a small vocabulary"""
+    cfg = dict(WIDE_SHAPES[request.param])
+    wtype = lva.LV_Q4_0 if cfg.pop("wtype") == "q4_0" else lva.LV_Q8_0
+    p = str(tmp_path_factory.mktemp("wide") / f"wide_{request.param}.ggml")
+    lva.write_model(p, wtype=wtype, seed=9, vocab=2048, layers=2, **cfg)
     return p
 
 
@@ -179,7 +188,7 @@ def test_persistent_kernel_matches_oracle_and_operator_path(lva, orc, ctx, wide_
         got_pk, got_ops = pk.logits(), ops.logits()
         _check_logits(got_pk, want)
         _check_logits(got_ops, want)
-        assert np.max(np.abs(got_pk - got_ops)) <= 1e-4 * np.max(np.abs(want))
+        assert np.max(np.abs(got_pk - got_ops)) <= 3e-4 * np.max(np.abs(want))   # two fp32 summation orders
         pos += 1
     # both paths left the same cache behind (up to fp16 rounding of differently ordered fp32 sums)
     for layer in range(2):
