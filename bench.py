@@ -16,6 +16,7 @@ import argparse
 import importlib
 import json
 import os
+import re
 import sys
 import time
 
@@ -26,6 +27,17 @@ if ROOT not in sys.path:
 CONTEXT = 512
 HBM_PEAK_GBS = 8000.0
 SHAPE = dict(vocab=32000, dim=4096, heads=32, layers=32, ff=11008)
+
+
+def recorded_traffic():
+    """HBM bytes per launch of the decode kernel as counted by the hardware (FETCH_SIZE + WRITE_SIZE, calibrated on a
+    plain copy): a figure from a separate rocprofv3 --pmc run, kept with its commands under profiles/; None if absent."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "mega_decode_kernel_7b_q4_0_ctx512_pmc.md")
+    try:
+        m = re.search(r"^traffic_bytes_per_launch = (\d+)", open(path).read(), re.M)
+        return int(m.group(1)) if m else None
+    except OSError:
+        return None
 
 
 def algorithmic_bytes(pos):
@@ -157,7 +169,7 @@ def main():
                    "decode_path": path_kind, "device": device, "compute_units": cus},
         "roofline": {"bound": "hbm", "kernel": "mega_decode_kernel (one launch per token)" if path_kind == "persistent" else "decode step (all launches)",
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "algorithmic_bytes_per_launch": int(avg_bytes), "avg_launch_ms": round(avg_ms, 4), "traffic": None},
+                     "algorithmic_bytes_per_launch": int(avg_bytes), "avg_launch_ms": round(avg_ms, 4), "traffic": recorded_traffic()},
         "cpu_baseline": cpu,
     }
     print(json.dumps(out), flush=True)

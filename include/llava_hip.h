@@ -136,6 +136,8 @@ int lv_dev_free(lv_ctx *ctx, void *dptr);
 int lv_dev_upload(lv_ctx *ctx, void *dptr, const void *src, uint64_t bytes);
 int lv_dev_download(lv_ctx *ctx, void *dst, const void *dptr, uint64_t bytes);
 int lv_dev_zero(lv_ctx *ctx, void *dptr, uint64_t bytes);
+/* device-to-device copy on the context's stream (asynchronous); size and pointers multiples of 16 */
+int lv_dev_copy(lv_ctx *ctx, void *dst, const void *src, uint64_t bytes);
 int lv_ctx_sync(lv_ctx *ctx);
 
 /* ---- GPU time between two points of a stream, by HIP events recorded on that very stream (the reference has

@@ -308,6 +308,23 @@ extern "C" int lv_dev_zero(lv_ctx *c, void *dptr, uint64_t bytes)
     return zero_async(dptr, bytes, c->stream);
 }
 
+// plain device-to-device copy (16 bytes per thread per pass): the yardstick for achievable HBM bandwidth and for
+// calibrating hardware traffic counters
+__global__ void copy_kernel(uint4 *__restrict__ dst, const uint4 *__restrict__ src, uint64_t n16)
+{
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (uint64_t)gridDim.x * blockDim.x) dst[i] = src[i];
+}
+
+extern "C" int lv_dev_copy(lv_ctx *c, void *dst, const void *src, uint64_t bytes)
+{
+    if (!c || (bytes && (!dst || !src))) return fail(LV_ERR_ARG, "lv_dev_copy: null argument");
+    if (bytes % 16 || ((uintptr_t)dst | (uintptr_t)src) % 16) return fail(LV_ERR_ARG, "lv_dev_copy: size and pointers must be multiples of 16");
+    if (bytes == 0) return LV_OK;
+    copy_kernel<<<dim3(256 * 16), dim3(256), 0, c->stream>>>(static_cast<uint4 *>(dst), static_cast<const uint4 *>(src), bytes / 16);
+    HIP_TRY(hipGetLastError());
+    return LV_OK;
+}
+
 // -----------------------------------------------------------------------------------------------------------
 // matrices
 // -----------------------------------------------------------------------------------------------------------

@@ -5,6 +5,7 @@
     python llama-vulkan_amd/measure.py decode-q8     7B q8_0, cache positions 1920..2047 (128 greedy steps)
     python llama-vulkan_amd/measure.py decode-13b    13B q4_0, 32-token prompt + 256 greedy steps
     python llama-vulkan_amd/measure.py prefill-13b   13B q8_0, 512-token prompt evaluated in one lv_step_begin
+    python llama-vulkan_amd/measure.py copy          1 GiB device-to-device copy: achievable bandwidth, counter calibration
     python llama-vulkan_amd/measure.py all
 
 Every figure is algorithmic bytes (weights as stored in the GGML file, 18 B / 34 B per 32 weights, plus vectors and the
@@ -64,6 +65,20 @@ def gemv_cases(ctx):
                 ctx.matrix_free(m)
             ctx.free(x)
             ctx.free(out)
+
+
+def copy_case(ctx):
+    n = 1 << 30
+    src, dst = ctx.zeros(n), ctx.zeros(n)
+    lva.check(ctx.lib.lv_dev_copy(ctx.h, dst, src, n))
+    ctx.sync()
+    ctx.timer_start()
+    for _ in range(4):
+        lva.check(ctx.lib.lv_dev_copy(ctx.h, dst, src, n))
+    ms = ctx.timer_stop() / 4
+    emit(case="copy", bytes_read=n, bytes_written=n, ms=round(ms, 4), GBps_read_plus_write=round(2 * n / ms / 1e6, 1))
+    ctx.free(src)
+    ctx.free(dst)
 
 
 def model_file(preset, wtype, seed):
@@ -135,6 +150,8 @@ def main():
     ctx = lva.Context(0)
     name, cus, hbm = ctx.info()
     emit(case="device", name=name, compute_units=cus, hbm_GiB=hbm >> 30)
+    if which in ("copy", "all"):
+        copy_case(ctx)
     if which in ("gemv", "all"):
         gemv_cases(ctx)
     if which in ("decode-q8", "all"):
