@@ -297,15 +297,17 @@ struct MegaLds {
     float xs[XS];                    // the phase's input vector (during attention: exp(score) of the chunk)
     float red[RED_ROWS * RED_COLS];  // per-row partial sums, one column per slab
     float xown[S::ROWS_C];           // this workgroup's rows of the residual stream
-    float scratch[S::NW];
+    float scratch[2 * S::NW];        // two halves: mean, then variance
     float attn_red[S::NW * (S::R + 1)];
 };
 
+// Sum over the workgroup through NW floats of LDS.  One barrier: the caller guarantees that nobody still reads
+// `scratch` from an earlier use (consecutive sums use different halves of the scratch area, and every phase has
+// barriers of its own before the next pair of sums).
 template <int NW>
 __device__ __forceinline__ float block_sum(float v, float *scratch /* NW floats */)
 {
     v = wave_sum(v);
-    lds_barrier();
     if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = v;
     lds_barrier();
     float t = 0.f;
@@ -342,7 +344,7 @@ __device__ __forceinline__ void acquire_vector(float *xs, const float *src, cons
             const float c = want[j] ? v[j] - mean : 0.f;
             q = fmaf(c, c, q);
         }
-        const float inv = rsqrtf(block_sum<NW>(q, scratch) / (float)N);
+        const float inv = rsqrtf(block_sum<NW>(q, scratch + NW) / (float)N);
 #pragma unroll
         for (int j = 0; j < PER; j++)
             if (want[j]) xs[threadIdx.x + j * T] = (v[j] * wn[j]) * inv;
@@ -426,7 +428,6 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
                 chunk = (chunk + 3) & ~3u;
                 const uint32_t p_begin = min((uint32_t)c * chunk, n_valid), p_end = min(p_begin + chunk, n_valid);
                 const int sub = lane & 15, rsel = w * 4 + (lane >> 4);
-                float *e_lds = xs;            // chunk <= backlog/CPH + 3 floats; xs is free between phases A and C
                 constexpr int RPR = NW * 4;   // cache rows per round of the workgroup
                 constexpr int PRE = 2;        // rounds whose K, V and rotation rows are requested before the query arrives
                 const size_t row_off = (size_t)h * R + sub * 8;
@@ -463,7 +464,8 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
                 MEGA_STAMP(3);
                 const float scale = rsqrtf((float)R);
                 float den = 0.f;
-                auto score_round = [&](uint32_t p, const uint4 &kraw, const float4 &t0, const float4 &t1) {
+                // exp(score / sqrt(R)) of cache row p for this 16-lane group's query head; every lane of the group gets it
+                auto weight_of = [&](uint32_t p, const uint4 &kraw, const float4 &t0, const float4 &t1) -> float {
                     float s = 0.f;
                     if (p < p_end) {
                         float kf[8];
@@ -482,25 +484,13 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
                             s = fmaf(stn[i], crs, s);
                         }
                     }
-                    s = group16_sum(s);
-                    float e = 0.f;
-                    if (p < p_end) {
-                        e = __expf(s * scale);
-                        if (sub == 0) e_lds[p - p_begin] = e;
-                    }
+                    s = group16_sum(s);   // the same bits in all 16 lanes
+                    const float e = p < p_end ? __expf(s * scale) : 0.f;
                     den += (sub == 0) ? e : 0.f;
+                    return e;
                 };
-#pragma unroll
-                for (int r = 0; r < PRE; r++) score_round(p_begin + r * RPR + rsel, kpre[r], tpre[r][0], tpre[r][1]);
-                for (uint32_t p0 = p_begin + PRE * RPR; p0 < p_end; p0 += RPR) {
-                    const uint32_t p = p0 + rsel;
-                    const uint32_t pc = (p < p_end && p != pos) ? p : 0;
-                    const float4 *tp = reinterpret_cast<const float4 *>(a.trig + (size_t)(p < p_end ? pos - p : 0) * (R / 2) + sub * 4);
-                    score_round(p, *reinterpret_cast<const uint4 *>(kc + (size_t)pc * D + row_off), tp[0], tp[1]);
-                }
-                lds_barrier();
                 float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-                auto pv_round = [&](uint32_t p, const uint4 &vraw) {
+                auto add_row = [&](uint32_t p, float e, const uint4 &vraw) {
                     if (p < p_end) {
                         float vf[8];
                         unpack8(vf, vraw);
@@ -508,17 +498,23 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
 #pragma unroll
                             for (int i = 0; i < 8; i++) vf[i] = qkv[16 + i];
                         }
-                        const float e = e_lds[p - p_begin];
 #pragma unroll
                         for (int i = 0; i < 8; i++) acc[i] = fmaf(e, vf[i], acc[i]);
                     }
                 };
+                // a row's weight is computed and used by the same 16 lanes: no exchange through LDS, no barrier
 #pragma unroll
-                for (int r = 0; r < PRE; r++) pv_round(p_begin + r * RPR + rsel, vpre[r]);
+                for (int r = 0; r < PRE; r++) {
+                    const uint32_t p = p_begin + r * RPR + rsel;
+                    add_row(p, weight_of(p, kpre[r], tpre[r][0], tpre[r][1]), vpre[r]);
+                }
                 for (uint32_t p0 = p_begin + PRE * RPR; p0 < p_end; p0 += RPR) {
                     const uint32_t p = p0 + rsel;
                     const uint32_t pc = (p < p_end && p != pos) ? p : 0;
-                    pv_round(p, *reinterpret_cast<const uint4 *>(vc + (size_t)pc * D + row_off));
+                    const float4 *tp = reinterpret_cast<const float4 *>(a.trig + (size_t)(p < p_end ? pos - p : 0) * (R / 2) + sub * 4);
+                    const uint4 kraw = *reinterpret_cast<const uint4 *>(kc + (size_t)pc * D + row_off);
+                    const uint4 vraw = *reinterpret_cast<const uint4 *>(vc + (size_t)pc * D + row_off);
+                    add_row(p, weight_of(p, kraw, tp[0], tp[1]), vraw);
                 }
 #pragma unroll
                 for (int off = 16; off < 64; off <<= 1) {
@@ -568,7 +564,6 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
             for (int c = 0; c < S::CPH; c++) { n += nd[c]; d += nd[S::CPH + c]; }
             st_dev(xc + S::OFF_O + b * R + st, n / d);
         }
-        lds_barrier();  // xs (attention scratch) is about to be overwritten
 
         // ================= C: x += Wo o ============================================================================
         MEGA_STAMP(5);
