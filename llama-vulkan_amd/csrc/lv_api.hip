@@ -574,13 +574,23 @@ extern "C" int lv_kernel_gemv_silu(lv_ctx *c, float *out, const lv_matrix *w3, c
 static int launch_gemm_presplit(hipStream_t st, float *out, uint32_t ldo, const lv_matrix &w, uint32_t n, const uint16_t *xh, const uint16_t *xl,
                                 bool accumulate);
 
+// fp32 activations -> fp16 halves in the element order the GEMM for weight type `ftype` expects
+static int launch_split(hipStream_t st, uint16_t *xh, uint16_t *xl, const float *x, uint32_t n, uint32_t K, uint32_t ftype)
+{
+    const uint32_t n_pad = (n + kGemmTile - 1) / kGemmTile * kGemmTile;
+    const dim3 grid((K / 4 + 255) / 256, n_pad);
+    if (ftype == LV_Q4_0) split_half_kernel<4><<<grid, dim3(256), 0, st>>>(xh, xl, x, n, K);
+    else split_half_kernel<8><<<grid, dim3(256), 0, st>>>(xh, xl, x, n, K);
+    HIP_TRY(hipGetLastError());
+    return LV_OK;
+}
+
 static int launch_gemm(hipStream_t st, float *out, uint32_t ldo, const lv_matrix &w, const float *x, uint32_t n, uint16_t *xh, uint16_t *xl,
                        bool accumulate)
 {
     const uint32_t K = w.view.cols, n_pad = (n + kGemmTile - 1) / kGemmTile * kGemmTile;
     if (K % 32) return fail(LV_ERR_ARG, "gemm: %u columns", K);
-    split_half_kernel<<<dim3((K / 4 + 255) / 256, n_pad), dim3(256), 0, st>>>(xh, xl, x, n, K);
-    HIP_TRY(hipGetLastError());
+    LV_TRY(launch_split(st, xh, xl, x, n, K, w.ftype));
     return launch_gemm_presplit(st, out, ldo, w, n, xh, xl, accumulate);
 }
 
@@ -591,9 +601,17 @@ static int launch_gemm_presplit(hipStream_t st, float *out, uint32_t ldo, const 
     const uint32_t n_pad = (n + kGemmTile - 1) / kGemmTile * kGemmTile;
     GemmArgs a{};
     a.out = out; a.xh = xh; a.xl = xl; a.w = w.view; a.n = n; a.ldo = ldo; a.accumulate = accumulate ? 1 : 0;
-    const dim3 grid((w.view.rows + kGemmTile - 1) / kGemmTile, n_pad / kGemmTile);
-    if (w.ftype == LV_Q4_0) gemm_kernel<4><<<grid, dim3(256), 0, st>>>(a);
-    else if (w.ftype == LV_Q8_0) gemm_kernel<8><<<grid, dim3(256), 0, st>>>(a);
+    // 128-row workgroups unless those would leave CUs idle: then 64-row ones, twice as many
+    const uint32_t token_tiles = n_pad / kGemmTile;
+    const bool narrow = (uint64_t)((w.view.rows + 127) / 128) * token_tiles < 512;
+    const dim3 grid((w.view.rows + (narrow ? 63 : 127)) / (narrow ? 64 : 128), token_tiles);
+    if (w.ftype == LV_Q4_0) {
+        if (narrow) gemm_kernel<4, 64><<<grid, dim3(256), 0, st>>>(a);
+        else gemm_kernel<4, 128><<<grid, dim3(256), 0, st>>>(a);
+    } else if (w.ftype == LV_Q8_0) {
+        if (narrow) gemm_kernel<8, 64><<<grid, dim3(256), 0, st>>>(a);
+        else gemm_kernel<8, 128><<<grid, dim3(256), 0, st>>>(a);
+    }
     else return fail(LV_ERR_ARG, "gemm: matrix type %u", w.ftype);
     HIP_TRY(hipGetLastError());
     return LV_OK;
@@ -1203,10 +1221,13 @@ static int record_prefill(lv_session *s, uint32_t idx0, uint32_t n, bool with_he
         const LayerWeights &lw = m->layers[li];
         normalize_kernel<<<dim3(n), dim3(256), 0, st>>>(s->pf_xn, s->pf_x, lw.attn_norm, D);
         HIP_TRY(hipGetLastError());
-        split_half_kernel<<<dim3((D / 4 + 255) / 256, (n + kGemmTile - 1) / kGemmTile * kGemmTile), dim3(256), 0, st>>>(s->pf_xh, s->pf_xl, s->pf_xn, n, D);
+        LV_TRY(launch_split(st, s->pf_xh, s->pf_xl, s->pf_xn, n, D, lw.wq.ftype));
         LV_TRY(launch_gemm_presplit(st, s->pf_q, D, lw.wq, n, s->pf_xh, s->pf_xl, false));
-        LV_TRY(launch_gemm_presplit(st, s->pf_k, D, lw.wk, n, s->pf_xh, s->pf_xl, false));
-        LV_TRY(launch_gemm_presplit(st, s->pf_v, D, lw.wv, n, s->pf_xh, s->pf_xl, false));
+        // one split serves all three when they share a weight type (the element order depends on it)
+        if (lw.wk.ftype == lw.wq.ftype) LV_TRY(launch_gemm_presplit(st, s->pf_k, D, lw.wk, n, s->pf_xh, s->pf_xl, false));
+        else LV_TRY(launch_gemm(st, s->pf_k, D, lw.wk, s->pf_xn, n, s->pf_xh, s->pf_xl, false));
+        if (lw.wv.ftype == lw.wk.ftype) LV_TRY(launch_gemm_presplit(st, s->pf_v, D, lw.wv, n, s->pf_xh, s->pf_xl, false));
+        else LV_TRY(launch_gemm(st, s->pf_v, D, lw.wv, s->pf_xn, n, s->pf_xh, s->pf_xl, false));
         kv_append_kernel<<<kv_grid, dim3(256), 0, st>>>(kv_ptr(s, li, 0), s->pf_k, pos_ptr, idx0, D, s->backlog);
         kv_append_kernel<<<kv_grid, dim3(256), 0, st>>>(kv_ptr(s, li, 1), s->pf_v, pos_ptr, idx0, D, s->backlog);
         HIP_TRY(hipGetLastError());
@@ -1215,9 +1236,10 @@ static int record_prefill(lv_session *s, uint32_t idx0, uint32_t n, bool with_he
         LV_TRY(launch_gemm(st, s->pf_x, D, lw.wo, s->pf_vo, n, s->pf_xh, s->pf_xl, true));
         normalize_kernel<<<dim3(n), dim3(256), 0, st>>>(s->pf_xn, s->pf_x, lw.ffn_norm, D);
         HIP_TRY(hipGetLastError());
-        split_half_kernel<<<dim3((D / 4 + 255) / 256, (n + kGemmTile - 1) / kGemmTile * kGemmTile), dim3(256), 0, st>>>(s->pf_xh, s->pf_xl, s->pf_xn, n, D);
+        LV_TRY(launch_split(st, s->pf_xh, s->pf_xl, s->pf_xn, n, D, lw.w3.ftype));
         LV_TRY(launch_gemm_presplit(st, s->pf_g1, F, lw.w3, n, s->pf_xh, s->pf_xl, false));
-        LV_TRY(launch_gemm_presplit(st, s->pf_g2, F, lw.w1, n, s->pf_xh, s->pf_xl, false));
+        if (lw.w1.ftype == lw.w3.ftype) LV_TRY(launch_gemm_presplit(st, s->pf_g2, F, lw.w1, n, s->pf_xh, s->pf_xl, false));
+        else LV_TRY(launch_gemm(st, s->pf_g2, F, lw.w1, s->pf_xn, n, s->pf_xh, s->pf_xl, false));
         const size_t count = (size_t)n * F;
         silu_mul_kernel<<<dim3((unsigned)((count + 255) / 256)), dim3(256), 0, st>>>(s->pf_g1, s->pf_g1, s->pf_g2, count);
         HIP_TRY(hipGetLastError());

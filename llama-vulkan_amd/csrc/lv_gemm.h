@@ -8,8 +8,8 @@
 //     x*w ~= xh*wh + xl*wh + xh*wl                      (three MFMAs; the dropped xl*wl term is below 2^-22)
 // so the batched path agrees with the one-token fp32 path to fp32 rounding, not to fp16 rounding.
 //
-// Tiling: workgroup = 256 threads = 4 waves, output tile 128 tokens x 128 weight rows, K step 64 (two quant
-// blocks).  One thread dequantises one (row, block) pair per step; every wave owns a 64 x 64 sub-tile = 2 x 2
+// Tiling: workgroup = 256 threads = 4 waves, output tile 128 tokens x 128 (or 64) weight rows, K step 64 (two quant
+// blocks).  One thread dequantises one (row, block) pair per step; every wave owns a 64 x 64 (or 32 x 64) sub-tile of
 // v_mfma_f32_32x32x16_f16 tiles.  Global loads of step s+1 are issued before the MFMAs of step s.
 #pragma once
 
@@ -20,11 +20,13 @@ namespace lv {
 typedef _Float16 lv_h8 __attribute__((ext_vector_type(8)));
 typedef float lv_f16v __attribute__((ext_vector_type(16)));
 
-constexpr int kGemmTile = 128;  // tokens and rows per workgroup
+constexpr int kGemmTile = 128;  // tokens per workgroup (batches are padded to multiples of it)
 constexpr int kGemmK = 64;      // K per step
 constexpr int kGemmLd = kGemmK + 8;  // LDS row stride in halfs (the pad spreads 16-byte reads over the banks)
 
-// x[n][K] fp32 -> xh, xl [n_pad][K] fp16 (rows n..n_pad-1 zero)
+// x[n][K] fp32 -> xh, xl [n_pad][K] fp16 (rows n..n_pad-1 zero).  Inside every 32-element block the halves are stored
+// in the order the GEMM for weight type QT keeps its weight halves in (gemm_k_position).
+template <int QT>
 __global__ void split_half_kernel(uint16_t *__restrict__ xh, uint16_t *__restrict__ xl, const float *__restrict__ x, uint32_t n, uint32_t K)
 {
     const uint32_t row = blockIdx.y;
@@ -33,14 +35,19 @@ __global__ void split_half_kernel(uint16_t *__restrict__ xh, uint16_t *__restric
     float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
     if (row < n) v = *reinterpret_cast<const float4 *>(x + (size_t)row * K + i);
     const float f[4] = {v.x, v.y, v.z, v.w};
-    uint16_t h[4], l[4];
+    const uint32_t blk0 = i & ~31u, e0 = i & 31u;
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-        h[j] = float_to_half_bits(f[j]);
-        l[j] = float_to_half_bits(f[j] - half_bits_to_float(h[j]));
+        const uint16_t h = float_to_half_bits(f[j]);
+        const uint16_t l = float_to_half_bits(f[j] - half_bits_to_float(h));
+        int pos = (int)e0 + j;
+        if constexpr (QT == 4) {
+            const int hi = pos >= 16 ? 1 : 0, ee = pos & 15, ii = ee >> 2, b = ee & 3;
+            pos = 8 * ii + 2 * ((b & 1) * 2 + hi) + (b >> 1);
+        }
+        xh[(size_t)row * K + blk0 + pos] = h;
+        xl[(size_t)row * K + blk0 + pos] = l;
     }
-    *reinterpret_cast<uint2 *>(xh + (size_t)row * K + i) = make_uint2(h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16));
-    *reinterpret_cast<uint2 *>(xl + (size_t)row * K + i) = make_uint2(l[0] | ((uint32_t)l[1] << 16), l[2] | ((uint32_t)l[3] << 16));
 }
 
 // ff[n][F] = a * b / (exp(-b) + 1)   (matmul_silu_ff.comp:96 with a = W3 x, b = W1 x)
@@ -62,140 +69,187 @@ struct GemmArgs {
     int accumulate;         // out += instead of out =
 };
 
+typedef _Float16 lv_h2 __attribute__((ext_vector_type(2)));
+
+// Position inside a 32-element block at which the weight halves of element e are stored in LDS, and therefore at
+// which the activation halves must be stored too (split_half_kernel).  q8_0: natural order.  q4_0: the order in
+// which whole dwords of codes unpack into pairs of fp16 — dword i, shift 4j holds elements (4i, 4i+2), (16+4i, 18+4i),
+// (4i+1, 4i+3), (17+4i, 19+4i) for j = 0..3 (byte b of a block carries element b in its low and b+16 in its high nibble).
 template <int QT>
-__device__ __forceinline__ void gemm_dequant_block(uint16_t *wh, uint16_t *wl, const MatView &w, uint32_t row, uint32_t blk, bool valid,
-                                                   const uint4 &c0, const uint4 &c1, uint16_t dbits)
+__host__ __device__ constexpr int gemm_k_position(int e)
 {
-    // 32 weights of one block -> 32 hi + 32 lo halfs at wh/wl (contiguous in k)
-    const float d = valid ? half_bits_to_float(dbits) : 0.f;
-    float v[32];
+    if (QT != 4) return e;
+    const int hi = e >= 16 ? 1 : 0, ee = e & 15, i = ee >> 2, b = ee & 3;
+    const int j = (b & 1) * 2 + hi;
+    return 8 * i + 2 * j + (b >> 1);
+}
+
+// 32 weights of one block -> 32 hi + 32 lo halfs at wh/wl, in gemm_k_position order.  All in packed fp16 arithmetic:
+// the integer code as fp16 (1024 + u has the bit pattern 0x6400 | u), hi = RTE(code * d), lo = fma(code, d, -hi), the
+// rounding error of that product, which fp16 represents exactly.
+template <int QT>
+__device__ __forceinline__ void gemm_dequant_block(uint16_t *wh, uint16_t *wl, bool valid, const uint4 &c0, const uint4 &c1, uint16_t dbits)
+{
+    union { uint16_t u; _Float16 h; } db;
+    db.u = valid ? dbits : (uint16_t)0;
+    const _Float16 d = db.h;
+    const lv_h2 dd = {d, d};
+    uint32_t ph[16], pl[16];
+    auto emit = [&](int slot, uint32_t packed_codes, _Float16 bias) {
+        // packed_codes: two halfs 0x6400 | u
+        union { uint32_t u; lv_h2 h; } c, hi, lo;
+        c.u = packed_codes;
+        const lv_h2 bb = {bias, bias};
+        const lv_h2 code = c.h - bb;                 // exact: small integers
+        hi.h = code * dd;
+        lo.h = __builtin_elementwise_fma(code, dd, -hi.h);
+        ph[slot] = hi.u;
+        pl[slot] = lo.u;
+    };
     if constexpr (QT == 4) {
         const uint32_t q[4] = {c0.x, c0.y, c0.z, c0.w};
 #pragma unroll
         for (int i = 0; i < 4; i++)
 #pragma unroll
-            for (int b = 0; b < 4; b++) {
-                const uint32_t byte = (q[i] >> (8 * b)) & 0xffu;
-                v[4 * i + b] = (float)((int)(byte & 15u) - 8) * d;        // element j of the block: low nibble of byte j
-                v[16 + 4 * i + b] = (float)((int)(byte >> 4) - 8) * d;    // element j + 16: high nibble
-            }
+            for (int j = 0; j < 4; j++) emit(4 * i + j, ((q[i] >> (4 * j)) & 0x000f000fu) | 0x64006400u, (_Float16)1032.f);
     } else {
         const uint32_t q[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
 #pragma unroll
-        for (int i = 0; i < 8; i++)
-#pragma unroll
-            for (int b = 0; b < 4; b++) v[4 * i + b] = (float)(int)(int8_t)((q[i] >> (8 * b)) & 0xffu) * d;
+        for (int i = 0; i < 8; i++) {
+            const uint32_t u = q[i] ^ 0x80808080u;   // int8 -> biased unsigned
+            emit(2 * i, ((u & 0xffu) | ((u & 0xff00u) << 8)) | 0x64006400u, (_Float16)1152.f);
+            emit(2 * i + 1, (((u >> 16) & 0xffu) | ((u >> 8) & 0xff0000u)) | 0x64006400u, (_Float16)1152.f);
+        }
     }
-    (void)w; (void)row; (void)blk;
 #pragma unroll
     for (int g = 0; g < 4; g++) {
-        uint32_t ph[4], pl[4];
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const float a = v[8 * g + 2 * j], b = v[8 * g + 2 * j + 1];
-            const uint16_t ha = float_to_half_bits(a), hb = float_to_half_bits(b);
-            const uint16_t la = float_to_half_bits(a - half_bits_to_float(ha)), lb = float_to_half_bits(b - half_bits_to_float(hb));
-            ph[j] = ha | ((uint32_t)hb << 16);
-            pl[j] = la | ((uint32_t)lb << 16);
-        }
-        *reinterpret_cast<uint4 *>(wh + 8 * g) = make_uint4(ph[0], ph[1], ph[2], ph[3]);
-        *reinterpret_cast<uint4 *>(wl + 8 * g) = make_uint4(pl[0], pl[1], pl[2], pl[3]);
+        *reinterpret_cast<uint4 *>(wh + 8 * g) = make_uint4(ph[4 * g], ph[4 * g + 1], ph[4 * g + 2], ph[4 * g + 3]);
+        *reinterpret_cast<uint4 *>(wl + 8 * g) = make_uint4(pl[4 * g], pl[4 * g + 1], pl[4 * g + 2], pl[4 * g + 3]);
     }
 }
 
-template <int QT>
+// RM = weight rows per workgroup (128 or 64); tokens per workgroup: 128.  The four waves split the tile 2 x 2
+// (RM = 128: 64 tokens x 64 rows each) or 4 x 1 (RM = 64: 32 tokens x 64 rows each).  The narrow form doubles the
+// number of workgroups for matrices that would otherwise not fill 256 CUs.
+template <int QT, int RM>
 __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs a)
 {
-    constexpr int CPB = QT == 4 ? 1 : 2;  // uint4 of codes per block
-    __shared__ __attribute__((aligned(16))) uint16_t sXh[kGemmTile * kGemmLd], sXl[kGemmTile * kGemmLd], sWh[kGemmTile * kGemmLd],
-        sWl[kGemmTile * kGemmLd];
+    constexpr int CPB = QT == 4 ? 1 : 2;          // uint4 of codes per block
+    constexpr int TN = kGemmTile;                 // tokens per workgroup
+    constexpr int WN = RM / 64;                   // waves along the rows
+    constexpr int WM = 4 / WN;                    // waves along the tokens
+    constexpr int MT = TN / WM / 32;              // 32-token tiles per wave
+    __shared__ __attribute__((aligned(16))) uint16_t sXh[TN * kGemmLd], sXl[TN * kGemmLd], sWh[RM * kGemmLd], sWl[RM * kGemmLd];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
-    const uint32_t tok0 = blockIdx.y * kGemmTile, row0 = blockIdx.x * kGemmTile;
+    const int wm = wave / WN, wn = wave % WN;
+    const uint32_t tok0 = blockIdx.y * TN, row0 = blockIdx.x * RM;
     const uint32_t K = a.w.cols, nb = K / 32, steps = (K + kGemmK - 1) / kGemmK;
 
-    // this thread's weight block of a step: row r_w, block (2*step + b_w)
+    // this thread's weight block of a step: row r_w, block (2*step + b_w); with RM = 64 half of the threads have none
     const int r_w = tid >> 1, b_w = tid & 1;
+    const bool has_w = r_w < RM;
     const uint32_t wrow = row0 + r_w;
-    const bool wrow_ok = wrow < a.w.rows;
+    const bool wrow_ok = has_w && wrow < a.w.rows;
     // this thread's four 16-byte pieces of the activation tile of a step: token rows tid/8 + 32*i, halfs (tid%8)*8..+7
     const int xr = tid >> 3, xc = (tid & 7) * 8;
 
-    uint4 c0 = make_uint4(0, 0, 0, 0), c1 = c0;
-    uint16_t dbits = 0;
-    bool wvalid = false;
-    uint4 gh[4], gl[4];
-    auto fetch = [&](uint32_t step) {
+    // two register sets: the loads of step s + 2 are in flight while step s is multiplied (one step of MFMAs is
+    // shorter than a trip to memory)
+    struct Staged {
+        uint4 c0, c1;
+        uint16_t dbits;
+        bool wvalid;
+        uint4 gh[4], gl[4];
+    } pre[2];
+    auto fetch = [&](Staged &p, uint32_t step) {
         const uint32_t blk = 2 * step + b_w;
-        wvalid = wrow_ok && blk < nb;
-        const size_t sb = (size_t)(wvalid ? wrow : 0) * nb + (wvalid ? blk : 0);
-        c0 = a.w.codes[sb * CPB];
-        if constexpr (QT == 8) c1 = a.w.codes[sb * CPB + 1];
-        dbits = a.w.scales[sb];
+        p.wvalid = wrow_ok && blk < nb;
+        p.c0 = p.c1 = make_uint4(0, 0, 0, 0);
+        p.dbits = 0;
+        if (has_w) {
+            const size_t sb = (size_t)(p.wvalid ? wrow : 0) * nb + (p.wvalid ? blk : 0);
+            p.c0 = a.w.codes[sb * CPB];
+            if constexpr (QT == 8) p.c1 = a.w.codes[sb * CPB + 1];
+            p.dbits = a.w.scales[sb];
+        }
         const uint32_t k = step * kGemmK + xc;
         const bool kok = k < K;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const size_t off = (size_t)(tok0 + xr + 32 * i) * K + (kok ? k : 0);
-            gh[i] = *reinterpret_cast<const uint4 *>(a.xh + off);
-            gl[i] = *reinterpret_cast<const uint4 *>(a.xl + off);
-            if (!kok) gh[i] = gl[i] = make_uint4(0, 0, 0, 0);
+            p.gh[i] = *reinterpret_cast<const uint4 *>(a.xh + off);
+            p.gl[i] = *reinterpret_cast<const uint4 *>(a.xl + off);
+            if (!kok) p.gh[i] = p.gl[i] = make_uint4(0, 0, 0, 0);
         }
     };
 
-    lv_f16v acc[2][2];
+    lv_f16v acc[MT][2];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < MT; i++)
 #pragma unroll
         for (int j = 0; j < 2; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-    fetch(0);
-    for (uint32_t step = 0; step < steps; step++) {
+    fetch(pre[0], 0);
+    if (steps > 1) fetch(pre[1], 1);
+    auto one_step = [&](Staged &P, uint32_t step) {
         // registers -> LDS
-        gemm_dequant_block<QT>(sWh + r_w * kGemmLd + b_w * 32, sWl + r_w * kGemmLd + b_w * 32, a.w, wrow, 0, wvalid, c0, c1, dbits);
+        if (has_w) gemm_dequant_block<QT>(sWh + r_w * kGemmLd + b_w * 32, sWl + r_w * kGemmLd + b_w * 32, P.wvalid, P.c0, P.c1, P.dbits);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            *reinterpret_cast<uint4 *>(sXh + (xr + 32 * i) * kGemmLd + xc) = gh[i];
-            *reinterpret_cast<uint4 *>(sXl + (xr + 32 * i) * kGemmLd + xc) = gl[i];
+            *reinterpret_cast<uint4 *>(sXh + (xr + 32 * i) * kGemmLd + xc) = P.gh[i];
+            *reinterpret_cast<uint4 *>(sXl + (xr + 32 * i) * kGemmLd + xc) = P.gl[i];
         }
         __syncthreads();
-        if (step + 1 < steps) fetch(step + 1);
+        if (step + 2 < steps) fetch(P, step + 2);
 #pragma unroll
         for (int kk = 0; kk < kGemmK / 16; kk++) {
             const int ko = kk * 16 + (lane >> 5) * 8;
-            lv_h8 xh[2], xl[2], wh[2], wl[2];
+            lv_h8 xh[MT], xl[MT], wh[2], wl[2];
 #pragma unroll
-            for (int t = 0; t < 2; t++) {
-                const int xrow = wm * 64 + t * 32 + (lane & 31), wr = wn * 64 + t * 32 + (lane & 31);
+            for (int t = 0; t < MT; t++) {
+                const int xrow = (wm * MT + t) * 32 + (lane & 31);
                 xh[t] = *reinterpret_cast<const lv_h8 *>(sXh + xrow * kGemmLd + ko);
                 xl[t] = *reinterpret_cast<const lv_h8 *>(sXl + xrow * kGemmLd + ko);
+            }
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                const int wr = wn * 64 + t * 32 + (lane & 31);
                 wh[t] = *reinterpret_cast<const lv_h8 *>(sWh + wr * kGemmLd + ko);
                 wl[t] = *reinterpret_cast<const lv_h8 *>(sWl + wr * kGemmLd + ko);
             }
+            // product by product over all tiles: consecutive MFMAs never wait for each other's accumulator
 #pragma unroll
-            for (int i = 0; i < 2; i++)
+            for (int i = 0; i < MT; i++)
 #pragma unroll
-                for (int j = 0; j < 2; j++) {
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xl[i], wh[j], acc[i][j], 0, 0, 0);
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh[i], wl[j], acc[i][j], 0, 0, 0);
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh[i], wh[j], acc[i][j], 0, 0, 0);
-                }
+                for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xl[i], wh[j], acc[i][j], 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < MT; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh[i], wl[j], acc[i][j], 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < MT; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh[i], wh[j], acc[i][j], 0, 0, 0);
         }
         __syncthreads();
+    };
+    for (uint32_t step = 0; step < steps; step += 2) {
+        one_step(pre[0], step);
+        if (step + 1 < steps) one_step(pre[1], step + 1);
     }
 
     // D[i][j]: i = token within the 32-tile, j = weight row; lane l holds j = l%32 and, in register r,
     // i = 8*(r/4) + 4*(l/32) + r%4
 #pragma unroll
-    for (int ti = 0; ti < 2; ti++)
+    for (int ti = 0; ti < MT; ti++)
 #pragma unroll
         for (int tj = 0; tj < 2; tj++) {
             const uint32_t m = row0 + wn * 64 + tj * 32 + (lane & 31);
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const uint32_t n = tok0 + wm * 64 + ti * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
+                const uint32_t n = tok0 + (wm * MT + ti) * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
                 if (n < a.n && m < a.w.rows) {
                     float *dst = a.out + (size_t)n * a.ldo + m;
                     *dst = a.accumulate ? *dst + acc[ti][tj][r] : acc[ti][tj][r];
