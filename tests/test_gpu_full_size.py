@@ -92,3 +92,68 @@ def test_7b_operator_chain_agrees_with_persistent_kernel(lva, ctx, model_7b):
         a.begin([ta], pos); b.begin([tb], pos)
         pos += 1
     a.close(); b.close(); model.close()
+
+
+SHAPE_13B = dict(vocab=32000, dim=5120, heads=40, layers=40, ff=13824)
+
+
+def _model_file(lva, name, wtype, seed, shape):
+    base = "/dev/shm" if os.access("/dev/shm", os.W_OK) else "/tmp"
+    path = os.path.join(base, f"llava_measure_{name}_seed{seed}.ggml")     # shared with llama-vulkan_amd/measure.py
+    if not os.path.exists(path):
+        lva.write_model(path + ".tmp", wtype=wtype, seed=seed, **shape)
+        os.replace(path + ".tmp", path)
+    return path
+
+
+def test_13b_q4_0_prompt_8_then_8_greedy_steps(lva, orc, ctx):
+    """the 13B layer shape at its full depth of 40 layers on the persistent kernel, against the oracle"""
+    path = _model_file(lva, "13b_q4_0", lva.LV_Q4_0, 2, SHAPE_13B)
+    om = orc.Model(path)
+    osess = orc.Session(om, 128)
+    model = lva.Model(ctx, path)
+    s = lva.Session(model, 128)
+    assert s.path() == lva.PATH_PERSISTENT
+    prompt = lva.synth_tokens(8, 3, SHAPE_13B["vocab"], seed=2)
+    want = osess.eval(prompt)
+    s.begin(prompt, 0)
+    pos = 8
+    for step in range(8):
+        got = s.logits()
+        assert np.all(np.abs(got - want) <= 1e-2 + 1e-3 * np.abs(want)), (step, float(np.max(np.abs(got - want))))
+        tok = orc.greedy(want)
+        assert s.argmax() == tok, step
+        want = osess.eval(np.array([tok], dtype=np.uint32))
+        s.begin([tok], pos)
+        pos += 1
+    s.close(); model.close(); osess.close(); om.close()
+
+
+def test_7b_q8_0_long_context_steps_match_oracle(lva, orc, ctx):
+    """7B q8_0 with the cache filled to position 1920 by the batched prompt path, then greedy steps on the persistent
+    kernel; the oracle continues from a copy of that cache (evaluating 1920 tokens on the CPU would take minutes), so
+    this pins the decode steps at a long context, not the prompt evaluation (tests/test_gpu_gemm.py does that)."""
+    path = _model_file(lva, "7b_q8_0", lva.LV_Q8_0, 1, SHAPE)
+    model = lva.Model(ctx, path)
+    s = lva.Session(model, 2048)
+    assert s.path() == lva.PATH_PERSISTENT
+    first = 1920
+    prompt = lva.synth_tokens(first, 3, SHAPE["vocab"], seed=1)
+    s.begin(prompt, 0)
+    tok = s.argmax()
+    om = orc.Model(path)
+    osess = orc.Session(om, 2048)
+    for layer in range(SHAPE["layers"]):
+        for which in (0, 1):
+            osess.kv_load(layer, which, s.kv(layer, which, first))
+    osess.set_pos(first)
+    pos = first
+    for step in range(4):
+        want = osess.eval(np.array([tok], dtype=np.uint32))
+        s.begin([tok], pos)
+        got = s.logits()
+        assert np.all(np.abs(got - want) <= 1e-2 + 1e-3 * np.abs(want)), (step, float(np.max(np.abs(got - want))))
+        tok = orc.greedy(want)
+        assert s.argmax() == tok, step
+        pos += 1
+    s.close(); model.close(); osess.close(); om.close()
