@@ -20,6 +20,7 @@
 #include "lv_kernels.h"
 #include "lv_mega.h"
 #include "lv_gemm.h"
+#include "lv_gemv_wide.h"
 #include "lv_attn_batch.h"
 
 using namespace lv;
@@ -444,6 +445,14 @@ template <int QT, int MODE>
 static void launch_gemv_mode(const GemvArgs &a, uint32_t batch, hipStream_t st)
 {
     const uint32_t nb = a.w.cols / 32;
+    // matrices that can keep 256 workgroups busy go through the streaming kernel (x staged once per workgroup)
+    if (a.w.rows >= 2048 && a.w.cols <= (uint32_t)kWideMaxK && batch <= 8) {
+        const uint32_t rows_per_wg = (a.w.rows + 255) / 256;
+        const uint32_t ns = (nb + 63) / 64, nr = kWideWaves / ns, per_set = (rows_per_wg + nr - 1) / nr;
+        const size_t red_bytes = (size_t)per_set * nr * (MODE == kGemvSilu ? 2 : 1) * ns * sizeof(float);
+        gemv_wide_kernel<QT, MODE><<<dim3((a.w.rows + rows_per_wg - 1) / rows_per_wg, batch), dim3(kWideWaves * 64), red_bytes, st>>>(a, rows_per_wg);
+        return;
+    }
     if (nb <= 64) launch_gemv_cfg<QT, MODE, 1, 1>(a, batch, st);
     else if (nb <= 128) launch_gemv_cfg<QT, MODE, 2, 1>(a, batch, st);
     else if (nb <= 256) launch_gemv_cfg<QT, MODE, 4, 1>(a, batch, st);

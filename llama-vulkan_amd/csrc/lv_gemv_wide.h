@@ -1,0 +1,133 @@
+// lv_gemv_wide.h — the dequant-fused GEMV for matrices large enough to occupy the whole chip (one launch = one
+// matrix, the shapes of matmul.glsl / matmul_silu_ff.comp at LLaMA sizes).
+//
+// Same streaming scheme as the phases of the persistent kernel: up to 256 workgroups of 12 wavefronts, the input
+// vector staged once per workgroup in LDS, every wavefront bound to one 64-block column slab (its lanes keep
+// their 32 activations in registers) and walking its share of the workgroup's rows with a register queue of
+// loads kept four rows ahead.  The small-workgroup kernel in lv_kernels.h re-reads x for every 4-16 rows and has
+// one row's loads in flight per wave; at 4096 x 11008 that costs more time than the weights themselves.
+#pragma once
+
+#include "lv_kernels.h"
+
+namespace lv {
+
+constexpr int kWideWaves = 12;
+// rows requested ahead per wave.  Eight was measured too: slower at 4096 rows (a row set is then three rows long and
+// most of the queue's first turn is empty), no faster at 32000.
+template <int QT, int NMAT> constexpr int kWideDepth = 4;
+constexpr int kWideMaxK = 64 * 32 * kWideWaves;   // widest row: every wave one slab (24576 columns)
+
+struct WideTile {
+    uint4 c, c2;
+    uint16_t d;
+};
+
+template <int QT>
+__device__ __forceinline__ void wide_load(WideTile &t, const MatView &m, uint64_t blk, bool ok)
+{
+    const uint64_t b = ok ? blk : 0;     // rows / lanes without a block read block 0 and are discarded
+    if constexpr (QT == 4) {
+        t.c = m.codes[b];
+    } else {
+        t.c = m.codes[2 * b];
+        t.c2 = m.codes[2 * b + 1];
+    }
+    t.d = m.scales[b];
+}
+
+template <int QT>
+__device__ __forceinline__ float wide_dot(const WideTile &t, const float (&x)[32], float xsum)
+{
+    if constexpr (QT == 4) return (q4_block_dot(t.c, x) - 8.f * xsum) * half_bits_to_float(t.d);
+    else return (q8_block_dot(t.c, t.c2, x) - 128.f * xsum) * half_bits_to_float(t.d);
+}
+
+// NMAT = 2: the SiLU form, rows of w (W3) and w1 (W1) with the same index are walked together.
+template <int QT, int MODE>
+__global__ __launch_bounds__(kWideWaves * 64) void gemv_wide_kernel(GemvArgs a, uint32_t rows_per_wg)
+{
+    constexpr int NMAT = MODE == kGemvSilu ? 2 : 1;
+    constexpr int NW = kWideWaves;
+    __shared__ __attribute__((aligned(16))) float xs[kWideMaxK];
+    extern __shared__ float red[];       // [rows_per_wg rounded up to 4*NR][NMAT][NS]
+    const uint32_t N = a.w.rows, K = a.w.cols, nb = K / 32;
+    const uint32_t z = blockIdx.y;
+    const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int NS = (int)((nb + 63) / 64), NR = NW / NS;        // slabs; row sets (waves sharing a slab split the rows)
+    const int slab = w % NS, rset = w / NS;
+    const bool active = rset < NR;
+    const uint32_t blk_col = (uint32_t)slab * 64 + lane;
+    const bool lane_ok = active && blk_col < nb;
+    const uint32_t row0 = blockIdx.x * rows_per_wg;
+    const uint32_t n_rows = row0 < N ? min(rows_per_wg, N - row0) : 0;
+    const uint32_t per_set = (rows_per_wg + NR - 1) / NR;       // rows per row set (static upper bound)
+
+    // ---- x -> LDS -> registers -----------------------------------------------------------------------------------
+    const float *xz = a.x + (size_t)z * K;
+    for (uint32_t i = threadIdx.x * 4; i < K; i += NW * 64 * 4) *reinterpret_cast<float4 *>(xs + i) = *reinterpret_cast<const float4 *>(xz + i);
+    // the first rows' loads go out before the wait for x
+    constexpr int DEPTH = kWideDepth<QT, NMAT>;
+    WideTile q[NMAT][DEPTH];
+    auto fetch = [&](int slot, uint32_t i) {       // i = index of the row inside this wave's row set
+        const uint32_t r = (uint32_t)rset * per_set + i;
+        const bool ok = lane_ok && i < per_set && r < n_rows;
+        const uint64_t blk = (uint64_t)(row0 + r) * nb + blk_col;
+        wide_load<QT>(q[0][slot], a.w, blk, ok);
+        if constexpr (NMAT == 2) wide_load<QT>(q[1][slot], a.w1, blk, ok);
+    };
+#pragma unroll
+    for (int i = 0; i < DEPTH; i++) fetch(i, i);
+    __syncthreads();
+    float xr[32], xsum = 0.f;
+    {
+        const float4 *src = reinterpret_cast<const float4 *>(xs + (size_t)(lane_ok ? blk_col : 0) * 32);
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            float4 v = src[j];
+            if (!lane_ok) v = make_float4(0.f, 0.f, 0.f, 0.f);
+            xr[4 * j] = v.x; xr[4 * j + 1] = v.y; xr[4 * j + 2] = v.z; xr[4 * j + 3] = v.w;
+            xsum += (v.x + v.y) + (v.z + v.w);
+        }
+    }
+
+    // ---- rows, DEPTH per turn of the queue, reduced four at a time ---------------------------------------------------
+    const uint32_t per_set_q = (per_set + DEPTH - 1) / DEPTH * DEPTH;
+    for (uint32_t i0 = 0; i0 < per_set_q; i0 += DEPTH) {
+#pragma unroll
+        for (int g = 0; g < DEPTH; g += 4) {
+            float p[NMAT][4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+#pragma unroll
+                for (int mi = 0; mi < NMAT; mi++) p[mi][j] = wide_dot<QT>(q[mi][g + j], xr, xsum);
+                fetch(g + j, i0 + g + j + DEPTH);
+            }
+#pragma unroll
+            for (int mi = 0; mi < NMAT; mi++) {
+                const float s = quad_partials_sum(p[mi][0], p[mi][1], p[mi][2], p[mi][3]);
+                const uint32_t i = i0 + g + quad_partial_of_lane(lane);
+                if (active && (lane & 15) == 0 && i < per_set) red[(((size_t)rset * per_set + i) * NMAT + mi) * NS + slab] = s;
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- combine the slabs, write ---------------------------------------------------------------------------------------
+    for (uint32_t r = threadIdx.x; r < n_rows; r += NW * 64) {
+        // row r of the workgroup lives in row set r / per_set at index r % per_set: the same slot as above
+        float v[NMAT];
+#pragma unroll
+        for (int mi = 0; mi < NMAT; mi++) {
+            float t = 0.f;
+            for (int s = 0; s < NS; s++) t += red[((size_t)r * NMAT + mi) * NS + s];
+            v[mi] = t;
+        }
+        float *o = a.out + (size_t)z * N + row0 + r;
+        if constexpr (MODE == kGemvStore) *o = v[0];
+        else if constexpr (MODE == kGemvAdd) *o += v[0];
+        else *o = v[0] * v[NMAT - 1] / (__expf(-v[NMAT - 1]) + 1.f);
+    }
+}
+
+}  // namespace lv

@@ -83,7 +83,7 @@ def copy_case(ctx):
 
 def model_file(preset, wtype, seed):
     base = "/dev/shm" if os.access("/dev/shm", os.W_OK) else "/tmp"
-XX
+    path = os.path.join(base, f"llava_measure_{preset}_{'q4_0' if wtype == lva.LV_Q4_0 else 'q8_0'}_seed{seed}.ggml")
     if not os.path.exists(path):
         lva.write_model(path + ".tmp", wtype=wtype, seed=seed, **SHAPES[preset])
         os.replace(path + ".tmp", path)

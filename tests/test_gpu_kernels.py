@@ -46,6 +46,9 @@ def test_dequant_bit_exact(lva, orc, ctx, ftype_name, rows, cols):
 @pytest.mark.parametrize("ftype_name", ["q4_0", "q8_0"])
 @pytest.mark.parametrize("rows,cols,batch", [
     (64, 4096, 1), (40, 11008, 1), (48, 5120, 1), (24, 13824, 1), (37, 96, 3), (8, 32, 2), (19, 2048 + 64, 1), (256, 256, 1),
+    # 2048 rows and more: the streaming kernel (256 workgroups, x in LDS); ragged row counts, 1..12 column slabs per
+    # row (24576 columns is the widest row the library accepts)
+    (2048, 32, 1), (2049, 2048 + 64, 2), (4096, 4096, 1), (2500, 11008, 1), (2051, 13824, 3), (2048, 24576, 1),
 ])
 @pytest.mark.parametrize("accumulate", [False, True])
 def test_gemv_matches_oracle(lva, orc, ctx, ftype_name, rows, cols, batch, accumulate):
@@ -68,7 +71,7 @@ def test_gemv_matches_oracle(lva, orc, ctx, ftype_name, rows, cols, batch, accum
 
 
 @pytest.mark.parametrize("ftype_name", ["q4_0", "q8_0"])
-@pytest.mark.parametrize("rows,cols,batch", [(96, 4096, 1), (64, 5120, 1), (50, 256, 2)])
+@pytest.mark.parametrize("rows,cols,batch", [(96, 4096, 1), (64, 5120, 1), (50, 256, 2), (11008, 4096, 1), (2077, 5120, 2), (2048, 96, 1)])
 def test_gemv_silu_matches_oracle(lva, orc, ctx, ftype_name, rows, cols, batch):
     ftype = lva.LV_Q4_0 if ftype_name == "q4_0" else lva.LV_Q8_0
     w3 = lva.synth_quant(ftype, rows, cols, seed=31, tensor_id=3)
