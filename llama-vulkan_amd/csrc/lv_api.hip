@@ -101,10 +101,14 @@ struct lv_model {
 };
 
 // Shape classes the persistent kernel is compiled for: LLaMA-7B and LLaMA-13B layer shapes, q4_0 and q8_0.
-using Mega7Bq4 = MegaShape<4096, 11008, 32, 12, 4>;
-using Mega7Bq8 = MegaShape<4096, 11008, 32, 12, 8>;
-using Mega13Bq4 = MegaShape<5120, 13824, 40, 12, 4>;
-using Mega13Bq8 = MegaShape<5120, 13824, 40, 12, 8>;
+// Wavefronts per workgroup and queue depth per shape class, measured (tok/s at 12 waves with the shallow queue the
+// register file then allows -> as below): 7B q4_0 845 -> 897, 7B q8_0 469 -> 538, 13B q4_0 462 -> 499, 13B q8_0
+// 286 -> 322.  Two waves per SIMD leave each wave 256 registers, which buys the deeper queue; the 13B shapes have three
+// column slabs in the D-wide phases and seven in the F-wide one, so seven waves keep all but one busy everywhere.
+using Mega7Bq4 = MegaShape<4096, 11008, 32, 8, 4, 8>;
+using Mega7Bq8 = MegaShape<4096, 11008, 32, 8, 8, 4>;
+using Mega13Bq4 = MegaShape<5120, 13824, 40, 7, 4, 8>;
+using Mega13Bq8 = MegaShape<5120, 13824, 40, 7, 8, 4>;
 
 template <class Fn>
 static int mega_dispatch(int kind, Fn &&fn)

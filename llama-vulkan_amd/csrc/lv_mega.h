@@ -3,7 +3,7 @@
 // Why: at batch 1 a layer is five tiny dependent GEMVs (1-6 us of HBM time each).  Launched one by one
 // they spend more time draining, launching and refilling the memory pipeline than streaming weights.
 // Here one workgroup per CU stays resident for the whole token; every wavefront walks its own contiguous
-// weight stream with a register queue (4 q4_0 tiles or 2 q8_0 tiles deep) of 128-bit loads that keeps running across the phase
+// weight stream with a register queue (8 q4_0 tiles or 4 q8_0 tiles deep) of 128-bit loads that keeps running across the phase
 // boundaries, so HBM stays busy while the workgroups exchange the small activation vectors.
 //
 // Phases of a layer (llava_layer.cpp:53-73), each separated by a data hand-over through HBM/L2:
@@ -35,6 +35,11 @@ constexpr uint32_t kNotReady = 0xFFFFFFFFu;
 constexpr int kMegaWGs = 256;
 constexpr int kMegaVocabRows = 125;     // output-matrix rows per workgroup the head phase is laid out for (32000 / 256)
 constexpr uint32_t kSpinLimit = 1u << 20;
+// A consumer reaches a hand-over about when its producers store: a load issued at once samples memory before the
+// stores are visible (0.6 us) yet comes back only after the prefetched tiles ahead of it on the CU's return path
+// (1-2 us), and the second try pays that again.  Sleeping this many 64-clock units first makes the first try
+// succeed; measured optimum, flat between 16 and 32.
+constexpr int kPollDelay = 24;
 
 __device__ __forceinline__ uint32_t ld_dev(const uint32_t *p)
 {
@@ -61,13 +66,13 @@ constexpr int cdiv(int a, int b) { return (a + b - 1) / b; }
 constexpr int round_up(int a, int b) { return cdiv(a, b) * b; }
 
 // Static shape of one model class.  NW = wavefronts per workgroup.
-template <int D_, int F_, int H_, int NW_, int QT_>
+template <int D_, int F_, int H_, int NW_, int QT_, int DEPTH_ = 0>
 struct MegaShape {
     static constexpr int D = D_, F = F_, H = H_, NW = NW_, R = 128;
     static constexpr int QT = QT_;                               // 4: q4_0, 8: q8_0
     static constexpr int CODE = QT == 4 ? 16 : 32;               // bytes of codes per block
     static constexpr int TILE = 64 * CODE + 128;                 // bytes per tile: 64 blocks of codes, 64 fp16 scales
-    static constexpr int DEPTH = QT == 4 ? 4 : 2;                // tiles in flight per wave (about 4.5 KB either way)
+    static constexpr int DEPTH = DEPTH_ ? DEPTH_ : (QT == 4 ? 4 : 2);   // tiles in flight per wave
     static constexpr int NBD = D / 32, NBF = F / 32;            // blocks per row
     static constexpr int NSD = cdiv(NBD, 64), NSF = cdiv(NBF, 64);  // column slabs
     static constexpr int NRD = NW / NSD, NRF = NW / NSF;        // row sets (waves sharing a slab split the rows)
@@ -144,12 +149,13 @@ __device__ __forceinline__ float tile_dot(const MegaTile &t, const float (&xr)[3
 
 // ---- polling helpers ----------------------------------------------------------------------------------------
 // N values strided by `stride` elements starting at p; spins until none of them is the not-ready pattern.
-template <int N>
+template <int N, int SLEEP = 0>
 __device__ __forceinline__ void poll_values(float (&v)[N], const float *p, int stride, const bool (&want)[N], uint32_t *status,
                                             int group_stride = 0 /* when non-zero: element j lives at p[(j/8)*8*group_stride + j%8] */)
 {
     uint32_t spins = 0;
     bool pending;
+    if constexpr (SLEEP > 0) __builtin_amdgcn_s_sleep(SLEEP);
     do {
         pending = false;
 #pragma unroll
@@ -319,7 +325,7 @@ __device__ __forceinline__ float block_sum(float v, float *scratch /* NW floats 
 // Brings the N-float vector at `src` (being produced by other workgroups) into LDS, optionally normalised
 // (normalize.comp:34-64: mean, then mean-centred variance, no epsilon) with weights w.  One round trip to
 // memory when the data is there: the norm weights are requested before the wait, not after it.
-template <int N, int NW, bool NORM>
+template <int N, int NW, bool NORM, int SLEEP = 0>
 __device__ __forceinline__ void acquire_vector(float *xs, const float *src, const float *w, float *scratch, uint32_t *status)
 {
     constexpr int T = NW * 64, PER = cdiv(N, T);
@@ -332,7 +338,7 @@ __device__ __forceinline__ void acquire_vector(float *xs, const float *src, cons
 #pragma unroll
         for (int j = 0; j < PER; j++) wn[j] = want[j] ? w[threadIdx.x + j * T] : 0.f;
     }
-    poll_values<PER>(v, src + threadIdx.x, T, want, status);
+    poll_values<PER, SLEEP>(v, src + threadIdx.x, T, want, status);
     if constexpr (NORM) {
         float s = 0.f;
 #pragma unroll
@@ -400,7 +406,7 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
 
         // ================= A: norm + QKV ====================================================================
         MEGA_STAMP(0);
-        acquire_vector<D, NW, true>(xs, x_src, norm_w, scratch, status);
+        acquire_vector<D, NW, true, kPollDelay>(xs, x_src, norm_w, scratch, status);
         MEGA_STAMP(1);
         load_slab(xr, xsum, xs, mw.sD * 64 + lane, mw.laneD);
         gemv_phase<S, S::SEQ_A, S::TA, S::NSD>(q, mw, layer, xr, xsum, mw.sD, mw.rD, mw.actD, S::ROWS_A, red);
@@ -459,7 +465,7 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
                     bool want24[24];
 #pragma unroll
                     for (int i = 0; i < 24; i++) want24[i] = i < 8 || newest;
-                    poll_values<24>(qkv, xc + S::OFF_QKV + h * R + sub * 8, 1, want24, status, D / 8);
+                    poll_values<24, kPollDelay>(qkv, xc + S::OFF_QKV + h * R + sub * 8, 1, want24, status, D / 8);
                 }
                 MEGA_STAMP(3);
                 const float scale = rsqrtf((float)R);
@@ -567,7 +573,7 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
 
         // ================= C: x += Wo o ============================================================================
         MEGA_STAMP(5);
-        acquire_vector<D, NW, false>(xs, xc + S::OFF_O, nullptr, scratch, status);
+        acquire_vector<D, NW, false, kPollDelay>(xs, xc + S::OFF_O, nullptr, scratch, status);
         MEGA_STAMP(6);
         load_slab(xr, xsum, xs, mw.sD * 64 + lane, mw.laneD);
         gemv_phase<S, S::SEQ_C, S::TC, S::NSD>(q, mw, layer, xr, xsum, mw.sD, mw.rD, mw.actD, S::ROWS_C, red);
@@ -580,7 +586,7 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
 
         // ================= D: norm + SwiGLU ========================================================================
         MEGA_STAMP(7);
-        acquire_vector<D, NW, true>(xs, xc + S::OFF_X1, norm_w + D, scratch, status);
+        acquire_vector<D, NW, true, kPollDelay>(xs, xc + S::OFF_X1, norm_w + D, scratch, status);
         MEGA_STAMP(8);
         load_slab(xr, xsum, xs, mw.sD * 64 + lane, mw.laneD);
         gemv_phase<S, S::SEQ_D, S::TD, S::NSD>(q, mw, layer, xr, xsum, mw.sD, mw.rD, mw.actD, S::ROWS_D, red);
@@ -593,7 +599,7 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
 
         // ================= E: x += W2 ff ===========================================================================
         MEGA_STAMP(9);
-        acquire_vector<F, NW, false>(xs, xc + S::OFF_FF, nullptr, scratch, status);
+        acquire_vector<F, NW, false, kPollDelay>(xs, xc + S::OFF_FF, nullptr, scratch, status);
         MEGA_STAMP(10);
         load_slab(xr, xsum, xs, mw.sF * 64 + lane, mw.laneF);
         gemv_phase<S, S::SEQ_E, S::TE, S::NSF>(q, mw, layer, xr, xsum, mw.sF, mw.rF, mw.actF, S::ROWS_E, red);
@@ -612,7 +618,7 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
 
     // ================= head: norm + output matrix ====================================================================
     {
-        acquire_vector<D, NW, true>(xs, x_src, a.norms + (size_t)a.layers * 2 * D, scratch, status);
+        acquire_vector<D, NW, true, kPollDelay>(xs, x_src, a.norms + (size_t)a.layers * 2 * D, scratch, status);
         load_slab(xr, xsum, xs, mw.sD * 64 + lane, mw.laneD);
         const int rows = (int)mw.vocab_rows, per_set = (rows + S::NRD - 1) / S::NRD;
         // the head's slots are numbered from 0; tiles beyond per_set read the dummy tile
