@@ -101,7 +101,7 @@ def main():
     t0 = time.perf_counter()
     for _ in range(args.steps):
         sess.begin([tok], pos)
-        tok = sess.argmax()          # device argmax + 4-byte read back: the sampler is inside the step
+        tok = sess.argmax()          # the kernel leaves its greedy pick in pinned memory: the sampler is inside the step
         tokens.append(tok)
         pos += 1
     sess.wait()

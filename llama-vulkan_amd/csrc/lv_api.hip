@@ -150,7 +150,8 @@ struct lv_session {
     uint16_t *pf_xh = nullptr, *pf_xl = nullptr;
     float *xchg[2] = {nullptr, nullptr};  // hand-over buffer sets of the persistent kernel
     uint32_t xchg_turn = 0;
-    uint32_t *status_host = nullptr;      // pinned, written by the persistent kernel when a poll expires
+    uint32_t *status_host = nullptr;      // pinned, written by the persistent kernel: [0] a poll expired, [kStatusToken] greedy pick
+    bool pick_in_status = false;          // the last step ran the persistent kernel, whose greedy pick is in status_host
     bool in_flight = false;
     bool have_logits = false;
     bool trace = false;
@@ -601,7 +602,7 @@ static int launch_split(hipStream_t st, uint16_t *xh, uint16_t *xl, const float 
 static int launch_gemm(hipStream_t st, float *out, uint32_t ldo, const lv_matrix &w, const float *x, uint32_t n, uint16_t *xh, uint16_t *xl,
                        bool accumulate)
 {
-    const uint32_t K = w.view.cols, n_pad = (n + kGemmTile - 1) / kGemmTile * kGemmTile;
+    const uint32_t K = w.view.cols;
     if (K % 32) return fail(LV_ERR_ARG, "gemm: %u columns", K);
     LV_TRY(launch_split(st, xh, xl, x, n, K, w.ftype));
     return launch_gemm_presplit(st, out, ldo, w, n, xh, xl, accumulate);
@@ -983,7 +984,7 @@ static int session_alloc(lv_session *s)
     if (s->model->mega_kind) {
         size_t bytes = 0;
         LV_TRY(mega_dispatch(s->model->mega_kind, [&](auto shape) -> int {
-            bytes = (size_t)hp.layers * decltype(shape)::XCHG_LAYER * 4;
+            bytes = ((size_t)hp.layers * decltype(shape)::XCHG_LAYER + decltype(shape)::XCHG_TAIL) * 4;
             return LV_OK;
         }));
         for (int i = 0; i < 2; i++) {
@@ -1280,15 +1281,20 @@ extern "C" int lv_step_begin(lv_session *s, const uint32_t *tokens, uint32_t n, 
         if (tokens[i] >= s->model->hp.vocab) return fail(LV_ERR_RANGE, "lv_step_begin: token id %u of a vocabulary of %u", tokens[i], s->model->hp.vocab);
     HIP_TRY(hipSetDevice(s->model->ctx->device));
 
-    s->cfg_host[0] = pos;
-    memcpy(s->cfg_host + 1, tokens, (size_t)n * 4);
-    HIP_TRY(hipMemcpyAsync(s->cfg, s->cfg_host, (size_t)(1 + n) * 4, hipMemcpyHostToDevice, s->stream));
     s->have_logits = false;
+    s->pick_in_status = false;
 
     int path = LV_PATH_AUTO;
     (void)lv_session_path(s, &path);
-    if (n == 1 && path == LV_PATH_PERSISTENT && !s->trace) {
+    const bool persistent = n == 1 && path == LV_PATH_PERSISTENT && !s->trace;
+    if (!persistent) {             // the persistent kernel takes position and token id as launch arguments
+        s->cfg_host[0] = pos;
+        memcpy(s->cfg_host + 1, tokens, (size_t)n * 4);
+        HIP_TRY(hipMemcpyAsync(s->cfg, s->cfg_host, (size_t)(1 + n) * 4, hipMemcpyHostToDevice, s->stream));
+    }
+    if (persistent) {
         LV_TRY(launch_mega(s, pos, tokens[0]));
+        s->pick_in_status = true;  // the kernel leaves the greedy pick in the pinned status block
     } else if (n == 1 && (path == LV_PATH_GRAPH || (path == LV_PATH_PERSISTENT && s->use_graph)) && !s->trace) {
         if (!s->graph_exec) {
             HIP_TRY(hipStreamBeginCapture(s->stream, hipStreamCaptureModeThreadLocal));
@@ -1345,6 +1351,11 @@ extern "C" int lv_argmax(lv_session *s, uint32_t *token)
 {
     if (!s || !token) return fail(LV_ERR_ARG, "lv_argmax: null argument");
     if (!s->have_logits) return fail(LV_ERR_STATE, "lv_argmax: no step has produced logits");
+    if (s->pick_in_status) {
+        LV_TRY(lv_step_wait(s));
+        *token = s->status_host[kStatusToken];
+        return LV_OK;
+    }
     argmax_kernel<<<dim3(1), dim3(1024), 0, s->stream>>>(s->logits, s->model->hp.vocab, s->argmax_dev);
     HIP_TRY(hipGetLastError());
     HIP_TRY(hipMemcpyAsync(s->argmax_host, s->argmax_dev, 4, hipMemcpyDeviceToHost, s->stream));

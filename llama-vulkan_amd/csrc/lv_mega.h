@@ -35,6 +35,7 @@ constexpr uint32_t kNotReady = 0xFFFFFFFFu;
 constexpr int kMegaWGs = 256;
 constexpr int kMegaVocabRows = 125;     // output-matrix rows per workgroup the head phase is laid out for (32000 / 256)
 constexpr uint32_t kSpinLimit = 1u << 20;
+constexpr int kStatusToken = 2;         // word of the status block that receives the index of the largest logit
 // A consumer reaches a hand-over about when its producers store: a load issued at once samples memory before the
 // stores are visible (0.6 us) yet comes back only after the prefetched tiles ahead of it on the CU's return path
 // (1-2 us), and the second try pays that again.  Sleeping this many 64-clock units first makes the first try
@@ -86,6 +87,7 @@ struct MegaShape {
     // floats of one layer's hand-over buffers
     static constexpr int OFF_QKV = 0, OFF_PART = 3 * D, OFF_O = OFF_PART + H * CPH * PART, OFF_X1 = OFF_O + D,
                          OFF_FF = OFF_X1 + D, OFF_X2 = OFF_FF + F, XCHG_LAYER = OFF_X2 + D;
+    static constexpr int XCHG_TAIL = 2 * kMegaWGs;              // after the layers: every workgroup's best logit (value, index)
     static_assert((3 * D) % kMegaWGs == 0 && (2 * F) % kMegaWGs == 0 && D % kMegaWGs == 0, "rows must split over 256 workgroups");
     static_assert(H * R == D && CPH >= 1 && NRD >= 1 && NRF >= 1, "shape");
     // bytes of the weight stream of one layer
@@ -101,10 +103,10 @@ struct MegaArgs {
     const float *tok_f32;      // embedding table [vocab][D] (fp32)
     uint16_t *kv;              // [layers][2][backlog][D] fp16
     const float2 *trig;        // [backlog][64]
-    float *xchg;               // this token's hand-over buffers: [layers] x XCHG_LAYER floats, all kNotReady
+    float *xchg;               // this token's hand-over buffers: [layers] x XCHG_LAYER + XCHG_TAIL floats, all kNotReady
     float *xchg_rearm;         // the other set, re-armed to kNotReady during this token
     float *logits;             // [vocab]
-    uint32_t *status;          // host-visible; set non-zero when a poll loop expired
+    uint32_t *status;          // host-visible; [0] set non-zero when a poll loop expired, [kStatusToken] = greedy pick
     uint32_t layers, vocab, backlog, pos, token;
 };
 
@@ -385,7 +387,7 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
     // ---- re-arm the other buffer set for the next token ---------------------------------------------------------
 #ifndef LV_MEGA_NOWAIT   // (experiment builds leave stale, "ready" data in place to time the kernel without hand-over waits)
     {
-        const size_t n4 = (size_t)a.layers * S::XCHG_LAYER / 4;
+        const size_t n4 = ((size_t)a.layers * S::XCHG_LAYER + S::XCHG_TAIL) / 4;
         uint4 *dst = reinterpret_cast<uint4 *>(a.xchg_rearm);
         for (size_t i = (size_t)b * T + threadIdx.x; i < n4; i += (size_t)kMegaWGs * T)
             dst[i] = make_uint4(kNotReady, kNotReady, kNotReady, kNotReady);
@@ -637,9 +639,60 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
             }
         }
         lds_barrier();
+        // logits out; on the way the greedy pick (llava_session.cpp:144-152: index of the first strict maximum):
+        // every workgroup hands its best (value, index) to workgroup 0 like any other hand-over
+        float bv = -INFINITY;
+        uint32_t bi = kNotReady;
+        auto better = [](float ov, uint32_t oi, float mv, uint32_t mi) {
+            return oi != kNotReady && (mi == kNotReady || ov > mv || (ov == mv && oi < mi));
+        };
         for (int j = st; j < rows; j += T) {
             const uint32_t n = (uint32_t)b * rows + j;
-            if (n < a.vocab) a.logits[n] = red_row<S::NSD>(red, j);
+            if (n < a.vocab) {
+                const float v = red_row<S::NSD>(red, j);
+                a.logits[n] = v;
+                if (better(v, n, bv, bi)) { bv = v; bi = n; }
+            }
+        }
+        auto block_best = [&]() {          // result in thread 0
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) {
+                const float ov = __shfl_xor(bv, off, kWave);
+                const uint32_t oi = __shfl_xor(bi, off, kWave);
+                if (better(ov, oi, bv, bi)) { bv = ov; bi = oi; }
+            }
+            if (lane == 0) { scratch[w] = bv; scratch[NW + w] = __uint_as_float(bi); }
+            lds_barrier();
+            if (st == 0) {
+#pragma unroll
+                for (int i = 1; i < NW; i++) {
+                    const float ov = scratch[i];
+                    const uint32_t oi = __float_as_uint(scratch[NW + i]);
+                    if (better(ov, oi, bv, bi)) { bv = ov; bi = oi; }
+                }
+            }
+        };
+        block_best();
+        float *cand = a.xchg + (size_t)a.layers * S::XCHG_LAYER;
+        if (st == 0) {
+            // neither word may look like "not written yet": an all-ones NaN becomes the default NaN, a workgroup
+            // without rows reports index 0xFFFFFFFE
+            st_dev(cand + 2 * b, __float_as_uint(bv) == kNotReady ? __uint_as_float(0x7fc00000u) : bv);
+            st_dev(cand + 2 * b + 1, __uint_as_float(bi == kNotReady ? kNotReady - 1 : bi));
+        }
+        if (b == 0) {
+            lds_barrier();                 // thread 0 has read the scratch words of the first reduction
+            bv = -INFINITY;
+            bi = kNotReady;
+            if (st < kMegaWGs) {
+                float pair[2];
+                const bool want2[2] = {true, true};
+                poll_values<2, kPollDelay>(pair, cand + 2 * st, 1, want2, status);
+                const uint32_t oi = __float_as_uint(pair[1]);
+                if (oi < kNotReady - 1) { bv = pair[0]; bi = oi; }
+            }
+            block_best();
+            if (st == 0) status[kStatusToken] = bi == kNotReady ? 0u : bi;
         }
     }
 #ifdef LV_MEGA_TIMING
