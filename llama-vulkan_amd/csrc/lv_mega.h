@@ -437,7 +437,7 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
                 const uint32_t p_begin = min((uint32_t)c * chunk, n_valid), p_end = min(p_begin + chunk, n_valid);
                 const int sub = lane & 15, rsel = w * 4 + (lane >> 4);
                 constexpr int RPR = NW * 4;   // cache rows per round of the workgroup
-                constexpr int PRE = 2;        // rounds whose K, V and rotation rows are requested before the query arrives
+                constexpr int PRE = 2;        // rounds of K, V and rotation rows in flight (3 and 4 measured: no faster)
                 const size_t row_off = (size_t)h * R + sub * 8;
                 auto unpack8 = [](float (&f)[8], const uint4 &raw) {
                     const uint32_t wv[4] = {raw.x, raw.y, raw.z, raw.w};
@@ -447,19 +447,22 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
                         f[2 * i + 1] = half_bits_to_float((uint16_t)(wv[i] >> 16));
                     }
                 };
-                // Rows older than this token do not depend on it: ask for them first, then wait for q.
+                // Rows older than this token do not depend on it: ask for the first rounds, then wait for q.  The
+                // rounds form a queue PRE deep: a slot is refilled with the round PRE further on as soon as it is
+                // used (rounds past the end of the chunk read row 0 and are masked).
                 uint4 kpre[PRE], vpre[PRE];
                 float4 tpre[PRE][2];
-#pragma unroll
-                for (int r = 0; r < PRE; r++) {
-                    const uint32_t p = p_begin + r * RPR + rsel;
+                auto request_round = [&](int slot, uint32_t p0) {
+                    const uint32_t p = p0 + rsel;
                     const uint32_t pc = (p < p_end && p != pos) ? p : 0;  // any valid row; unused when masked
-                    kpre[r] = *reinterpret_cast<const uint4 *>(kc + (size_t)pc * D + row_off);
-                    vpre[r] = *reinterpret_cast<const uint4 *>(vc + (size_t)pc * D + row_off);
+                    kpre[slot] = *reinterpret_cast<const uint4 *>(kc + (size_t)pc * D + row_off);
+                    vpre[slot] = *reinterpret_cast<const uint4 *>(vc + (size_t)pc * D + row_off);
                     const float4 *tp = reinterpret_cast<const float4 *>(a.trig + (size_t)(p < p_end ? pos - p : 0) * (R / 2) + sub * 4);
-                    tpre[r][0] = tp[0];
-                    tpre[r][1] = tp[1];
-                }
+                    tpre[slot][0] = tp[0];
+                    tpre[slot][1] = tp[1];
+                };
+#pragma unroll
+                for (int r = 0; r < PRE; r++) request_round(r, p_begin + r * RPR);
                 // one wait for the query and, in the lanes that own the newest position, its K and V row
                 const bool newest = (pos >= p_begin && pos < p_end) && ((pos - p_begin) % RPR) == (uint32_t)rsel;
                 float qkv[24];
@@ -511,18 +514,13 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
                     }
                 };
                 // a row's weight is computed and used by the same 16 lanes: no exchange through LDS, no barrier
+                for (uint32_t p0 = p_begin; p0 < p_end; p0 += PRE * RPR) {
 #pragma unroll
-                for (int r = 0; r < PRE; r++) {
-                    const uint32_t p = p_begin + r * RPR + rsel;
-                    add_row(p, weight_of(p, kpre[r], tpre[r][0], tpre[r][1]), vpre[r]);
-                }
-                for (uint32_t p0 = p_begin + PRE * RPR; p0 < p_end; p0 += RPR) {
-                    const uint32_t p = p0 + rsel;
-                    const uint32_t pc = (p < p_end && p != pos) ? p : 0;
-                    const float4 *tp = reinterpret_cast<const float4 *>(a.trig + (size_t)(p < p_end ? pos - p : 0) * (R / 2) + sub * 4);
-                    const uint4 kraw = *reinterpret_cast<const uint4 *>(kc + (size_t)pc * D + row_off);
-                    const uint4 vraw = *reinterpret_cast<const uint4 *>(vc + (size_t)pc * D + row_off);
-                    add_row(p, weight_of(p, kraw, tp[0], tp[1]), vraw);
+                    for (int r = 0; r < PRE; r++) {
+                        const uint32_t p = p0 + r * RPR + rsel;
+                        add_row(p, weight_of(p, kpre[r], tpre[r][0], tpre[r][1]), vpre[r]);
+                        if (p0 + (r + PRE) * RPR < p_end) request_round(r, p0 + (r + PRE) * RPR);   // uniform condition
+                    }
                 }
 #pragma unroll
                 for (int off = 16; off < 64; off <<= 1) {
