@@ -122,7 +122,7 @@ static int mega_dispatch(int kind, Fn &&fn)
     }
 }
 
-constexpr uint32_t kAttnChunk = 64;   // cache positions per attention workgroup
+constexpr uint32_t kAttnChunk = kAttnChunkRows;   // cache positions per attention workgroup
 constexpr uint32_t kMaxStepTokens = 4096;
 
 struct lv_session {
@@ -497,7 +497,7 @@ static int launch_attention(hipStream_t st, float *out, const uint16_t *kc, cons
     a.pos_ptr = pos_ptr; a.pos_add = pos_add; a.heads = heads; a.backlog = backlog; a.chunk = kAttnChunk;
     a.splits = (backlog + kAttnChunk - 1) / kAttnChunk;
     const dim3 grid(heads, a.splits, batch);
-    const size_t lds = sizeof(float) * (kAttnChunk + 4 * (rot + 1));
+    const size_t lds = sizeof(float) * 4 * (rot + 1);
     switch (rot) {
     case 32: attention_kernel<32><<<grid, dim3(256), lds, st>>>(a); break;
     case 64: attention_kernel<64><<<grid, dim3(256), lds, st>>>(a); break;
@@ -1162,8 +1162,7 @@ static int record_token(lv_session *s, uint32_t idx, bool with_head)
         LV_TRY(launch_gemv(st, s->k, lw.wk, nullptr, s->xn, 1, kGemvStore));
         LV_TRY(launch_gemv(st, s->q, lw.wq, nullptr, s->xn, 1, kGemvStore));
         LV_TRY(launch_gemv(st, s->v, lw.wv, nullptr, s->xn, 1, kGemvStore));
-        kv_append_kernel<<<kv_grid, dim3(256), 0, st>>>(kv_ptr(s, li, 0), s->k, pos_ptr, idx, D, s->backlog);
-        kv_append_kernel<<<kv_grid, dim3(256), 0, st>>>(kv_ptr(s, li, 1), s->v, pos_ptr, idx, D, s->backlog);
+        kv_append2_kernel<<<dim3(kv_grid.x, kv_grid.y, 2), dim3(256), 0, st>>>(kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->k, s->v, pos_ptr, idx, D, s->backlog);
         HIP_TRY(hipGetLastError());
         LV_TRY(launch_attention(st, s->vo, kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->q, s->trig, s->attn_part, s->attn_counters,
                                 pos_ptr, idx, s->backlog, hp.heads, hp.rot, 1));
@@ -1242,8 +1241,7 @@ static int record_prefill(lv_session *s, uint32_t idx0, uint32_t n, bool with_he
         else LV_TRY(launch_gemm(st, s->pf_k, D, lw.wk, s->pf_xn, n, s->pf_xh, s->pf_xl, false));
         if (lw.wv.ftype == lw.wk.ftype) LV_TRY(launch_gemm_presplit(st, s->pf_v, D, lw.wv, n, s->pf_xh, s->pf_xl, false));
         else LV_TRY(launch_gemm(st, s->pf_v, D, lw.wv, s->pf_xn, n, s->pf_xh, s->pf_xl, false));
-        kv_append_kernel<<<kv_grid, dim3(256), 0, st>>>(kv_ptr(s, li, 0), s->pf_k, pos_ptr, idx0, D, s->backlog);
-        kv_append_kernel<<<kv_grid, dim3(256), 0, st>>>(kv_ptr(s, li, 1), s->pf_v, pos_ptr, idx0, D, s->backlog);
+        kv_append2_kernel<<<dim3(kv_grid.x, kv_grid.y, 2), dim3(256), 0, st>>>(kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->pf_k, s->pf_v, pos_ptr, idx0, D, s->backlog);
         HIP_TRY(hipGetLastError());
         LV_TRY(launch_attention_batch(st, s->pf_vo, kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->pf_q, s->trig, pos_ptr, idx0, n, s->backlog,
                                       hp.heads, hp.rot));

@@ -204,12 +204,47 @@ __device__ __forceinline__ float block_sum_256(float v, float *lds /* >= 4 float
     return (lds[0] + lds[1]) + (lds[2] + lds[3]);
 }
 
+// The row is read once, as 128-bit loads that are all in flight together, and kept in registers for the three passes
+// (up to 8192 floats, a multiple of 4); longer or odd rows walk memory three times.
 __global__ __launch_bounds__(256) void normalize_kernel(float *__restrict__ out, const float *__restrict__ x,
                                                         const float *__restrict__ w, uint32_t dim)
 {
     __shared__ float lds[4];
     const float *xr = x + (size_t)blockIdx.x * dim;
     float *outr = out + (size_t)blockIdx.x * dim;
+    if (dim <= 8192 && dim % 4 == 0) {
+        constexpr int PER = 8;
+        const uint32_t n4 = dim / 4;
+        float4 v[PER], wv[PER];
+#pragma unroll
+        for (int j = 0; j < PER; j++) {
+            const uint32_t i = threadIdx.x + j * 256;
+            const bool ok = i < n4;
+            v[j] = ok ? reinterpret_cast<const float4 *>(xr)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+            wv[j] = ok ? reinterpret_cast<const float4 *>(w)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+        float s = 0.f;
+#pragma unroll
+        for (int j = 0; j < PER; j++) s += (v[j].x + v[j].y) + (v[j].z + v[j].w);
+        const float mean = block_sum_256(s, lds) / (float)dim;
+        float q = 0.f;
+#pragma unroll
+        for (int j = 0; j < PER; j++) {
+            if (threadIdx.x + j * 256 < n4) {
+                const float c0 = v[j].x - mean, c1 = v[j].y - mean, c2 = v[j].z - mean, c3 = v[j].w - mean;
+                q = fmaf(c0, c0, q); q = fmaf(c1, c1, q); q = fmaf(c2, c2, q); q = fmaf(c3, c3, q);
+            }
+        }
+        const float inv = rsqrtf(block_sum_256(q, lds) / (float)dim);
+#pragma unroll
+        for (int j = 0; j < PER; j++) {
+            const uint32_t i = threadIdx.x + j * 256;
+            if (i < n4)
+                reinterpret_cast<float4 *>(outr)[i] = make_float4((v[j].x * wv[j].x) * inv, (v[j].y * wv[j].y) * inv, (v[j].z * wv[j].z) * inv,
+                                                                  (v[j].w * wv[j].w) * inv);
+        }
+        return;
+    }
     float s = 0.f;
     for (uint32_t i = threadIdx.x; i < dim; i += 256) s += xr[i];
     const float mean = block_sum_256(s, lds) / (float)dim;
@@ -231,6 +266,18 @@ __global__ void kv_append_kernel(uint16_t *__restrict__ cache, const float *__re
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
     const uint32_t z = blockIdx.y;
     const uint32_t row = (pos_ptr ? *pos_ptr : 0u) + pos_add + z;
+    if (i < dim && row < backlog) cache[(size_t)row * dim + i] = float_to_half_bits(in[(size_t)z * dim + i]);
+}
+
+// K and V rows of one layer in one launch (blockIdx.z: 0 = K, 1 = V)
+__global__ void kv_append2_kernel(uint16_t *__restrict__ kcache, uint16_t *__restrict__ vcache, const float *__restrict__ k_in,
+                                  const float *__restrict__ v_in, const uint32_t *pos_ptr, uint32_t pos_add, uint32_t dim, uint32_t backlog)
+{
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t z = blockIdx.y;
+    const uint32_t row = (pos_ptr ? *pos_ptr : 0u) + pos_add + z;
+    uint16_t *cache = blockIdx.z ? vcache : kcache;
+    const float *in = blockIdx.z ? v_in : k_in;
     if (i < dim && row < backlog) cache[(size_t)row * dim + i] = float_to_half_bits(in[(size_t)z * dim + i]);
 }
 
@@ -298,29 +345,44 @@ struct AttnArgs {
     uint32_t heads, backlog, chunk, splits;
 };
 
+constexpr int kAttnChunkRows = 64;       // cache positions per workgroup (AttnArgs::chunk must be this)
+
 template <int R>
 __global__ __launch_bounds__(256) void attention_kernel(AttnArgs a)
 {
     constexpr int LPR = R / 8;        // lanes per cache row
     constexpr int RPWV = 64 / LPR;    // rows per wave per load
-    constexpr int RPB = 4 * RPWV;     // rows per workgroup per load
+    constexpr int RPB = 4 * RPWV;     // rows per workgroup per round
+    constexpr int ROUNDS = kAttnChunkRows / RPB;
+    static_assert(ROUNDS >= 1 && ROUNDS * RPB == kAttnChunkRows, "chunk must be whole rounds");
     const uint32_t h = blockIdx.x, split = blockIdx.y, z = blockIdx.z;
     const uint32_t H = a.heads, D = H * R;
     const uint32_t cur = (a.pos_ptr ? *a.pos_ptr : 0u) + a.pos_add + z;  // this row's own cache position
     const uint32_t n_valid = min(cur + 1, a.backlog);
-    const uint32_t n_splits = (n_valid + a.chunk - 1) / a.chunk;         // splits that hold any position
+    const uint32_t n_splits = (n_valid + kAttnChunkRows - 1) / kAttnChunkRows;   // splits that hold any position
     if (split >= n_splits) return;
-    const uint32_t p_begin = split * a.chunk, p_end = min(p_begin + a.chunk, n_valid);
+    const uint32_t p_begin = split * kAttnChunkRows, p_end = min(p_begin + kAttnChunkRows, n_valid);
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int sub = lane % LPR;             // which 8 elements of the row
     const int rsel = wave * RPWV + lane / LPR;
 
-    extern __shared__ float lds[];          // e[chunk] then reduction scratch
-    float *e_lds = lds;
-    float *red = lds + a.chunk;             // [4][R+1]
+    extern __shared__ float lds[];
+    float *red = lds;                       // [4][R+1]
 
-    // this lane's 8 query values
+    // Every load of the chunk goes out before anything is used: K, V and rotation rows of all rounds, and the query.
+    uint4 kraw[ROUNDS], vraw[ROUNDS];
+    float4 t0[ROUNDS], t1[ROUNDS];
+#pragma unroll
+    for (int r = 0; r < ROUNDS; r++) {
+        const uint32_t p = p_begin + r * RPB + rsel;
+        const uint32_t pc = p < p_end ? p : p_begin;     // a valid row; its weight is forced to 0 below
+        kraw[r] = *reinterpret_cast<const uint4 *>(a.kcache + (size_t)pc * D + (size_t)h * R + sub * 8);
+        vraw[r] = *reinterpret_cast<const uint4 *>(a.vcache + (size_t)pc * D + (size_t)h * R + sub * 8);
+        const float4 *tp = reinterpret_cast<const float4 *>(a.trig + (size_t)(cur - pc) * (R / 2) + sub * 4);
+        t0[r] = tp[0];  // (c0,s0,c1,s1)
+        t1[r] = tp[1];  // (c2,s2,c3,s3)
+    }
     float qv[8];
     {
         const float4 *qp = reinterpret_cast<const float4 *>(a.q + (size_t)z * D + (size_t)h * R + sub * 8);
@@ -330,51 +392,33 @@ __global__ __launch_bounds__(256) void attention_kernel(AttnArgs a)
     }
     const float scale = rsqrtf((float)R);
 
-    // ---- scores -----------------------------------------------------------------------------------------
+    // A row's weight is computed and used by the same LPR lanes: no exchange through LDS between scores and P.V.
     float den = 0.f;
-    for (uint32_t p0 = p_begin; p0 < p_end; p0 += RPB) {
-        const uint32_t p = p0 + rsel;
-        float s = 0.f;
-        if (p < p_end) {
-            const uint4 kraw = *reinterpret_cast<const uint4 *>(a.kcache + (size_t)p * D + (size_t)h * R + sub * 8);
-            const float4 *tp = reinterpret_cast<const float4 *>(a.trig + (size_t)(cur - p) * (R / 2) + sub * 4);
-            const float4 t0 = tp[0], t1 = tp[1];  // (c0,s0,c1,s1), (c2,s2,c3,s3)
-            const uint32_t kw[4] = {kraw.x, kraw.y, kraw.z, kraw.w};
-            const float ct[4] = {t0.x, t0.z, t1.x, t1.z}, st[4] = {t0.y, t0.w, t1.y, t1.w};
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const float kx = half_bits_to_float((uint16_t)(kw[i] & 0xffffu));
-                const float ky = half_bits_to_float((uint16_t)(kw[i] >> 16));
-                const float qx = qv[2 * i], qy = qv[2 * i + 1];
-                const float dotp = fmaf(qy, ky, qx * kx);      // Q.K of the pair
-                const float crs = fmaf(qx, ky, -(qy * kx));    // Qx Ky - Qy Kx
-                s = fmaf(ct[i], dotp, s);
-                s = fmaf(st[i], crs, s);
-            }
+    for (int r = 0; r < ROUNDS; r++) {
+        const uint32_t p = p_begin + r * RPB + rsel;
+        const uint32_t kw[4] = {kraw[r].x, kraw[r].y, kraw[r].z, kraw[r].w};
+        const float ct[4] = {t0[r].x, t0[r].z, t1[r].x, t1[r].z}, st[4] = {t0[r].y, t0[r].w, t1[r].y, t1[r].w};
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float kx = half_bits_to_float((uint16_t)(kw[i] & 0xffffu));
+            const float ky = half_bits_to_float((uint16_t)(kw[i] >> 16));
+            const float qx = qv[2 * i], qy = qv[2 * i + 1];
+            const float dotp = fmaf(qy, ky, qx * kx);      // Q.K of the pair
+            const float crs = fmaf(qx, ky, -(qy * kx));    // Qx Ky - Qy Kx
+            s = fmaf(ct[i], dotp, s);
+            s = fmaf(st[i], crs, s);
         }
         s = group_sum<LPR>(s);
-        float e = 0.f;
-        if (p < p_end) {
-            e = __expf(s * scale);
-            if (sub == 0) e_lds[p - p_begin] = e;
-        }
+        const float e = p < p_end ? __expf(s * scale) : 0.f;
         den += (sub == 0) ? e : 0.f;
-    }
-    __syncthreads();
-
-    // ---- P.V --------------------------------------------------------------------------------------------
-    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    for (uint32_t p0 = p_begin; p0 < p_end; p0 += RPB) {
-        const uint32_t p = p0 + rsel;
-        if (p < p_end) {
-            const uint4 vraw = *reinterpret_cast<const uint4 *>(a.vcache + (size_t)p * D + (size_t)h * R + sub * 8);
-            const float e = e_lds[p - p_begin];
-            const uint32_t vw[4] = {vraw.x, vraw.y, vraw.z, vraw.w};
+        const uint32_t vw[4] = {vraw[r].x, vraw[r].y, vraw[r].z, vraw[r].w};
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                acc[2 * i] = fmaf(e, half_bits_to_float((uint16_t)(vw[i] & 0xffffu)), acc[2 * i]);
-                acc[2 * i + 1] = fmaf(e, half_bits_to_float((uint16_t)(vw[i] >> 16)), acc[2 * i + 1]);
-            }
+        for (int i = 0; i < 4; i++) {
+            acc[2 * i] = fmaf(e, half_bits_to_float((uint16_t)(vw[i] & 0xffffu)), acc[2 * i]);
+            acc[2 * i + 1] = fmaf(e, half_bits_to_float((uint16_t)(vw[i] >> 16)), acc[2 * i + 1]);
         }
     }
     // sum over the RPWV row groups of the wave (lanes with equal `sub`), then over the 4 waves via LDS
@@ -418,7 +462,14 @@ __global__ __launch_bounds__(256) void attention_kernel(AttnArgs a)
     const float *hp = a.part + ((size_t)z * H + h) * a.splits * (R + 1);
     if (threadIdx.x <= R) {
         float t = 0.f;
-        for (uint32_t s = 0; s < n_splits; s++) t += __builtin_nontemporal_load(hp + (size_t)s * (R + 1) + threadIdx.x);
+        for (uint32_t s0 = 0; s0 < n_splits; s0 += 8) {      // eight loads in flight, summed in split order
+            float v[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                v[j] = s0 + j < n_splits ? __builtin_nontemporal_load(hp + (size_t)(s0 + j) * (R + 1) + threadIdx.x) : 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; j++) t += v[j];
+        }
         red[threadIdx.x] = t;
     }
     __syncthreads();
