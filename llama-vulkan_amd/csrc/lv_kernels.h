@@ -442,7 +442,8 @@ __global__ __launch_bounds__(256) void attention_kernel(AttnArgs a)
         if (n_splits == 1) {
             red[c] = t;  // finished here: normalise below
         } else {
-            my_part[c] = t;
+            // write-through store at device scope: visible to every other workgroup once it is acknowledged
+            __hip_atomic_store(reinterpret_cast<uint32_t *>(my_part + c), __float_as_uint(t), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
     if (n_splits == 1) {
@@ -452,23 +453,27 @@ __global__ __launch_bounds__(256) void attention_kernel(AttnArgs a)
     }
 
     // ---- cross-workgroup combine: the last split to arrive sums all partials in split order ---------------
+    // Ordering without a release fence (which at device scope writes back the whole L2): the partials are
+    // write-through stores, the wave waits for their acknowledgement, then the workgroup counts itself in; the
+    // last workgroup reads the partials with device-scope loads, which do not hit stale lines.
     __shared__ uint32_t arrived;
-    __threadfence();
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    if (threadIdx.x == 0) arrived = atomicAdd(&a.counters[(size_t)z * H + h], 1u);
+    if (threadIdx.x == 0) arrived = __hip_atomic_fetch_add(&a.counters[(size_t)z * H + h], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (arrived != n_splits - 1) return;
-    __threadfence();
     const float *hp = a.part + ((size_t)z * H + h) * a.splits * (R + 1);
     if (threadIdx.x <= R) {
         float t = 0.f;
         for (uint32_t s0 = 0; s0 < n_splits; s0 += 8) {      // eight loads in flight, summed in split order
-            float v[8];
+            uint32_t v[8];
 #pragma unroll
             for (int j = 0; j < 8; j++)
-                v[j] = s0 + j < n_splits ? __builtin_nontemporal_load(hp + (size_t)(s0 + j) * (R + 1) + threadIdx.x) : 0.f;
+                v[j] = s0 + j < n_splits ? __hip_atomic_load(reinterpret_cast<const uint32_t *>(hp + (size_t)(s0 + j) * (R + 1) + threadIdx.x),
+                                                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                                         : 0u;
 #pragma unroll
-            for (int j = 0; j < 8; j++) t += v[j];
+            for (int j = 0; j < 8; j++) t += __uint_as_float(v[j]);
         }
         red[threadIdx.x] = t;
     }
