@@ -483,6 +483,30 @@ static int launch_gemv(hipStream_t st, float *out, const lv_matrix &w, const lv_
     return LV_OK;
 }
 
+// Three same-shape matrices applied to one vector (the q, k and v projections of a token) as one launch when the
+// streaming kernel covers the shape, else as three.
+static int launch_gemv3(hipStream_t st, float *const out[3], const lv_matrix *const w[3], const float *x)
+{
+    const lv_matrix &w0 = *w[0];
+    bool same = true;
+    for (int i = 1; i < 3; i++) same = same && w[i]->ftype == w0.ftype && w[i]->view.rows == w0.view.rows && w[i]->view.cols == w0.view.cols;
+    if (same && w0.view.rows >= 2048 && w0.view.cols <= (uint32_t)kWideMaxK) {
+        GemvArgs3 a{};
+        for (int i = 0; i < 3; i++) { a.m[i].w = w[i]->view; a.m[i].x = x; a.m[i].out = out[i]; }
+        const uint32_t rows = w0.view.rows, nb = w0.view.cols / 32;
+        const uint32_t rows_per_wg = (rows + 255) / 256;
+        const uint32_t ns = (nb + 63) / 64, nr = kWideWaves / ns, per_set = (rows_per_wg + nr - 1) / nr;
+        const size_t red_bytes = (size_t)per_set * nr * ns * sizeof(float);
+        const dim3 grid((rows + rows_per_wg - 1) / rows_per_wg, 3);
+        if (w0.ftype == LV_Q4_0) gemv_wide3_kernel<4><<<grid, dim3(kWideWaves * 64), red_bytes, st>>>(a, rows_per_wg);
+        else gemv_wide3_kernel<8><<<grid, dim3(kWideWaves * 64), red_bytes, st>>>(a, rows_per_wg);
+        HIP_TRY(hipGetLastError());
+        return LV_OK;
+    }
+    for (int i = 0; i < 3; i++) LV_TRY(launch_gemv(st, out[i], *w[i], nullptr, x, 1, kGemvStore));
+    return LV_OK;
+}
+
 static size_t attn_part_floats(uint32_t batch, uint32_t heads, uint32_t splits, uint32_t rot)
 {
     return (size_t)batch * heads * splits * (rot + 1);
@@ -1159,9 +1183,11 @@ static int record_token(lv_session *s, uint32_t idx, bool with_head)
         normalize_kernel<<<dim3(1), dim3(256), 0, st>>>(s->xn, s->x, lw.attn_norm, D);
         HIP_TRY(hipGetLastError());
         LV_TRY(trace_copy(s, li, LV_TRACE_NORM_IN, s->xn, D));
-        LV_TRY(launch_gemv(st, s->k, lw.wk, nullptr, s->xn, 1, kGemvStore));
-        LV_TRY(launch_gemv(st, s->q, lw.wq, nullptr, s->xn, 1, kGemvStore));
-        LV_TRY(launch_gemv(st, s->v, lw.wv, nullptr, s->xn, 1, kGemvStore));
+        {
+            float *const outs[3] = {s->k, s->q, s->v};
+            const lv_matrix *const mats[3] = {&lw.wk, &lw.wq, &lw.wv};
+            LV_TRY(launch_gemv3(st, outs, mats, s->xn));
+        }
         kv_append2_kernel<<<dim3(kv_grid.x, kv_grid.y, 2), dim3(256), 0, st>>>(kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->k, s->v, pos_ptr, idx, D, s->backlog);
         HIP_TRY(hipGetLastError());
         LV_TRY(launch_attention(st, s->vo, kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->q, s->trig, s->attn_part, s->attn_counters,

@@ -45,14 +45,11 @@ __device__ __forceinline__ float wide_dot(const WideTile &t, const float (&x)[32
 
 // NMAT = 2: the SiLU form, rows of w (W3) and w1 (W1) with the same index are walked together.
 template <int QT, int MODE>
-__global__ __launch_bounds__(kWideWaves * 64) void gemv_wide_kernel(GemvArgs a, uint32_t rows_per_wg)
+__device__ __forceinline__ void gemv_wide_body(const GemvArgs &a, uint32_t rows_per_wg, uint32_t z /* batch row */, float *xs, float *red)
 {
     constexpr int NMAT = MODE == kGemvSilu ? 2 : 1;
     constexpr int NW = kWideWaves;
-    __shared__ __attribute__((aligned(16))) float xs[kWideMaxK];
-    extern __shared__ float red[];       // [rows_per_wg rounded up to 4*NR][NMAT][NS]
     const uint32_t N = a.w.rows, K = a.w.cols, nb = K / 32;
-    const uint32_t z = blockIdx.y;
     const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int NS = (int)((nb + 63) / 64), NR = NW / NS;        // slabs; row sets (waves sharing a slab split the rows)
     const int slab = w % NS, rset = w / NS;
@@ -128,6 +125,26 @@ __global__ __launch_bounds__(kWideWaves * 64) void gemv_wide_kernel(GemvArgs a, 
         else if constexpr (MODE == kGemvAdd) *o += v[0];
         else *o = v[0] * v[NMAT - 1] / (__expf(-v[NMAT - 1]) + 1.f);
     }
+}
+
+template <int QT, int MODE>
+__global__ __launch_bounds__(kWideWaves * 64) void gemv_wide_kernel(GemvArgs a, uint32_t rows_per_wg)
+{
+    __shared__ __attribute__((aligned(16))) float xs[kWideMaxK];
+    extern __shared__ float red[];       // [rows_per_wg rounded up to 4*NR][NMAT][NS]
+    gemv_wide_body<QT, MODE>(a, rows_per_wg, blockIdx.y, xs, red);
+}
+
+// Three matrices with the same input vector in one launch (Wq, Wk, Wv of a layer): blockIdx.y selects the matrix.
+struct GemvArgs3 {
+    GemvArgs m[3];
+};
+template <int QT>
+__global__ __launch_bounds__(kWideWaves * 64) void gemv_wide3_kernel(GemvArgs3 a, uint32_t rows_per_wg)
+{
+    __shared__ __attribute__((aligned(16))) float xs[kWideMaxK];
+    extern __shared__ float red[];
+    gemv_wide_body<QT, kGemvStore>(a.m[blockIdx.y], rows_per_wg, 0, xs, red);
 }
 
 }  // namespace lv
