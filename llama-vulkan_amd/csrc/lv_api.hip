@@ -446,12 +446,17 @@ static void launch_gemv_cfg(const GemvArgs &a, uint32_t batch, hipStream_t st)
     gemv_kernel<QT, MODE, CW, P, RPW><<<dim3(grid, batch), dim3(256), 0, st>>>(a);
 }
 
+// matrices that can keep 256 workgroups busy go through the streaming kernel (x staged once per workgroup)
+static bool gemv_streams(const MatView &w, uint32_t batch)
+{
+    return w.rows >= 2048 && w.cols <= (uint32_t)kWideMaxK && batch <= 8;
+}
+
 template <int QT, int MODE>
 static void launch_gemv_mode(const GemvArgs &a, uint32_t batch, hipStream_t st)
 {
     const uint32_t nb = a.w.cols / 32;
-    // matrices that can keep 256 workgroups busy go through the streaming kernel (x staged once per workgroup)
-    if (a.w.rows >= 2048 && a.w.cols <= (uint32_t)kWideMaxK && batch <= 8) {
+    if (gemv_streams(a.w, batch)) {
         const uint32_t rows_per_wg = (a.w.rows + 255) / 256;
         const uint32_t ns = (nb + 63) / 64, nr = kWideWaves / ns, per_set = (rows_per_wg + nr - 1) / nr;
         const size_t red_bytes = (size_t)per_set * nr * (MODE == kGemvSilu ? 2 : 1) * ns * sizeof(float);
@@ -465,14 +470,17 @@ static void launch_gemv_mode(const GemvArgs &a, uint32_t batch, hipStream_t st)
     else launch_gemv_cfg<QT, MODE, 4, 3>(a, batch, st);
 }
 
+// norm_w (optional): x is normalised inside the kernel; only valid when gemv_streams(w, batch)
 static int launch_gemv(hipStream_t st, float *out, const lv_matrix &w, const lv_matrix *w1, const float *x, uint32_t batch,
-                       int mode)
+                       int mode, const float *norm_w = nullptr)
 {
     GemvArgs a{};
     a.w = w.view;
     if (w1) a.w1 = w1->view;
     a.x = x;
     a.out = out;
+    a.norm_w = norm_w;
+    if (norm_w && !gemv_streams(a.w, batch)) return fail(LV_ERR_ARG, "gemv: fused normalisation needs the streaming kernel");
     const bool q4 = w.ftype == LV_Q4_0;
     switch (mode) {
     case kGemvStore: q4 ? launch_gemv_mode<4, kGemvStore>(a, batch, st) : launch_gemv_mode<8, kGemvStore>(a, batch, st); break;
@@ -485,14 +493,31 @@ static int launch_gemv(hipStream_t st, float *out, const lv_matrix &w, const lv_
 
 // Three same-shape matrices applied to one vector (the q, k and v projections of a token) as one launch when the
 // streaming kernel covers the shape, else as three.
-static int launch_gemv3(hipStream_t st, float *const out[3], const lv_matrix *const w[3], const float *x)
+struct Gemv3Extras {
+    const float *norm_w = nullptr;                 // normalise x inside the kernel
+    uint16_t *cache[3] = {nullptr, nullptr, nullptr};  // append result i to this cache plane as fp16
+    const uint32_t *pos_ptr = nullptr;
+    uint32_t pos_add = 0, backlog = 0;
+};
+static bool gemv3_streams(const lv_matrix *const w[3])
 {
     const lv_matrix &w0 = *w[0];
     bool same = true;
     for (int i = 1; i < 3; i++) same = same && w[i]->ftype == w0.ftype && w[i]->view.rows == w0.view.rows && w[i]->view.cols == w0.view.cols;
-    if (same && w0.view.rows >= 2048 && w0.view.cols <= (uint32_t)kWideMaxK) {
+    return same && gemv_streams(w0.view, 1);
+}
+static int launch_gemv3(hipStream_t st, float *const out[3], const lv_matrix *const w[3], const float *x, const Gemv3Extras *ex = nullptr)
+{
+    const lv_matrix &w0 = *w[0];
+    if (gemv3_streams(w)) {
         GemvArgs3 a{};
-        for (int i = 0; i < 3; i++) { a.m[i].w = w[i]->view; a.m[i].x = x; a.m[i].out = out[i]; }
+        for (int i = 0; i < 3; i++) {
+            a.m[i].w = w[i]->view; a.m[i].x = x; a.m[i].out = out[i];
+            if (ex) {
+                a.m[i].norm_w = ex->norm_w; a.m[i].cache = ex->cache[i]; a.m[i].pos_ptr = ex->pos_ptr; a.m[i].pos_add = ex->pos_add;
+                a.m[i].backlog = ex->backlog;
+            }
+        }
         const uint32_t rows = w0.view.rows, nb = w0.view.cols / 32;
         const uint32_t rows_per_wg = (rows + 255) / 256;
         const uint32_t ns = (nb + 63) / 64, nr = kWideWaves / ns, per_set = (rows_per_wg + nr - 1) / nr;
@@ -503,6 +528,7 @@ static int launch_gemv3(hipStream_t st, float *const out[3], const lv_matrix *co
         HIP_TRY(hipGetLastError());
         return LV_OK;
     }
+    if (ex) return fail(LV_ERR_ARG, "gemv3: fused extras need the streaming kernel");
     for (int i = 0; i < 3; i++) LV_TRY(launch_gemv(st, out[i], *w[i], nullptr, x, 1, kGemvStore));
     return LV_OK;
 }
@@ -1180,32 +1206,49 @@ static int record_token(lv_session *s, uint32_t idx, bool with_head)
     const dim3 kv_grid((D + 255) / 256, 1);
     for (uint32_t li = 0; li < hp.layers; li++) {
         const LayerWeights &lw = m->layers[li];
-        normalize_kernel<<<dim3(1), dim3(256), 0, st>>>(s->xn, s->x, lw.attn_norm, D);
-        HIP_TRY(hipGetLastError());
-        LV_TRY(trace_copy(s, li, LV_TRACE_NORM_IN, s->xn, D));
-        {
-            float *const outs[3] = {s->k, s->q, s->v};
-            const lv_matrix *const mats[3] = {&lw.wk, &lw.wq, &lw.wv};
+        float *const outs[3] = {s->k, s->q, s->v};
+        const lv_matrix *const mats[3] = {&lw.wk, &lw.wq, &lw.wv};
+        // Without tracing, at shapes the streaming kernel covers, normalisation and the cache append ride along with
+        // the projections (one launch instead of five); the trace wants the normalised vector in memory.
+        const bool fused = !s->trace && gemv3_streams(mats) && gemv_streams(lw.w3.view, 1);
+        if (fused) {
+            Gemv3Extras ex;
+            ex.norm_w = lw.attn_norm;
+            ex.cache[0] = kv_ptr(s, li, 0); ex.cache[2] = kv_ptr(s, li, 1);
+            ex.pos_ptr = pos_ptr; ex.pos_add = idx; ex.backlog = s->backlog;
+            LV_TRY(launch_gemv3(st, outs, mats, s->x, &ex));
+        } else {
+            normalize_kernel<<<dim3(1), dim3(256), 0, st>>>(s->xn, s->x, lw.attn_norm, D);
+            HIP_TRY(hipGetLastError());
+            LV_TRY(trace_copy(s, li, LV_TRACE_NORM_IN, s->xn, D));
             LV_TRY(launch_gemv3(st, outs, mats, s->xn));
+            kv_append2_kernel<<<dim3(kv_grid.x, kv_grid.y, 2), dim3(256), 0, st>>>(kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->k, s->v, pos_ptr, idx, D, s->backlog);
+            HIP_TRY(hipGetLastError());
         }
-        kv_append2_kernel<<<dim3(kv_grid.x, kv_grid.y, 2), dim3(256), 0, st>>>(kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->k, s->v, pos_ptr, idx, D, s->backlog);
-        HIP_TRY(hipGetLastError());
         LV_TRY(launch_attention(st, s->vo, kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->q, s->trig, s->attn_part, s->attn_counters,
                                 pos_ptr, idx, s->backlog, hp.heads, hp.rot, 1));
         LV_TRY(launch_gemv(st, s->x, lw.wo, nullptr, s->vo, 1, kGemvAdd));
         LV_TRY(trace_copy(s, li, LV_TRACE_POST_ATTN, s->x, D));
-        normalize_kernel<<<dim3(1), dim3(256), 0, st>>>(s->xn, s->x, lw.ffn_norm, D);
-        HIP_TRY(hipGetLastError());
-        LV_TRY(trace_copy(s, li, LV_TRACE_POST_ATTN_NORM, s->xn, D));
-        LV_TRY(launch_gemv(st, s->ff, lw.w3, &lw.w1, s->xn, 1, kGemvSilu));
+        if (fused) {
+            LV_TRY(launch_gemv(st, s->ff, lw.w3, &lw.w1, s->x, 1, kGemvSilu, lw.ffn_norm));
+        } else {
+            normalize_kernel<<<dim3(1), dim3(256), 0, st>>>(s->xn, s->x, lw.ffn_norm, D);
+            HIP_TRY(hipGetLastError());
+            LV_TRY(trace_copy(s, li, LV_TRACE_POST_ATTN_NORM, s->xn, D));
+            LV_TRY(launch_gemv(st, s->ff, lw.w3, &lw.w1, s->xn, 1, kGemvSilu));
+        }
         LV_TRY(trace_copy(s, li, LV_TRACE_FF, s->ff, F));
         LV_TRY(launch_gemv(st, s->x, lw.w2, nullptr, s->ff, 1, kGemvAdd));
         LV_TRY(trace_copy(s, li, LV_TRACE_OUT, s->x, D));
     }
     if (with_head) {
-        normalize_kernel<<<dim3(1), dim3(256), 0, st>>>(s->xn, s->x, m->norm, D);
-        HIP_TRY(hipGetLastError());
-        LV_TRY(launch_gemv(st, s->logits, m->output, nullptr, s->xn, 1, kGemvStore));
+        if (!s->trace && gemv_streams(m->output.view, 1)) {
+            LV_TRY(launch_gemv(st, s->logits, m->output, nullptr, s->x, 1, kGemvStore, m->norm));
+        } else {
+            normalize_kernel<<<dim3(1), dim3(256), 0, st>>>(s->xn, s->x, m->norm, D);
+            HIP_TRY(hipGetLastError());
+            LV_TRY(launch_gemv(st, s->logits, m->output, nullptr, s->xn, 1, kGemvStore));
+        }
     }
     return LV_OK;
 }

@@ -43,9 +43,30 @@ __device__ __forceinline__ float wide_dot(const WideTile &t, const float (&x)[32
     else return (q8_block_dot(t.c, t.c2, x) - 128.f * xsum) * half_bits_to_float(t.d);
 }
 
+// Workgroup barrier that orders LDS traffic only: the weight loads in flight stay in flight.
+__device__ __forceinline__ void wide_lds_barrier()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+// sum over the workgroup through kWideWaves floats of LDS (one barrier; the caller alternates scratch areas)
+__device__ __forceinline__ float wide_block_sum(float v, float *scratch, int w, int lane)
+{
+    v = wave_sum(v);
+    if (lane == 0) scratch[w] = v;
+    wide_lds_barrier();
+    float t = 0.f;
+#pragma unroll
+    for (int i = 0; i < kWideWaves; i++) t += scratch[i];
+    return t;
+}
+
 // NMAT = 2: the SiLU form, rows of w (W3) and w1 (W1) with the same index are walked together.
 template <int QT, int MODE>
-__device__ __forceinline__ void gemv_wide_body(const GemvArgs &a, uint32_t rows_per_wg, uint32_t z /* batch row */, float *xs, float *red)
+__device__ __forceinline__ void gemv_wide_body(const GemvArgs &a, uint32_t rows_per_wg, uint32_t z /* batch row */, float *xs, float *red,
+                                               float *stat /* 32 floats */)
 {
     constexpr int NMAT = MODE == kGemvSilu ? 2 : 1;
     constexpr int NW = kWideWaves;
@@ -60,10 +81,7 @@ __device__ __forceinline__ void gemv_wide_body(const GemvArgs &a, uint32_t rows_
     const uint32_t n_rows = row0 < N ? min(rows_per_wg, N - row0) : 0;
     const uint32_t per_set = (rows_per_wg + NR - 1) / NR;       // rows per row set (static upper bound)
 
-    // ---- x -> LDS -> registers -----------------------------------------------------------------------------------
-    const float *xz = a.x + (size_t)z * K;
-    for (uint32_t i = threadIdx.x * 4; i < K; i += NW * 64 * 4) *reinterpret_cast<float4 *>(xs + i) = *reinterpret_cast<const float4 *>(xz + i);
-    // the first rows' loads go out before the wait for x
+    // the first rows' loads go out before anything else
     constexpr int DEPTH = kWideDepth<QT, NMAT>;
     WideTile q[NMAT][DEPTH];
     auto fetch = [&](int slot, uint32_t i) {       // i = index of the row inside this wave's row set
@@ -75,7 +93,30 @@ __device__ __forceinline__ void gemv_wide_body(const GemvArgs &a, uint32_t rows_
     };
 #pragma unroll
     for (int i = 0; i < DEPTH; i++) fetch(i, i);
-    __syncthreads();
+
+    // ---- x -> LDS -> registers; optionally normalised on the way (normalize.comp:34-64) ---------------------------
+    // With norm weights, LDS gets x*w and the scalar rsqrt(mean((x - mean)^2)) multiplies the row sums at the end.
+    const float *xz = a.x + (size_t)z * K;
+    float inv = 1.f;
+    if (a.norm_w) {
+        float s = 0.f;
+        for (uint32_t i = threadIdx.x * 4; i < K; i += NW * 64 * 4) {
+            const float4 v = *reinterpret_cast<const float4 *>(xz + i), wv = *reinterpret_cast<const float4 *>(a.norm_w + i);
+            s += (v.x + v.y) + (v.z + v.w);
+            *reinterpret_cast<float4 *>(xs + i) = make_float4(v.x * wv.x, v.y * wv.y, v.z * wv.z, v.w * wv.w);
+        }
+        const float mean = wide_block_sum(s, stat, w, lane) / (float)K;
+        float qd = 0.f;
+        for (uint32_t i = threadIdx.x * 4; i < K; i += NW * 64 * 4) {
+            const float4 v = *reinterpret_cast<const float4 *>(xz + i);   // second look at x: cache hits
+            const float c0 = v.x - mean, c1 = v.y - mean, c2 = v.z - mean, c3 = v.w - mean;
+            qd = fmaf(c0, c0, qd); qd = fmaf(c1, c1, qd); qd = fmaf(c2, c2, qd); qd = fmaf(c3, c3, qd);
+        }
+        inv = rsqrtf(wide_block_sum(qd, stat + 16, w, lane) / (float)K);   // its barrier also publishes xs
+    } else {
+        for (uint32_t i = threadIdx.x * 4; i < K; i += NW * 64 * 4) *reinterpret_cast<float4 *>(xs + i) = *reinterpret_cast<const float4 *>(xz + i);
+        wide_lds_barrier();
+    }
     float xr[32], xsum = 0.f;
     {
         const float4 *src = reinterpret_cast<const float4 *>(xs + (size_t)(lane_ok ? blk_col : 0) * 32);
@@ -108,7 +149,7 @@ __device__ __forceinline__ void gemv_wide_body(const GemvArgs &a, uint32_t rows_
             }
         }
     }
-    __syncthreads();
+    wide_lds_barrier();
 
     // ---- combine the slabs, write ---------------------------------------------------------------------------------------
     for (uint32_t r = threadIdx.x; r < n_rows; r += NW * 64) {
@@ -120,10 +161,20 @@ __device__ __forceinline__ void gemv_wide_body(const GemvArgs &a, uint32_t rows_
             for (int s = 0; s < NS; s++) t += red[((size_t)r * NMAT + mi) * NS + s];
             v[mi] = t;
         }
+#pragma unroll
+        for (int mi = 0; mi < NMAT; mi++) v[mi] *= inv;
         float *o = a.out + (size_t)z * N + row0 + r;
-        if constexpr (MODE == kGemvStore) *o = v[0];
-        else if constexpr (MODE == kGemvAdd) *o += v[0];
-        else *o = v[0] * v[NMAT - 1] / (__expf(-v[NMAT - 1]) + 1.f);
+        if constexpr (MODE == kGemvStore) {
+            *o = v[0];
+            if (a.cache) {
+                const uint32_t row = (a.pos_ptr ? *a.pos_ptr : 0u) + a.pos_add + z;
+                if (row < a.backlog) a.cache[(size_t)row * N + row0 + r] = float_to_half_bits(v[0]);
+            }
+        } else if constexpr (MODE == kGemvAdd) {
+            *o += v[0];
+        } else {
+            *o = v[0] * v[NMAT - 1] / (__expf(-v[NMAT - 1]) + 1.f);
+        }
     }
 }
 
@@ -131,8 +182,9 @@ template <int QT, int MODE>
 __global__ __launch_bounds__(kWideWaves * 64) void gemv_wide_kernel(GemvArgs a, uint32_t rows_per_wg)
 {
     __shared__ __attribute__((aligned(16))) float xs[kWideMaxK];
+    __shared__ float stat[32];
     extern __shared__ float red[];       // [rows_per_wg rounded up to 4*NR][NMAT][NS]
-    gemv_wide_body<QT, MODE>(a, rows_per_wg, blockIdx.y, xs, red);
+    gemv_wide_body<QT, MODE>(a, rows_per_wg, blockIdx.y, xs, red, stat);
 }
 
 // Three matrices with the same input vector in one launch (Wq, Wk, Wv of a layer): blockIdx.y selects the matrix.
@@ -143,8 +195,9 @@ template <int QT>
 __global__ __launch_bounds__(kWideWaves * 64) void gemv_wide3_kernel(GemvArgs3 a, uint32_t rows_per_wg)
 {
     __shared__ __attribute__((aligned(16))) float xs[kWideMaxK];
+    __shared__ float stat[32];
     extern __shared__ float red[];
-    gemv_wide_body<QT, kGemvStore>(a.m[blockIdx.y], rows_per_wg, 0, xs, red);
+    gemv_wide_body<QT, kGemvStore>(a.m[blockIdx.y], rows_per_wg, 0, xs, red, stat);
 }
 
 }  // namespace lv

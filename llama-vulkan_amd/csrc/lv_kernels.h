@@ -93,6 +93,11 @@ struct GemvArgs {
     MatView w1;      // second matrix of the SiLU form
     const float *x;  // [batch][K]
     float *out;      // [batch][N]
+    // extras of the streaming kernel (all optional):
+    const float *norm_w = nullptr;     // x is normalised with these weights first (normalize.comp) instead of by a launch of its own
+    uint16_t *cache = nullptr;         // the result is also appended, as fp16, to this K or V plane [backlog][N] (copy_to_cache.comp)
+    const uint32_t *pos_ptr = nullptr; // ... at row *pos_ptr + pos_add
+    uint32_t pos_add = 0, backlog = 0;
 };
 
 template <int QT>
