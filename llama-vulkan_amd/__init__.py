@@ -43,7 +43,7 @@ class HParams(C.Structure):
 class MkgConfig(C.Structure):
     _fields_ = [("vocab", C.c_uint32), ("dim", C.c_uint32), ("heads", C.c_uint32), ("layers", C.c_uint32),
                 ("ff", C.c_uint32), ("multiple_of", C.c_uint32), ("wtype", C.c_uint32), ("seed", C.c_uint64),
-                ("sigma", C.c_float)]
+                ("sigma", C.c_float), ("tok_type", C.c_uint32)]
 
 
 _libs = {}
@@ -233,10 +233,11 @@ PRESETS = {
 }
 
 
-def write_model(path, wtype=LV_Q4_0, seed=0, sigma=0.02, preset=None, **shape):
+def write_model(path, wtype=LV_Q4_0, seed=0, sigma=0.02, preset=None, tok_type=0, **shape):
+    """tok_type: 0 = f32 embedding table (the published configs), LV_Q4_0 / LV_Q8_0 = quantised like the matrices"""
     cfg = dict(PRESETS[preset]) if preset else {}
     cfg.update(shape)
-    c = MkgConfig(cfg["vocab"], cfg["dim"], cfg["heads"], cfg["layers"], cfg["ff"], 256, wtype, seed, sigma)
+    c = MkgConfig(cfg["vocab"], cfg["dim"], cfg["heads"], cfg["layers"], cfg["ff"], 256, wtype, seed, sigma, tok_type)
     rc = mkggml().mkg_write_model(os.fsencode(path), C.byref(c))
     if rc != 0:
         raise OSError(-rc, os.strerror(-rc), path)

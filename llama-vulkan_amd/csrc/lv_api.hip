@@ -98,6 +98,7 @@ struct lv_model {
     int mega_kind = 0;              // 0 none, else a compiled shape class of the persistent kernel (mega_dispatch)
     uint8_t *mega_stream = nullptr;
     float *mega_norms = nullptr;    // [layers][2][D] + final norm [D]
+    float *tok_f32_own = nullptr;   // fp32 copy of a quantised embedding table (the persistent kernel reads rows as fp32)
 };
 
 // Shape classes the persistent kernel is compiled for: LLaMA-7B and LLaMA-13B layer shapes, q4_0 and q8_0.
@@ -816,7 +817,7 @@ static int build_mega(lv_model *m)
 {
     const lv_hparams &hp = m->hp;
     const uint32_t ft = m->output.ftype;
-    bool uniform = (ft == LV_Q4_0 || ft == LV_Q8_0) && m->tok_ftype == LV_F32;
+    bool uniform = ft == LV_Q4_0 || ft == LV_Q8_0;
     for (const LayerWeights &lw : m->layers)
         for (const lv_matrix *x : {&lw.wq, &lw.wk, &lw.wv, &lw.wo, &lw.w1, &lw.w2, &lw.w3}) uniform = uniform && x->ftype == ft;
     if (!uniform || (int)m->ctx->props.multiProcessorCount < kMegaWGs) return LV_OK;
@@ -830,6 +831,21 @@ static int build_mega(lv_model *m)
         });
         if (!fits) continue;
         LV_TRY(mega_dispatch(kind, [&](auto shape) { return build_mega_stream<decltype(shape)>(m); }));
+        if (m->tok_ftype != LV_F32) {
+            // llava_buffer.cpp:339-401 dequantises the token's row on the host at every step; here the whole table is
+            // expanded once (exact: a code times an fp16 scale is representable in fp32)
+            const uint64_t nb = (uint64_t)hp.vocab * (hp.dim / 32);
+            hipError_t e = hipMalloc(reinterpret_cast<void **>(&m->tok_f32_own), nb * 32 * sizeof(float));
+            if (e != hipSuccess)
+                return fail(e == hipErrorOutOfMemory ? LV_ERR_OOM : LV_ERR_HIP, "fp32 embedding table of %llu bytes: %s",
+                            (unsigned long long)(nb * 128), hipGetErrorString(e));
+            const unsigned grid = (unsigned)((nb + 255) / 256);
+            if (m->tok_ftype == LV_Q4_0) dequant_kernel<4><<<dim3(grid), dim3(256), 0, m->ctx->stream>>>(m->tok_quant.view, 0, nb, m->tok_f32_own);
+            else dequant_kernel<8><<<dim3(grid), dim3(256), 0, m->ctx->stream>>>(m->tok_quant.view, 0, nb, m->tok_f32_own);
+            HIP_TRY(hipGetLastError());
+            HIP_TRY(hipStreamSynchronize(m->ctx->stream));
+            m->tok_f32 = m->tok_f32_own;
+        }
         m->mega_kind = kind;
         break;
     }
@@ -948,6 +964,7 @@ extern "C" int lv_model_upload(lv_ctx *c, const void *base, uint64_t base_size, 
     if (rc != LV_OK) {
         (void)hipFree(m->mega_stream);
         (void)hipFree(m->mega_norms);
+        (void)hipFree(m->tok_f32_own);
         (void)hipFree(m->arena);
         delete m;
         return rc;
@@ -962,6 +979,7 @@ extern "C" int lv_model_destroy(lv_model *m)
     (void)hipSetDevice(m->ctx->device);
     (void)hipFree(m->mega_stream);
     (void)hipFree(m->mega_norms);
+    (void)hipFree(m->tok_f32_own);
     (void)hipFree(m->arena);
     delete m;
     return LV_OK;

@@ -35,6 +35,8 @@ typedef struct {
     uint32_t wtype; /* MKG_Q4_0 or MKG_Q8_0 for the matrices */
     uint64_t seed;
     float sigma;    /* 0.02 in the published configs */
+    uint32_t tok_type; /* 0: embedding table in f32 (the published configs); MKG_Q4_0 / MKG_Q8_0: quantised like the matrices,
+                          as files converted from real checkpoints have it */
 } mkg_config;
 
 /* ---------------- RNG ---------------- */
@@ -205,7 +207,7 @@ static uint32_t build_table(const mkg_config *c, mkg_tensor **out)
     do { snprintf(t[k].name, sizeof t[k].name, fmt, arg); t[k].ftype = ft; t[k].n_dims = 2; t[k].ne0 = cols; t[k].ne1 = rows; k++; } while (0)
 #define ADD1(fmt, arg, len) \
     do { snprintf(t[k].name, sizeof t[k].name, fmt, arg); t[k].ftype = MKG_F32; t[k].n_dims = 1; t[k].ne0 = len; t[k].ne1 = 1; k++; } while (0)
-    ADD2("tok_embeddings.weight%s", "", MKG_F32, c->dim, c->vocab);
+    ADD2("tok_embeddings.weight%s", "", c->tok_type ? c->tok_type : MKG_F32, c->dim, c->vocab);
     ADD1("norm.weight%s", "", c->dim);
     ADD2("output.weight%s", "", c->wtype, c->dim, c->vocab);
     for (uint32_t i = 0; i < c->layers; i++) {
@@ -240,7 +242,7 @@ static int pwrite_all(int fd, const void *src, size_t n, off_t at)
 int mkg_write_model(const char *path, const mkg_config *c)
 {
     if (!c || c->heads == 0 || c->dim % c->heads || c->dim % 32 || c->ff % 32 || c->vocab < 259 ||
-        (c->wtype != MKG_Q4_0 && c->wtype != MKG_Q8_0))
+        (c->wtype != MKG_Q4_0 && c->wtype != MKG_Q8_0) || (c->tok_type != 0 && c->tok_type != MKG_Q4_0 && c->tok_type != MKG_Q8_0))
         return -EINVAL;
 
     /* pass 1: sizes */
@@ -318,14 +320,14 @@ int mkg_write_model(const char *path, const mkg_config *c)
 static void usage(void)
 {
     fprintf(stderr,
-            "usage: mkggml OUT --preset 7b|13b|tiny [--wtype q4_0|q8_0] [--seed N]\n"
+            "usage: mkggml OUT --preset 7b|13b|tiny [--wtype q4_0|q8_0] [--tok-type f32|q4_0|q8_0] [--seed N]\n"
             "       mkggml OUT --dim D --heads H --layers L --ff F --vocab V [--wtype ...] [--seed N] [--sigma S]\n");
 }
 
 int main(int argc, char **argv)
 {
     if (argc < 2) { usage(); return 2; }
-    mkg_config c = { 32000, 4096, 32, 32, 11008, 256, MKG_Q4_0, 0, 0.02f };
+    mkg_config c = { 32000, 4096, 32, 32, 11008, 256, MKG_Q4_0, 0, 0.02f, 0 };
     for (int i = 2; i < argc; i++) {
         const char *a = argv[i], *v = (i + 1 < argc) ? argv[i + 1] : NULL;
         if (!v) { usage(); return 2; }
@@ -335,6 +337,7 @@ int main(int argc, char **argv)
             else if (!strcmp(v, "tiny")) { c.dim = 256; c.heads = 4; c.layers = 2; c.ff = 704; c.vocab = 512; }
             else { usage(); return 2; }
         } else if (!strcmp(a, "--wtype")) c.wtype = !strcmp(v, "q8_0") ? MKG_Q8_0 : MKG_Q4_0;
+        else if (!strcmp(a, "--tok-type")) c.tok_type = !strcmp(v, "q8_0") ? MKG_Q8_0 : !strcmp(v, "q4_0") ? MKG_Q4_0 : 0;
         else if (!strcmp(a, "--seed")) c.seed = strtoull(v, NULL, 0);
         else if (!strcmp(a, "--sigma")) c.sigma = (float)atof(v);
         else if (!strcmp(a, "--dim")) c.dim = (uint32_t)atoi(v);

@@ -225,3 +225,32 @@ def test_persistent_kernel_refused_for_other_shapes(lva, ctx, tiny_models):
     assert s.path() == lva.PATH_GRAPH
     assert ctx.lib.lv_session_set_path(s.h, lva.PATH_PERSISTENT) == -1
     s.close(); model.close()
+
+
+@pytest.mark.parametrize("wname,tname", [("q4_0", "q4_0"), ("q8_0", "q8_0"), ("q4_0", "q8_0")])
+def test_quantised_embedding_table_all_paths(lva, orc, ctx, tmp_path, wname, tname):
+    """files converted from real checkpoints quantise tok_embeddings like the matrices (llava_buffer.cpp:339-401 dequantises
+    the token's row per step); the persistent kernel reads rows from an fp32 expansion made at upload, the operator
+    chain dequantises the row on the device: both against the oracle, which dequantises the row on the host"""
+    wt = {"q4_0": lva.LV_Q4_0, "q8_0": lva.LV_Q8_0}
+    p = str(tmp_path / "qtok.ggml")
+    lva.write_model(p, wtype=wt[wname], tok_type=wt[tname], seed=12, vocab=2048, layers=2, dim=4096, heads=32, ff=11008)
+    om = orc.Model(p)
+    osess = orc.Session(om, 128)
+    model = lva.Model(ctx, p)
+    pk, ops = lva.Session(model, 128), lva.Session(model, 128)
+    assert pk.path() == lva.PATH_PERSISTENT
+    ops.set_path(lva.PATH_GRAPH)
+    prompt = lva.synth_tokens(5, 3, 2048, seed=2)
+    want = osess.eval(prompt)
+    pk.begin(prompt, 0); ops.begin(prompt, 0)
+    pos = len(prompt)
+    for step in range(6):
+        _check_logits(pk.logits(), want)
+        _check_logits(ops.logits(), want)
+        tok = orc.greedy(want)
+        assert pk.argmax() == tok == ops.argmax(), step
+        want = osess.eval([tok])
+        pk.begin([tok], pos); ops.begin([tok], pos)
+        pos += 1
+    pk.close(); ops.close(); model.close(); osess.close(); om.close()
