@@ -2,14 +2,16 @@
 // (q4_0 / q8_0), on the matrix cores (reference: the *_batch.comp shader variants selected by
 // llava_session.cpp:243-255 when more than one token is pending).
 //
-// Arithmetic: fp16 MFMA with fp32 accumulation, on operands split in two fp16 halves each.  A dequantised weight
-// (q-8)*d or q*d has at most 19 significant bits, an fp32 activation 24: w = wh + wl, x = xh + xl with
-// wh = fp16(w), wl = fp16(w - wh) (exact for weights, 2^-22 relative for activations), and
-//     x*w ~= xh*wh + xl*wh + xh*wl                      (three MFMAs; the dropped xl*wl term is below 2^-22)
-// so the batched path agrees with the one-token fp32 path to fp32 rounding, not to fp16 rounding.
+// Arithmetic: fp16 MFMA with fp32 accumulation, in the order of the reference's shaders (matmul.glsl:41-74: the block
+// dot on the integer codes first, then times the block's scale, then added to the running sum).  A code (q-8 or q) is
+// a small integer, exact in fp16; an fp32 activation is split in two fp16 halves, x = xh + xl (2^-22 relative):
+//     sum_k x[k]*code[k] = sum_k xh[k]*code[k] + sum_k xl[k]*code[k]      (two MFMAs per 16 k, every product exact)
+// per block of 32 k into a scratch accumulator, which is then multiplied by the block's scale d[row] (one scale per
+// lane: in the MFMA result a lane holds one weight row) and added to the fp32 result.  The batched path therefore
+// agrees with the one-token fp32 path to fp32 rounding, not to fp16 rounding.
 //
 // Tiling: workgroup = 256 threads = 4 waves, output tile 128 tokens x 128 (or 64) weight rows, K step 64 (two quant
-// blocks).  One thread dequantises one (row, block) pair per step; every wave owns a 64 x 64 (or 32 x 64) sub-tile of
+// blocks).  One thread unpacks one (row, block) pair per step; every wave owns a 64 x 64 (or 32 x 64) sub-tile of
 // v_mfma_f32_32x32x16_f16 tiles.  Global loads of step s+1 are issued before the MFMAs of step s.
 #pragma once
 
@@ -84,27 +86,20 @@ __host__ __device__ constexpr int gemm_k_position(int e)
     return 8 * i + 2 * j + (b >> 1);
 }
 
-// 32 weights of one block -> 32 hi + 32 lo halfs at wh/wl, in gemm_k_position order.  All in packed fp16 arithmetic:
-// the integer code as fp16 (1024 + u has the bit pattern 0x6400 | u), hi = RTE(code * d), lo = fma(code, d, -hi), the
-// rounding error of that product, which fp16 represents exactly.
+// 32 codes of one block -> 32 halfs at w, in gemm_k_position order, as the integers they are (q4_0: q - 8, q8_0: q):
+// 1024 + u has the fp16 bit pattern 0x6400 | u, and subtracting 1024 + offset is exact.  A block outside the matrix
+// becomes zeros.
 template <int QT>
-__device__ __forceinline__ void gemm_dequant_block(uint16_t *wh, uint16_t *wl, bool valid, const uint4 &c0, const uint4 &c1, uint16_t dbits)
+__device__ __forceinline__ void gemm_codes_block(uint16_t *w, bool valid, const uint4 &c0, const uint4 &c1)
 {
-    union { uint16_t u; _Float16 h; } db;
-    db.u = valid ? dbits : (uint16_t)0;
-    const _Float16 d = db.h;
-    const lv_h2 dd = {d, d};
-    uint32_t ph[16], pl[16];
+    uint32_t ph[16];
     auto emit = [&](int slot, uint32_t packed_codes, _Float16 bias) {
         // packed_codes: two halfs 0x6400 | u
-        union { uint32_t u; lv_h2 h; } c, hi, lo;
+        union { uint32_t u; lv_h2 h; } c, v;
         c.u = packed_codes;
         const lv_h2 bb = {bias, bias};
-        const lv_h2 code = c.h - bb;                 // exact: small integers
-        hi.h = code * dd;
-        lo.h = __builtin_elementwise_fma(code, dd, -hi.h);
-        ph[slot] = hi.u;
-        pl[slot] = lo.u;
+        v.h = c.h - bb;                              // exact: small integers
+        ph[slot] = valid ? v.u : 0u;
     };
     if constexpr (QT == 4) {
         const uint32_t q[4] = {c0.x, c0.y, c0.z, c0.w};
@@ -122,10 +117,7 @@ __device__ __forceinline__ void gemm_dequant_block(uint16_t *wh, uint16_t *wl, b
         }
     }
 #pragma unroll
-    for (int g = 0; g < 4; g++) {
-        *reinterpret_cast<uint4 *>(wh + 8 * g) = make_uint4(ph[4 * g], ph[4 * g + 1], ph[4 * g + 2], ph[4 * g + 3]);
-        *reinterpret_cast<uint4 *>(wl + 8 * g) = make_uint4(pl[4 * g], pl[4 * g + 1], pl[4 * g + 2], pl[4 * g + 3]);
-    }
+    for (int g = 0; g < 4; g++) *reinterpret_cast<uint4 *>(w + 8 * g) = make_uint4(ph[4 * g], ph[4 * g + 1], ph[4 * g + 2], ph[4 * g + 3]);
 }
 
 // RM = weight rows per workgroup (128 or 64); tokens per workgroup: 128.  The four waves split the tile 2 x 2
@@ -139,7 +131,8 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs a)
     constexpr int WN = RM / 64;                   // waves along the rows
     constexpr int WM = 4 / WN;                    // waves along the tokens
     constexpr int MT = TN / WM / 32;              // 32-token tiles per wave
-    __shared__ __attribute__((aligned(16))) uint16_t sXh[TN * kGemmLd], sXl[TN * kGemmLd], sWh[RM * kGemmLd], sWl[RM * kGemmLd];
+    __shared__ __attribute__((aligned(16))) uint16_t sXh[TN * kGemmLd], sXl[TN * kGemmLd], sW[RM * kGemmLd];
+    __shared__ float sD[2][RM];                   // scale of (block of the step, row)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
     const uint32_t tok0 = blockIdx.y * TN, row0 = blockIdx.x * RM;
@@ -195,7 +188,10 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs a)
     if (steps > 1) fetch(pre[1], 1);
     auto one_step = [&](Staged &P, uint32_t step) {
         // registers -> LDS
-        if (has_w) gemm_dequant_block<QT>(sWh + r_w * kGemmLd + b_w * 32, sWl + r_w * kGemmLd + b_w * 32, P.wvalid, P.c0, P.c1, P.dbits);
+        if (has_w) {
+            gemm_codes_block<QT>(sW + r_w * kGemmLd + b_w * 32, P.wvalid, P.c0, P.c1);
+            sD[b_w][r_w] = P.wvalid ? half_bits_to_float(P.dbits) : 0.f;
+        }
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             *reinterpret_cast<uint4 *>(sXh + (xr + 32 * i) * kGemmLd + xc) = P.gh[i];
@@ -204,34 +200,48 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs a)
         __syncthreads();
         if (step + 2 < steps) fetch(P, step + 2);
 #pragma unroll
-        for (int kk = 0; kk < kGemmK / 16; kk++) {
-            const int ko = kk * 16 + (lane >> 5) * 8;
-            lv_h8 xh[MT], xl[MT], wh[2], wl[2];
+        for (int b = 0; b < kGemmK / 32; b++) {          // the two quant blocks of the step
+            lv_f16v blk[MT][2];
 #pragma unroll
-            for (int t = 0; t < MT; t++) {
-                const int xrow = (wm * MT + t) * 32 + (lane & 31);
-                xh[t] = *reinterpret_cast<const lv_h8 *>(sXh + xrow * kGemmLd + ko);
-                xl[t] = *reinterpret_cast<const lv_h8 *>(sXl + xrow * kGemmLd + ko);
+            for (int i = 0; i < MT; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) blk[i][j][r] = 0.f;
+#pragma unroll
+            for (int kk = 2 * b; kk < 2 * b + 2; kk++) {
+                const int ko = kk * 16 + (lane >> 5) * 8;
+                lv_h8 xh[MT], xl[MT], wc[2];
+#pragma unroll
+                for (int t = 0; t < MT; t++) {
+                    const int xrow = (wm * MT + t) * 32 + (lane & 31);
+                    xh[t] = *reinterpret_cast<const lv_h8 *>(sXh + xrow * kGemmLd + ko);
+                    xl[t] = *reinterpret_cast<const lv_h8 *>(sXl + xrow * kGemmLd + ko);
+                }
+#pragma unroll
+                for (int t = 0; t < 2; t++) {
+                    const int wr = wn * 64 + t * 32 + (lane & 31);
+                    wc[t] = *reinterpret_cast<const lv_h8 *>(sW + wr * kGemmLd + ko);
+                }
+                // product by product over all tiles: consecutive MFMAs do not wait for each other's accumulator
+#pragma unroll
+                for (int i = 0; i < MT; i++)
+#pragma unroll
+                    for (int j = 0; j < 2; j++) blk[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xl[i], wc[j], blk[i][j], 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < MT; i++)
+#pragma unroll
+                    for (int j = 0; j < 2; j++) blk[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh[i], wc[j], blk[i][j], 0, 0, 0);
             }
+            // times the block's scale: a lane's sixteen results of a tile belong to one weight row
 #pragma unroll
-            for (int t = 0; t < 2; t++) {
-                const int wr = wn * 64 + t * 32 + (lane & 31);
-                wh[t] = *reinterpret_cast<const lv_h8 *>(sWh + wr * kGemmLd + ko);
-                wl[t] = *reinterpret_cast<const lv_h8 *>(sWl + wr * kGemmLd + ko);
+            for (int j = 0; j < 2; j++) {
+                const float d = sD[b][wn * 64 + j * 32 + (lane & 31)];
+#pragma unroll
+                for (int i = 0; i < MT; i++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) acc[i][j][r] = fmaf(blk[i][j][r], d, acc[i][j][r]);
             }
-            // product by product over all tiles: consecutive MFMAs never wait for each other's accumulator
-#pragma unroll
-            for (int i = 0; i < MT; i++)
-#pragma unroll
-                for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xl[i], wh[j], acc[i][j], 0, 0, 0);
-#pragma unroll
-            for (int i = 0; i < MT; i++)
-#pragma unroll
-                for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh[i], wl[j], acc[i][j], 0, 0, 0);
-#pragma unroll
-            for (int i = 0; i < MT; i++)
-#pragma unroll
-                for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh[i], wh[j], acc[i][j], 0, 0, 0);
         }
         __syncthreads();
     };
