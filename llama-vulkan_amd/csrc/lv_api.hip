@@ -131,7 +131,8 @@ struct lv_session {
     hipStream_t stream = nullptr;
     uint32_t backlog = 0;
     uint16_t *kv = nullptr;  // [layers][2][backlog][dim]
-    float2 *trig = nullptr;  // [backlog][rot/2]
+    float2 *trig = nullptr;  // [backlog][rot/2]: cos/sin of delta * theta_i as the shader evaluates it
+    float2 *trig_abs = nullptr;  // [backlog][rot/2]: cos/sin of p * theta_i (batched attention)
     // activations (batch 1)
     float *x = nullptr, *xn = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *vo = nullptr, *ff = nullptr,
           *logits = nullptr;
@@ -559,11 +560,11 @@ static int launch_attention(hipStream_t st, float *out, const uint16_t *kc, cons
     return LV_OK;
 }
 
-static int launch_attention_batch(hipStream_t st, float *out, const uint16_t *kc, const uint16_t *vc, const float *q, const float2 *trig,
+static int launch_attention_batch(hipStream_t st, float *out, const uint16_t *kc, const uint16_t *vc, const float *q, const float2 *trig_abs,
                                   const uint32_t *pos_ptr, uint32_t pos_add, uint32_t n, uint32_t backlog, uint32_t heads, uint32_t rot)
 {
     AttnBatchArgs a{};
-    a.out = out; a.kcache = kc; a.vcache = vc; a.q = q; a.trig = trig; a.pos_ptr = pos_ptr; a.pos_add = pos_add;
+    a.out = out; a.kcache = kc; a.vcache = vc; a.q = q; a.trig_abs = trig_abs; a.pos_ptr = pos_ptr; a.pos_add = pos_add;
     a.n = n; a.heads = heads; a.backlog = backlog;
     const dim3 grid(heads, (n + kAttnBatchQ - 1) / kAttnBatchQ);
     switch (rot) {
@@ -591,10 +592,27 @@ static void build_trig(std::vector<float2> &t, uint32_t rows, uint32_t rot)
         }
 }
 
-static int upload_trig(float2 **dev, uint32_t rows, uint32_t rot, hipStream_t st)
+// cos/sin of p * theta_i for the batched attention, which rotates rows by their absolute position: theta_i rounded to
+// fp32 as above, the product and the functions in double (the difference of two such angles then differs from the
+// shader's fp32-rounded delta * theta_i by that one rounding only)
+static void build_trig_abs(std::vector<float2> &t, uint32_t rows, uint32_t rot)
+{
+    const uint32_t half = rot / 2;
+    t.resize((size_t)rows * half);
+    for (uint32_t i = 0; i < half; i++) {
+        const double freq = (double)powf(10000.0f, -(float)i / (float)half);
+        for (uint32_t d = 0; d < rows; d++) {
+            const double ang = (double)d * freq;
+            t[(size_t)d * half + i] = make_float2((float)cos(ang), (float)sin(ang));
+        }
+    }
+}
+
+static int upload_trig(float2 **dev, uint32_t rows, uint32_t rot, hipStream_t st, bool absolute = false)
 {
     std::vector<float2> t;
-    build_trig(t, rows, rot);
+    if (absolute) build_trig_abs(t, rows, rot);
+    else build_trig(t, rows, rot);
     HIP_TRY(hipMalloc(reinterpret_cast<void **>(dev), t.size() * sizeof(float2)));
     HIP_TRY(hipMemcpyAsync(*dev, t.data(), t.size() * sizeof(float2), hipMemcpyHostToDevice, st));
     HIP_TRY(hipStreamSynchronize(st));
@@ -1016,7 +1034,7 @@ extern "C" int lv_session_destroy(lv_session *s)
     (void)hipSetDevice(s->model->ctx->device);
     if (s->stream) (void)hipStreamSynchronize(s->stream);
     drop_graph(s);
-    void *dev[] = {s->kv, s->trig, s->x, s->xn, s->q, s->k, s->v, s->vo, s->ff, s->logits, s->attn_part, s->attn_counters,
+    void *dev[] = {s->kv, s->trig, s->trig_abs, s->x, s->xn, s->q, s->k, s->v, s->vo, s->ff, s->logits, s->attn_part, s->attn_counters,
                    s->cfg, s->argmax_dev, s->trace_buf, s->pf_x, s->pf_xn, s->pf_q, s->pf_k, s->pf_v, s->pf_vo, s->pf_g1, s->pf_g2,
                    s->pf_xh, s->pf_xl};
     for (void *p : dev) (void)hipFree(p);
@@ -1116,12 +1134,15 @@ extern "C" int lv_session_reserve(lv_session *s, uint32_t backlog)
 
     (void)hipFree(s->trig);
     s->trig = nullptr;
+    (void)hipFree(s->trig_abs);
+    s->trig_abs = nullptr;
     (void)hipFree(s->attn_part);
     s->attn_part = nullptr;
     (void)hipFree(s->attn_counters);
     s->attn_counters = nullptr;
     s->backlog = 0;
     LV_TRY(upload_trig(&s->trig, backlog, hp.rot, s->stream));
+    LV_TRY(upload_trig(&s->trig_abs, backlog, hp.rot, s->stream, true));
     const uint32_t splits = (backlog + kAttnChunk - 1) / kAttnChunk;
     HIP_TRY(hipMalloc(reinterpret_cast<void **>(&s->attn_part), attn_part_floats(1, hp.heads, splits, hp.rot) * sizeof(float)));
     HIP_TRY(hipMalloc(reinterpret_cast<void **>(&s->attn_counters), (size_t)hp.heads * 4));
@@ -1330,7 +1351,7 @@ static int record_prefill(lv_session *s, uint32_t idx0, uint32_t n, bool with_he
         else LV_TRY(launch_gemm(st, s->pf_v, D, lw.wv, s->pf_xn, n, s->pf_xh, s->pf_xl, false));
         kv_append2_kernel<<<dim3(kv_grid.x, kv_grid.y, 2), dim3(256), 0, st>>>(kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->pf_k, s->pf_v, pos_ptr, idx0, D, s->backlog);
         HIP_TRY(hipGetLastError());
-        LV_TRY(launch_attention_batch(st, s->pf_vo, kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->pf_q, s->trig, pos_ptr, idx0, n, s->backlog,
+        LV_TRY(launch_attention_batch(st, s->pf_vo, kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->pf_q, s->trig_abs, pos_ptr, idx0, n, s->backlog,
                                       hp.heads, hp.rot));
         LV_TRY(launch_gemm(st, s->pf_x, D, lw.wo, s->pf_vo, n, s->pf_xh, s->pf_xl, true));
         normalize_kernel<<<dim3(n), dim3(256), 0, st>>>(s->pf_xn, s->pf_x, lw.ffn_norm, D);

@@ -2,19 +2,28 @@
 // kqv_matching.comp with gl_GlobalInvocationID.z > 0.  Query row z sits at cache position pos + z and sees
 // positions 0 .. pos + z; all rows of the batch are in the cache before this runs.
 //
-// Same arithmetic as the one-query kernel: relative rotation per (query, position) pair with the angle
-// float(delta) * theta_i (mhsa.comp:45-58), e = exp(score / sqrt(R)) without max subtraction (softmax.comp:33),
-// out = sum e * V / sum e (kqv_matching.comp:35-41), V and K read back from the fp16 cache.
+// Arithmetic.  mhsa.comp:45-58 rotates every (query, position) pair by the relative angle delta * theta_i:
+//     s = sum_i cos(delta theta_i) (qx kx + qy ky) + sin(delta theta_i) (qx ky - qy kx),   delta = pos_q - pos_k.
+// That is Re[conj(q') k'] with q' = e^{i pos_q theta} q and k' = e^{i pos_k theta} k: rotating each query row and each
+// cache row ONCE by its own position turns the score into a plain dot product, which the matrix cores take (fp32 MFMA:
+// products and sums in fp32).  The rotation angles come from a table of cos/sin(p * theta_i) with theta_i rounded to
+// fp32 as the shader's pow() result is and the product taken exactly; the shader rounds delta * theta_i to fp32 before
+// its cos/sin, so the two differ by that one rounding of the angle (below 1.3e-4 rad at a distance of 2047, far inside
+// the tolerance that GLSL's own cos/sin precision needs).  The one-query kernels keep the per-pair form.
+// Then e = exp(s / sqrt(R)) without max subtraction (softmax.comp:33), out = sum e V / sum e (kqv_matching.comp:35-41),
+// K and V read back from the fp16 cache.  Without a running maximum there is nothing to rescale: both sums simply
+// accumulate over the tiles.
 //
-// One workgroup = one head x 32 query rows; it walks the cache in tiles of 64 positions staged through LDS, so
-// a K/V row is fetched once per 32 queries instead of once per query.
+// One workgroup = one head x 64 query rows, four waves = 2 query tiles x 2 position tiles of 32; the cache is walked
+// in tiles of 64 positions staged through LDS (K rotated, as fp32, x and y components apart; V transposed, fp16, even
+// and odd positions apart: both so that an MFMA operand is a run of consecutive LDS words per lane).
 #pragma once
 
 #include "lv_kernels.h"
 
 namespace lv {
 
-constexpr int kAttnBatchQ = 32;   // query rows per workgroup
+constexpr int kAttnBatchQ = 64;   // query rows per workgroup
 constexpr int kAttnBatchK = 64;   // cache positions per tile
 
 struct AttnBatchArgs {
@@ -22,119 +31,179 @@ struct AttnBatchArgs {
     const uint16_t *kcache; // [backlog][H*R] fp16
     const uint16_t *vcache;
     const float *q;         // [n][H*R]
-    const float2 *trig;     // [backlog][R/2] (cos, sin) of delta * theta_i
+    const float2 *trig_abs; // [backlog][R/2] (cos, sin) of p * theta_i
     const uint32_t *pos_ptr;
     uint32_t pos_add;       // row z of the batch sits at *pos_ptr + pos_add + z
     uint32_t n, heads, backlog;
 };
 
+typedef float lv_f32x16 __attribute__((ext_vector_type(16)));
+
 template <int R>
 struct AttnBatchLds {
-    float q[kAttnBatchQ][R + 4];                            // +4: rows stay 16-byte aligned and start in different banks
-    float k[kAttnBatchK][R + 2];                            // +2: neighbouring positions start in different banks
-    uint16_t v[kAttnBatchK][R];
-    float2 trig[kAttnBatchQ + kAttnBatchK][R / 2 + 1];      // rows: delta0 .. delta0 + 95
-    float p[kAttnBatchQ][kAttnBatchK + 1];
+    static constexpr int KP = R / 2 + 4;     // row stride of kx / ky in floats (16-byte aligned, rows start in different banks)
+    static constexpr int VP = kAttnBatchK / 2 + 8;   // row stride of vt in halfs
+    static constexpr int PP = 16 + 4;        // row stride of the probability tiles in floats
+    float kx[kAttnBatchK][KP], ky[kAttnBatchK][KP];   // rotated K: components 2i and 2i+1 of the pairs
+    uint16_t vt[2][R][VP];                   // V transposed: [position parity][dim][position / 2]
+    float ps[4][2][32][PP];                  // per wave: exp(score) [position parity][query row][position / 2]
+    float den[2][2][32];                     // [position tile][query tile][query row]
 };
 
 template <int R>
 __global__ __launch_bounds__(256) void attention_batch_kernel(AttnBatchArgs a)
 {
-    constexpr int TQ = kAttnBatchQ, TK = kAttnBatchK, DPT = R / 8;   // output dims per thread
-    __shared__ __attribute__((aligned(16))) AttnBatchLds<R> l;
+    constexpr int TQ = kAttnBatchQ, TK = kAttnBatchK;
+    constexpr int KS = R / 2;     // MFMA steps of a score tile (2 k each)
+    constexpr int DT = R / 32;    // 32-wide tiles of the head dimension
+    using L = AttnBatchLds<R>;
+    __shared__ __attribute__((aligned(16))) L l;
     const uint32_t h = blockIdx.x, z0 = blockIdx.y * TQ;
     const uint32_t H = a.heads, D = H * R;
     const uint32_t pos0 = (a.pos_ptr ? *a.pos_ptr : 0u) + a.pos_add;  // cache position of batch row 0
-    const int t = threadIdx.x;
-    const int zi = t >> 3, sub = t & 7;      // this thread's query row of the tile; its share of keys / dims
-    const uint32_t z = z0 + zi;
-    const bool zok = z < a.n;
-    const uint32_t my_pos = pos0 + z;        // own cache position
-    const uint32_t last_pos = min(pos0 + min(z0 + TQ, a.n) - 1, a.backlog - 1);  // newest position any row of the tile sees
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int qt = wave & 1, pt = wave >> 1;      // this wave's query tile and position sub-tile
+    const int n32 = lane & 31, hh = lane >> 5;
+    const uint32_t last_row = min(z0 + TQ, a.n) - 1;                  // last query row of the workgroup
+    const uint32_t last_pos = min(pos0 + last_row, a.backlog - 1);    // newest position any of them sees
 
-    for (int i = t; i < TQ * R / 4; i += 256) {
-        const int row = i / (R / 4), c4 = i % (R / 4);
-        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (z0 + row < a.n) v = *reinterpret_cast<const float4 *>(a.q + (size_t)(z0 + row) * D + (size_t)h * R + c4 * 4);
-        *reinterpret_cast<float4 *>(&l.q[row][c4 * 4]) = v;
+    // ---- this lane's query operands: row n32 of the wave's tile, rotated to its own position ------------------
+    // operand j of the score MFMAs is component 2j + hh of q' (hh = 0: x of pair j, hh = 1: y of pair j)
+    float qf[KS];
+    {
+        const uint32_t z = z0 + 32 * qt + n32;
+        const bool zok = z < a.n;
+        const uint32_t pq = min(pos0 + z, a.backlog - 1);
+        const float *qr = a.q + (size_t)(zok ? z : 0) * D + (size_t)h * R;
+        const float2 *tr = a.trig_abs + (size_t)pq * (R / 2);
+#pragma unroll
+        for (int j = 0; j < KS; j += 2) {
+            const float4 q2 = *reinterpret_cast<const float4 *>(qr + 2 * j);      // pairs j, j + 1
+            const float4 cs = *reinterpret_cast<const float4 *>(tr + j);          // (c, s) of pairs j, j + 1
+            // e^{i phi} (x + i y) = (x c - y s) + i (x s + y c)
+            const float x0 = q2.x * cs.x - q2.y * cs.y, y0 = q2.x * cs.y + q2.y * cs.x;
+            const float x1 = q2.z * cs.z - q2.w * cs.w, y1 = q2.z * cs.w + q2.w * cs.z;
+            qf[j] = zok ? (hh ? y0 : x0) : 0.f;
+            qf[j + 1] = zok ? (hh ? y1 : x1) : 0.f;
+        }
     }
 
     const float scale = rsqrtf((float)R);
-    float acc[DPT];
+    lv_f32x16 acc[DT];
 #pragma unroll
-    for (int i = 0; i < DPT; i++) acc[i] = 0.f;
-    float den = 0.f;
+    for (int d = 0; d < DT; d++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[d][r] = 0.f;
+    float den = 0.f;      // sum of this lane's probability operands: query row n32, positions of parity hh
 
     for (uint32_t k0 = 0; k0 <= last_pos; k0 += TK) {
-        __syncthreads();  // the previous tile is consumed (and l.q is written, first time round)
-        // ---- stage K (as fp32), V (fp16) and the rotation rows of this tile --------------------------------
+        __syncthreads();  // the previous tile is consumed
+        // ---- stage K (rotated, fp32) and V (transposed, fp16) of this tile ------------------------------------------
         for (int i = t; i < TK * R / 8; i += 256) {
             const int row = i / (R / 8), c8 = i % (R / 8);
             const uint32_t p = min(k0 + row, a.backlog - 1);
             const uint4 kraw = *reinterpret_cast<const uint4 *>(a.kcache + (size_t)p * D + (size_t)h * R + c8 * 8);
             const uint4 vraw = *reinterpret_cast<const uint4 *>(a.vcache + (size_t)p * D + (size_t)h * R + c8 * 8);
+            const float4 cs0 = *reinterpret_cast<const float4 *>(a.trig_abs + (size_t)p * (R / 2) + c8 * 4);
+            const float4 cs1 = *reinterpret_cast<const float4 *>(a.trig_abs + (size_t)p * (R / 2) + c8 * 4 + 2);
             const uint32_t kw[4] = {kraw.x, kraw.y, kraw.z, kraw.w};
+            const float c[4] = {cs0.x, cs0.z, cs1.x, cs1.z}, s[4] = {cs0.y, cs0.w, cs1.y, cs1.w};
+            float xr[4], yr[4];
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                l.k[row][c8 * 8 + 2 * j] = half_bits_to_float((uint16_t)(kw[j] & 0xffffu));
-                l.k[row][c8 * 8 + 2 * j + 1] = half_bits_to_float((uint16_t)(kw[j] >> 16));
+                const float x = half_bits_to_float((uint16_t)(kw[j] & 0xffffu)), y = half_bits_to_float((uint16_t)(kw[j] >> 16));
+                xr[j] = x * c[j] - y * s[j];
+                yr[j] = x * s[j] + y * c[j];
             }
-            *reinterpret_cast<uint4 *>(&l.v[row][c8 * 8]) = vraw;
-        }
-        // delta of (query row zi, tile position kj) = (pos0 + z0 + zi) - (k0 + kj) = base + zi + (TK - 1 - kj), base = pos0 + z0 - k0 - (TK - 1)
-        const int base = (int)(pos0 + z0) - (int)k0 - (TK - 1);
-        for (int i = t; i < (TQ + TK) * (R / 2); i += 256) {
-            const int row = i / (R / 2), c = i % (R / 2);
-            const int delta = base + row;
-            const int dc = delta < 0 ? 0 : (delta >= (int)a.backlog ? (int)a.backlog - 1 : delta);  // rows of masked pairs are never used
-            l.trig[row][c] = a.trig[(size_t)dc * (R / 2) + c];
-        }
-        __syncthreads();
-
-        // ---- scores: this thread does keys sub, sub + 8, ... of its query row ---------------------------------
-#pragma unroll 1
-        for (int m = 0; m < TK / 8; m++) {
-            const int kj = sub + 8 * m;
-            const uint32_t p = k0 + kj;
-            float e = 0.f;
-            if (zok && p <= my_pos && p < a.backlog) {
-                const float2 *tr = l.trig[zi + (TK - 1 - kj)];
-                float s = 0.f;
-#pragma unroll 8
-                for (int i = 0; i < R / 2; i++) {
-                    const float2 qq = *reinterpret_cast<const float2 *>(&l.q[zi][2 * i]);
-                    const float2 kk = *reinterpret_cast<const float2 *>(&l.k[kj][2 * i]);
-                    const float2 cs = tr[i];
-                    const float dotp = fmaf(qq.y, kk.y, qq.x * kk.x);
-                    const float crs = fmaf(qq.x, kk.y, -(qq.y * kk.x));
-                    s = fmaf(cs.x, dotp, s);
-                    s = fmaf(cs.y, crs, s);
-                }
-                e = __expf(s * scale);
-            }
-            l.p[zi][kj] = e;
-            den += e;
-        }
-        __syncthreads();
-
-        // ---- P.V: this thread owns dims sub*DPT .. +DPT-1 of its query row ------------------------------------
-        const uint32_t lim = min((uint32_t)TK, last_pos + 1 - k0);
-        for (uint32_t kj = 0; kj < lim; kj++) {
-            const float e = l.p[zi][kj];
-            const uint16_t *vr = &l.v[kj][sub * DPT];
+            *reinterpret_cast<float4 *>(&l.kx[row][c8 * 4]) = make_float4(xr[0], xr[1], xr[2], xr[3]);
+            *reinterpret_cast<float4 *>(&l.ky[row][c8 * 4]) = make_float4(yr[0], yr[1], yr[2], yr[3]);
+            const uint32_t vw[4] = {vraw.x, vraw.y, vraw.z, vraw.w};
 #pragma unroll
-            for (int i = 0; i < DPT; i++) acc[i] = fmaf(e, half_bits_to_float(vr[i]), acc[i]);
+            for (int j = 0; j < 4; j++) {
+                l.vt[row & 1][c8 * 8 + 2 * j][row >> 1] = (uint16_t)(vw[j] & 0xffffu);
+                l.vt[row & 1][c8 * 8 + 2 * j + 1][row >> 1] = (uint16_t)(vw[j] >> 16);
+            }
+        }
+        __syncthreads();
+
+        // ---- scores of (query tile qt) x (positions k0 + 32 pt ..): S = Q' K'^T ----------------------------------------
+        lv_f32x16 sc;
+#pragma unroll
+        for (int r = 0; r < 16; r++) sc[r] = 0.f;
+        {
+            const float *kr = hh ? &l.ky[32 * pt + n32][0] : &l.kx[32 * pt + n32][0];   // position n32 of the sub-tile
+#pragma unroll
+            for (int j = 0; j < KS; j += 4) {
+                const float4 k4 = *reinterpret_cast<const float4 *>(kr + j);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(qf[j], k4.x, sc, 0, 0, 0);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(qf[j + 1], k4.y, sc, 0, 0, 0);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(qf[j + 2], k4.z, sc, 0, 0, 0);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(qf[j + 3], k4.w, sc, 0, 0, 0);
+            }
+        }
+        // in sc a lane holds position n32 of the sub-tile and query rows i = 8 (r / 4) + 4 hh + r % 4
+        {
+            const uint32_t p = k0 + 32 * pt + n32;
+            float *prow = &l.ps[wave][n32 & 1][0][n32 >> 1];
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int i = 8 * (r / 4) + 4 * hh + (r % 4);
+                const uint32_t z = z0 + 32 * qt + i;
+                const bool ok = z < a.n && p <= pos0 + z && p < a.backlog;
+                prow[i * L::PP] = ok ? __expf(sc[r] * scale) : 0.f;
+            }
+        }
+        // ---- O += P V: the probabilities come back as the A operand (row = query n32, k = position 2j + hh) ------------
+        float pf[16];
+        {
+            const float *pr = &l.ps[wave][hh][n32][0];
+#pragma unroll
+            for (int j = 0; j < 16; j += 4) {
+                const float4 p4 = *reinterpret_cast<const float4 *>(pr + j);
+                pf[j] = p4.x; pf[j + 1] = p4.y; pf[j + 2] = p4.z; pf[j + 3] = p4.w;
+                den += (p4.x + p4.y) + (p4.z + p4.w);
+            }
+        }
+#pragma unroll
+        for (int d = 0; d < DT; d++) {
+            // B operand: V[position 32 pt + 2j + hh][dim 32 d + n32], sixteen consecutive halfs of the transposed tile
+            const uint16_t *vr = &l.vt[hh][32 * d + n32][16 * pt];
+            const uint4 va = *reinterpret_cast<const uint4 *>(vr), vb = *reinterpret_cast<const uint4 *>(vr + 8);
+            const uint32_t vw[8] = {va.x, va.y, va.z, va.w, vb.x, vb.y, vb.z, vb.w};
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                acc[d] = __builtin_amdgcn_mfma_f32_32x32x2f32(pf[2 * j], half_bits_to_float((uint16_t)(vw[j] & 0xffffu)), acc[d], 0, 0, 0);
+                acc[d] = __builtin_amdgcn_mfma_f32_32x32x2f32(pf[2 * j + 1], half_bits_to_float((uint16_t)(vw[j] >> 16)), acc[d], 0, 0, 0);
+            }
         }
     }
 
-    // the 8 threads of a query row hold partial denominators
-    den += __shfl_xor(den, 1, kWave);
-    den += __shfl_xor(den, 2, kWave);
-    den += __shfl_xor(den, 4, kWave);
-    if (zok) {
-        float *o = a.out + (size_t)z * D + (size_t)h * R + sub * DPT;
+    // ---- combine the two position tiles, divide, write -------------------------------------------------------------
+    den += __shfl_xor(den, 32, kWave);                    // both parities: all positions this wave saw, query row n32
+    if (hh == 0) l.den[pt][qt][n32] = den;
+    __syncthreads();                                      // also: every wave is done with kx / ky
+    static_assert(sizeof(l.kx) + sizeof(l.ky) >= (size_t)2 * DT * 16 * 64 * sizeof(float) && offsetof(L, ky) == offsetof(L, kx) + sizeof(l.kx),
+                  "the exchange area below spans kx and ky");
+    float *xch = &l.kx[0][0];                             // reused: [query tile][dim tile][register][lane]
+    if (pt == 1) {
 #pragma unroll
-        for (int i = 0; i < DPT; i++) o[i] = acc[i] / den;
+        for (int d = 0; d < DT; d++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) xch[((qt * DT + d) * 16 + r) * 64 + lane] = acc[d][r];
+    }
+    __syncthreads();
+    if (pt == 0) {
+#pragma unroll
+        for (int d = 0; d < DT; d++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int i = 8 * (r / 4) + 4 * hh + (r % 4);
+                const uint32_t z = z0 + 32 * qt + i;
+                if (z < a.n) {
+                    const float total = acc[d][r] + xch[((qt * DT + d) * 16 + r) * 64 + lane];
+                    a.out[(size_t)z * D + (size_t)h * R + 32 * d + n32] = total / (l.den[0][qt][i] + l.den[1][qt][i]);
+                }
+            }
     }
 }
 
