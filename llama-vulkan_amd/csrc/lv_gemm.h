@@ -123,13 +123,15 @@ __device__ __forceinline__ void gemm_codes_block(uint16_t *w, bool valid, const 
 // RM = weight rows per workgroup (128 or 64); tokens per workgroup: 128.  The four waves split the tile 2 x 2
 // (RM = 128: 64 tokens x 64 rows each) or 4 x 1 (RM = 64: 32 tokens x 64 rows each).  The narrow form doubles the
 // number of workgroups for matrices that would otherwise not fill 256 CUs.
-template <int QT, int RM>
-__global__ __launch_bounds__(256) void gemm_kernel(GemmArgs a)
+template <int QT, int RM, int NWV = 4>
+__global__ __launch_bounds__(NWV * 64) void gemm_kernel(GemmArgs a)
 {
     constexpr int CPB = QT == 4 ? 1 : 2;          // uint4 of codes per block
     constexpr int TN = kGemmTile;                 // tokens per workgroup
     constexpr int WN = RM / 64;                   // waves along the rows
-    constexpr int WM = 4 / WN;                    // waves along the tokens
+    constexpr int WM = NWV / WN;                  // waves along the tokens
+    constexpr int NT = NWV * 64;                  // threads
+    constexpr int XP = TN * 8 / NT;               // 16-byte pieces of an activation half-tile per thread
     constexpr int MT = TN / WM / 32;              // 32-token tiles per wave
     __shared__ __attribute__((aligned(16))) uint16_t sXh[TN * kGemmLd], sXl[TN * kGemmLd], sW[RM * kGemmLd];
     __shared__ float sD[2][RM];                   // scale of (block of the step, row)
@@ -145,6 +147,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs a)
     const bool wrow_ok = has_w && wrow < a.w.rows;
     // this thread's four 16-byte pieces of the activation tile of a step: token rows tid/8 + 32*i, halfs (tid%8)*8..+7
     const int xr = tid >> 3, xc = (tid & 7) * 8;
+    constexpr int XR = NT / 8;                    // token rows covered per piece index
 
     // two register sets: the loads of step s + 2 are in flight while step s is multiplied (one step of MFMAs is
     // shorter than a trip to memory)
@@ -152,7 +155,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs a)
         uint4 c0, c1;
         uint16_t dbits;
         bool wvalid;
-        uint4 gh[4], gl[4];
+        uint4 gh[XP], gl[XP];
     } pre[2];
     auto fetch = [&](Staged &p, uint32_t step) {
         const uint32_t blk = 2 * step + b_w;
@@ -168,8 +171,8 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs a)
         const uint32_t k = step * kGemmK + xc;
         const bool kok = k < K;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const size_t off = (size_t)(tok0 + xr + 32 * i) * K + (kok ? k : 0);
+        for (int i = 0; i < XP; i++) {
+            const size_t off = (size_t)(tok0 + xr + XR * i) * K + (kok ? k : 0);
             p.gh[i] = *reinterpret_cast<const uint4 *>(a.xh + off);
             p.gl[i] = *reinterpret_cast<const uint4 *>(a.xl + off);
             if (!kok) p.gh[i] = p.gl[i] = make_uint4(0, 0, 0, 0);
@@ -193,9 +196,9 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs a)
             sD[b_w][r_w] = P.wvalid ? half_bits_to_float(P.dbits) : 0.f;
         }
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            *reinterpret_cast<uint4 *>(sXh + (xr + 32 * i) * kGemmLd + xc) = P.gh[i];
-            *reinterpret_cast<uint4 *>(sXl + (xr + 32 * i) * kGemmLd + xc) = P.gl[i];
+        for (int i = 0; i < XP; i++) {
+            *reinterpret_cast<uint4 *>(sXh + (xr + XR * i) * kGemmLd + xc) = P.gh[i];
+            *reinterpret_cast<uint4 *>(sXl + (xr + XR * i) * kGemmLd + xc) = P.gl[i];
         }
         __syncthreads();
         if (step + 2 < steps) fetch(P, step + 2);
