@@ -202,3 +202,15 @@ def test_c_abi_exports_every_declared_symbol(lva):
     assert len(names) >= 40
     for n in names:
         assert hasattr(lib, n), f"include/llava_hip.h declares {n} but libllava_hip.so does not export it"
+
+
+def test_every_python_file_of_the_package_compiles():
+    """measure.py, build.py and bench.py only run on a GPU box: a syntax error in them must not wait for one"""
+    import glob
+    import py_compile
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    files = glob.glob(os.path.join(root, "*.py")) + glob.glob(os.path.join(root, "llama-vulkan_amd", "*.py")) + \
+        glob.glob(os.path.join(root, "oracle", "*.py")) + glob.glob(os.path.join(root, "tests", "**", "*.py"), recursive=True)
+    assert len(files) > 10
+    for f in files:
+        py_compile.compile(f, doraise=True)
