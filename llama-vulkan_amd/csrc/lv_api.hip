@@ -1394,15 +1394,17 @@ extern "C" int lv_step_begin(lv_session *s, const uint32_t *tokens, uint32_t n, 
 
     int path = LV_PATH_AUTO;
     (void)lv_session_path(s, &path);
-    const bool persistent = n == 1 && path == LV_PATH_PERSISTENT && !s->trace;
+    // the persistent kernel also takes the short steps (a few prompt or add_text tokens) below the size at which the
+    // batched path pays: one launch per token, each 1.7 x faster than the operator chain's token
+    const bool persistent = n < kPrefillMin && path == LV_PATH_PERSISTENT && !s->trace;
     if (!persistent) {             // the persistent kernel takes position and token id as launch arguments
         s->cfg_host[0] = pos;
         memcpy(s->cfg_host + 1, tokens, (size_t)n * 4);
         HIP_TRY(hipMemcpyAsync(s->cfg, s->cfg_host, (size_t)(1 + n) * 4, hipMemcpyHostToDevice, s->stream));
     }
     if (persistent) {
-        LV_TRY(launch_mega(s, pos, tokens[0]));
-        s->pick_in_status = true;  // the kernel leaves the greedy pick in the pinned status block
+        for (uint32_t i = 0; i < n; i++) LV_TRY(launch_mega(s, pos + i, tokens[i]));
+        s->pick_in_status = true;  // the kernel leaves the greedy pick (of the last token) in the pinned status block
     } else if (n == 1 && (path == LV_PATH_GRAPH || (path == LV_PATH_PERSISTENT && s->use_graph)) && !s->trace) {
         if (!s->graph_exec) {
             HIP_TRY(hipStreamBeginCapture(s->stream, hipStreamCaptureModeThreadLocal));

@@ -174,7 +174,7 @@ def test_persistent_kernel_matches_oracle_and_operator_path(lva, orc, ctx, wide_
     ops.set_path(lva.PATH_KERNELS)
     prompt = lva.synth_tokens(8, 3, 2048, seed=1)
     want = osess.eval(prompt)
-    pk.begin(prompt, 0)                               # prompts go through the operator path in both sessions
+    pk.begin(prompt, 0)                               # a short prompt: one persistent launch per token
     ops.begin(prompt, 0)
     got_pk, got_ops = pk.logits(), ops.logits()
     _check_logits(got_pk, want)
