@@ -105,11 +105,17 @@ int lv_session_use_graph(lv_session *s, int enable);
  * llava_command_buffer.cpp:47-55); here there are three, all computing the same step:
  *   LV_PATH_KERNELS     one launch per operator on the session's stream
  *   LV_PATH_GRAPH       the same launches captured once into a hipGraph and replayed
- *   LV_PATH_PERSISTENT  one persistent kernel for the whole token (7B-class q4_0 models on a 256-CU device)
+ *   LV_PATH_PERSISTENT  one persistent kernel for the whole token (LLaMA-7B and -13B layer shapes, q4_0 or q8_0, on a
+ *                       256-CU device)
  *   LV_PATH_AUTO        persistent when the model has that form, else graph (or kernels if graphs are off) */
 enum { LV_PATH_AUTO = 0, LV_PATH_KERNELS = 1, LV_PATH_GRAPH = 2, LV_PATH_PERSISTENT = 3 };
 int lv_session_set_path(lv_session *s, int path);
 int lv_session_path(const lv_session *s, int *path);
+/* Workgroups of the persistent kernel wait for each other's results by polling, a bounded number of times; a wait
+ * that runs out makes the kernel finish anyway and lv_step_wait return LV_ERR_HIP (the reference's waitForFences
+ * timeout, llava_command_buffer.cpp:25-27, is the nearest counterpart).  polls = 0 restores the default bound; tests of
+ * that failure path set 1.  The step can simply be issued again afterwards. */
+int lv_session_set_wait_limit(lv_session *s, uint32_t polls);
 
 /* ---- cache dump / restore: replaces llava_layer_session_data::dump_kv_cache / restore_kv_cache
  *      (llava_layer_session_data.cpp:165-181).  which: 0 = K, 1 = V.  n_tokens rows of `dim` fp16 values. */

@@ -91,6 +91,7 @@ _HIP_SIGS = {
     "lv_session_backlog": [_VP, C.POINTER(_U32)],
     "lv_session_use_graph": [_VP, _I],
     "lv_session_set_path": [_VP, _I],
+    "lv_session_set_wait_limit": [_VP, C.c_uint32],
     "lv_session_path": [_VP, C.POINTER(_I)],
     "lv_step_begin": [_VP, _VP, _U32, _U32],
     "lv_step_wait": [_VP],
@@ -352,6 +353,9 @@ class Session:
 
     def set_path(self, path):
         check(self.lib.lv_session_set_path(self.h, int(path)))
+
+    def set_wait_limit(self, polls):
+        check(self.lib.lv_session_set_wait_limit(self.h, int(polls)))
 
     def path(self):
         p = C.c_int()

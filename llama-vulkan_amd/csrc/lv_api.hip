@@ -153,6 +153,7 @@ struct lv_session {
     float *xchg[2] = {nullptr, nullptr};  // hand-over buffer sets of the persistent kernel
     uint32_t xchg_turn = 0;
     uint32_t *status_host = nullptr;      // pinned, written by the persistent kernel: [0] a poll expired, [kStatusToken] greedy pick
+    uint32_t wait_limit = 0;              // polls per hand-over of the persistent kernel; 0 = default
     bool pick_in_status = false;          // the last step ran the persistent kernel, whose greedy pick is in status_host
     bool in_flight = false;
     bool have_logits = false;
@@ -1203,6 +1204,7 @@ static int launch_mega(lv_session *s, uint32_t pos, uint32_t token)
     a.logits = s->logits;
     a.status = s->status_host;
     a.layers = m->hp.layers; a.vocab = m->hp.vocab; a.backlog = s->backlog; a.pos = pos; a.token = token;
+    a.spin_limit = s->wait_limit ? s->wait_limit : kSpinLimit;
     s->xchg_turn++;
     void *params[] = {&a};
     return mega_dispatch(m->mega_kind, [&](auto shape) -> int {
@@ -1471,6 +1473,13 @@ extern "C" int lv_argmax(lv_session *s, uint32_t *token)
     HIP_TRY(hipMemcpyAsync(s->argmax_host, s->argmax_dev, 4, hipMemcpyDeviceToHost, s->stream));
     LV_TRY(lv_step_wait(s));
     *token = *s->argmax_host;
+    return LV_OK;
+}
+
+extern "C" int lv_session_set_wait_limit(lv_session *s, uint32_t polls)
+{
+    if (!s) return fail(LV_ERR_ARG, "lv_session_set_wait_limit: session is null");
+    s->wait_limit = polls;
     return LV_OK;
 }
 

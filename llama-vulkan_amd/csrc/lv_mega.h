@@ -34,7 +34,7 @@ namespace lv {
 constexpr uint32_t kNotReady = 0xFFFFFFFFu;
 constexpr int kMegaWGs = 256;
 constexpr int kMegaVocabRows = 125;     // output-matrix rows per workgroup the head phase is laid out for (32000 / 256)
-constexpr uint32_t kSpinLimit = 1u << 20;
+constexpr uint32_t kSpinLimit = 1u << 20;   // default bound on the polls of one hand-over (MegaArgs::spin_limit)
 constexpr int kStatusToken = 2;         // word of the status block that receives the index of the largest logit
 // A consumer reaches a hand-over about when its producers store: a load issued at once samples memory before the
 // stores are visible (0.6 us) yet comes back only after the prefetched tiles ahead of it on the CU's return path
@@ -108,6 +108,7 @@ struct MegaArgs {
     float *logits;             // [vocab]
     uint32_t *status;          // host-visible; [0] set non-zero when a poll loop expired, [kStatusToken] = greedy pick
     uint32_t layers, vocab, backlog, pos, token;
+    uint32_t spin_limit;       // polls per hand-over before the step is given up (kSpinLimit; tests of the failure path lower it)
 };
 
 // Optional phase timestamps (built only with -DLV_MEGA_TIMING): workgroup 0 records the 100 MHz wall clock at
@@ -153,7 +154,7 @@ __device__ __forceinline__ float tile_dot(const MegaTile &t, const float (&xr)[3
 // N values strided by `stride` elements starting at p; spins until none of them is the not-ready pattern.
 template <int N, int SLEEP = 0>
 __device__ __forceinline__ void poll_values(float (&v)[N], const float *p, int stride, const bool (&want)[N], uint32_t *status,
-                                            int group_stride = 0 /* when non-zero: element j lives at p[(j/8)*8*group_stride + j%8] */)
+                                            uint32_t spin_limit, int group_stride = 0 /* when non-zero: element j lives at p[(j/8)*8*group_stride + j%8] */)
 {
     uint32_t spins = 0;
     bool pending;
@@ -168,7 +169,7 @@ __device__ __forceinline__ void poll_values(float (&v)[N], const float *p, int s
             v[j] = __uint_as_float(u);
             pending |= (u == kNotReady);
         }
-    } while (pending && ++spins < kSpinLimit);
+    } while (pending && ++spins < spin_limit);
     if (pending) *status = 1u;
 }
 
@@ -328,7 +329,7 @@ __device__ __forceinline__ float block_sum(float v, float *scratch /* NW floats 
 // (normalize.comp:34-64: mean, then mean-centred variance, no epsilon) with weights w.  One round trip to
 // memory when the data is there: the norm weights are requested before the wait, not after it.
 template <int N, int NW, bool NORM, int SLEEP = 0>
-__device__ __forceinline__ void acquire_vector(float *xs, const float *src, const float *w, float *scratch, uint32_t *status)
+__device__ __forceinline__ void acquire_vector(float *xs, const float *src, const float *w, float *scratch, uint32_t *status, uint32_t spin_limit)
 {
     constexpr int T = NW * 64, PER = cdiv(N, T);
     float v[PER];
@@ -340,7 +341,7 @@ __device__ __forceinline__ void acquire_vector(float *xs, const float *src, cons
 #pragma unroll
         for (int j = 0; j < PER; j++) wn[j] = want[j] ? w[threadIdx.x + j * T] : 0.f;
     }
-    poll_values<PER, SLEEP>(v, src + threadIdx.x, T, want, status);
+    poll_values<PER, SLEEP>(v, src + threadIdx.x, T, want, status, spin_limit);
     if constexpr (NORM) {
         float s = 0.f;
 #pragma unroll
@@ -378,6 +379,7 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
     const int b = mw.b, w = mw.w, lane = mw.lane;
     const int st = threadIdx.x;
     uint32_t *status = a.status;
+    const uint32_t spin_limit = a.spin_limit;
 
     // ---- start the weight stream ------------------------------------------------------------------------------
     MegaTile q[S::DEPTH];
@@ -408,7 +410,7 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
 
         // ================= A: norm + QKV ====================================================================
         MEGA_STAMP(0);
-        acquire_vector<D, NW, true, kPollDelay>(xs, x_src, norm_w, scratch, status);
+        acquire_vector<D, NW, true, kPollDelay>(xs, x_src, norm_w, scratch, status, spin_limit);
         MEGA_STAMP(1);
         load_slab(xr, xsum, xs, mw.sD * 64 + lane, mw.laneD);
         gemv_phase<S, S::SEQ_A, S::TA, S::NSD>(q, mw, layer, xr, xsum, mw.sD, mw.rD, mw.actD, S::ROWS_A, red);
@@ -470,7 +472,7 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
                     bool want24[24];
 #pragma unroll
                     for (int i = 0; i < 24; i++) want24[i] = i < 8 || newest;
-                    poll_values<24, kPollDelay>(qkv, xc + S::OFF_QKV + h * R + sub * 8, 1, want24, status, D / 8);
+                    poll_values<24, kPollDelay>(qkv, xc + S::OFF_QKV + h * R + sub * 8, 1, want24, status, spin_limit, D / 8);
                 }
                 MEGA_STAMP(3);
                 const float scale = rsqrtf((float)R);
@@ -563,7 +565,7 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
                     nd[S::CPH + c] = __uint_as_float(ud);
                     pending |= (un == kNotReady) | (ud == kNotReady);
                 }
-            } while (pending && ++spins < kSpinLimit);
+            } while (pending && ++spins < spin_limit);
             if (pending) *status = 1u;
             float n = 0.f, d = 0.f;
 #pragma unroll
@@ -573,7 +575,7 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
 
         // ================= C: x += Wo o ============================================================================
         MEGA_STAMP(5);
-        acquire_vector<D, NW, false, kPollDelay>(xs, xc + S::OFF_O, nullptr, scratch, status);
+        acquire_vector<D, NW, false, kPollDelay>(xs, xc + S::OFF_O, nullptr, scratch, status, spin_limit);
         MEGA_STAMP(6);
         load_slab(xr, xsum, xs, mw.sD * 64 + lane, mw.laneD);
         gemv_phase<S, S::SEQ_C, S::TC, S::NSD>(q, mw, layer, xr, xsum, mw.sD, mw.rD, mw.actD, S::ROWS_C, red);
@@ -586,7 +588,7 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
 
         // ================= D: norm + SwiGLU ========================================================================
         MEGA_STAMP(7);
-        acquire_vector<D, NW, true, kPollDelay>(xs, xc + S::OFF_X1, norm_w + D, scratch, status);
+        acquire_vector<D, NW, true, kPollDelay>(xs, xc + S::OFF_X1, norm_w + D, scratch, status, spin_limit);
         MEGA_STAMP(8);
         load_slab(xr, xsum, xs, mw.sD * 64 + lane, mw.laneD);
         gemv_phase<S, S::SEQ_D, S::TD, S::NSD>(q, mw, layer, xr, xsum, mw.sD, mw.rD, mw.actD, S::ROWS_D, red);
@@ -599,7 +601,7 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
 
         // ================= E: x += W2 ff ===========================================================================
         MEGA_STAMP(9);
-        acquire_vector<F, NW, false, kPollDelay>(xs, xc + S::OFF_FF, nullptr, scratch, status);
+        acquire_vector<F, NW, false, kPollDelay>(xs, xc + S::OFF_FF, nullptr, scratch, status, spin_limit);
         MEGA_STAMP(10);
         load_slab(xr, xsum, xs, mw.sF * 64 + lane, mw.laneF);
         gemv_phase<S, S::SEQ_E, S::TE, S::NSF>(q, mw, layer, xr, xsum, mw.sF, mw.rF, mw.actF, S::ROWS_E, red);
@@ -618,7 +620,7 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
 
     // ================= head: norm + output matrix ====================================================================
     {
-        acquire_vector<D, NW, true, kPollDelay>(xs, x_src, a.norms + (size_t)a.layers * 2 * D, scratch, status);
+        acquire_vector<D, NW, true, kPollDelay>(xs, x_src, a.norms + (size_t)a.layers * 2 * D, scratch, status, spin_limit);
         load_slab(xr, xsum, xs, mw.sD * 64 + lane, mw.laneD);
         const int rows = (int)mw.vocab_rows, per_set = (rows + S::NRD - 1) / S::NRD;
         // the head's slots are numbered from 0; tiles beyond per_set read the dummy tile
@@ -685,7 +687,7 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
             if (st < kMegaWGs) {
                 float pair[2];
                 const bool want2[2] = {true, true};
-                poll_values<2, kPollDelay>(pair, cand + 2 * st, 1, want2, status);
+                poll_values<2, kPollDelay>(pair, cand + 2 * st, 1, want2, status, spin_limit);
                 const uint32_t oi = __float_as_uint(pair[1]);
                 if (oi < kNotReady - 1) { bv = pair[0]; bi = oi; }
             }

@@ -254,3 +254,29 @@ def test_quantised_embedding_table_all_paths(lva, orc, ctx, tmp_path, wname, tna
         pk.begin([tok], pos); ops.begin([tok], pos)
         pos += 1
     pk.close(); ops.close(); model.close(); osess.close(); om.close()
+
+
+def test_persistent_kernel_gives_up_a_wait_and_the_step_can_be_repeated(lva, orc, ctx, wide_model):
+    """failure path: with the poll bound set to 1 the workgroups stop waiting for each other at once; the kernel still
+    runs to its end (nothing hangs), the step is reported as failed, and the same step issued again with the default
+    bound gives the oracle's result"""
+    om = orc.Model(wide_model)
+    osess = orc.Session(om, 128)
+    model = lva.Model(ctx, wide_model)
+    s = lva.Session(model, 128)
+    assert s.path() == lva.PATH_PERSISTENT
+    prompt = lva.synth_tokens(4, 3, 2048, seed=3)
+    want = osess.eval(prompt)
+    s.begin(prompt, 0)
+    _check_logits(s.logits(), want)
+    tok = orc.greedy(want)
+    s.set_wait_limit(1)
+    s.begin([tok], 4)
+    with pytest.raises(lva.LvError):
+        s.wait()
+    s.set_wait_limit(0)
+    want = osess.eval([tok])
+    s.begin([tok], 4)                 # the same cache row again
+    _check_logits(s.logits(), want)
+    assert s.argmax() == orc.greedy(want)
+    s.close(); model.close(); osess.close(); om.close()
