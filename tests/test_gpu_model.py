@@ -280,3 +280,30 @@ def test_persistent_kernel_gives_up_a_wait_and_the_step_can_be_repeated(lva, orc
     _check_logits(s.logits(), want)
     assert s.argmax() == orc.greedy(want)
     s.close(); model.close(); osess.close(); om.close()
+
+
+@pytest.mark.parametrize("vocab", [259, 2049])
+def test_vocabulary_sizes_that_do_not_divide_over_the_workgroups(lva, orc, ctx, tmp_path, vocab):
+    """the output matrix is split over 256 workgroups; 2049 rows leave the last ones short, 259 leave most of them
+    without a row (their 'best logit' must not be mistaken for one): logits and greedy pick on both decode paths"""
+    p = str(tmp_path / "odd.ggml")
+    lva.write_model(p, wtype=lva.LV_Q4_0, seed=5, vocab=vocab, layers=2, dim=4096, heads=32, ff=11008)
+    om = orc.Model(p)
+    osess = orc.Session(om, 128)
+    model = lva.Model(ctx, p)
+    pk, ops = lva.Session(model, 128), lva.Session(model, 128)
+    assert pk.path() == lva.PATH_PERSISTENT
+    ops.set_path(lva.PATH_GRAPH)
+    prompt = lva.synth_tokens(5, 3, vocab, seed=2)
+    want = osess.eval(prompt)
+    pk.begin(prompt, 0); ops.begin(prompt, 0)
+    pos = len(prompt)
+    for step in range(4):
+        _check_logits(pk.logits(), want)
+        _check_logits(ops.logits(), want)
+        tok = orc.greedy(want)
+        assert pk.argmax() == tok == ops.argmax(), step
+        want = osess.eval([tok])
+        pk.begin([tok], pos); ops.begin([tok], pos)
+        pos += 1
+    pk.close(); ops.close(); model.close(); osess.close(); om.close()
