@@ -307,3 +307,29 @@ def test_vocabulary_sizes_that_do_not_divide_over_the_workgroups(lva, orc, ctx, 
         pk.begin([tok], pos); ops.begin([tok], pos)
         pos += 1
     pk.close(); ops.close(); model.close(); osess.close(); om.close()
+
+
+def test_persistent_kernel_up_to_the_last_cache_row(lva, orc, ctx, wide_model):
+    """every position of a 128-row cache, the last one included (chunk boundaries of the attention phase move with the
+    position); a step past the end is refused"""
+    om = orc.Model(wide_model)
+    osess = orc.Session(om, 128)
+    model = lva.Model(ctx, wide_model)
+    s = lva.Session(model, 128)
+    assert s.path() == lva.PATH_PERSISTENT
+    prompt = lva.synth_tokens(3, 3, 2048, seed=4)
+    want = osess.eval(prompt)
+    s.begin(prompt, 0)
+    pos = len(prompt)
+    while True:
+        _check_logits(s.logits(), want)
+        tok = orc.greedy(want)
+        assert s.argmax() == tok, pos
+        if pos == 128:
+            break
+        want = osess.eval([tok])
+        s.begin([tok], pos)
+        pos += 1
+    with pytest.raises(lva.LvError):
+        s.begin([tok], 128)
+    s.close(); model.close(); osess.close(); om.close()
