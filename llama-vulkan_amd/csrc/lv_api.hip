@@ -13,6 +13,7 @@
 #include <cstdio>
 #include <cstring>
 #include <map>
+#include <mutex>
 #include <new>
 #include <string>
 #include <vector>
@@ -68,6 +69,12 @@ struct lv_ctx {
     uint32_t *attn_counters = nullptr;
     size_t attn_part_floats = 0, attn_counter_words = 0;
     hipEvent_t ev_start = nullptr, ev_stop = nullptr;
+    // Persistent decode kernels of different sessions (one per thread, llava_context.h:47-49 has the same pools and
+    // mutexes for the same reason) must not overlap on the device: each occupies every CU and its workgroups wait
+    // for each other.  A launch on another session's stream first waits for the event the last launch recorded.
+    std::mutex mega_mutex;
+    hipEvent_t mega_done = nullptr;
+    const void *mega_last = nullptr;      // session whose launch mega_done belongs to
 };
 
 struct lv_matrix {
@@ -202,6 +209,7 @@ extern "C" int lv_ctx_destroy(lv_ctx *c)
     (void)hipFree(c->attn_counters);
     if (c->ev_start) (void)hipEventDestroy(c->ev_start);
     if (c->ev_stop) (void)hipEventDestroy(c->ev_stop);
+    if (c->mega_done) (void)hipEventDestroy(c->mega_done);
     (void)hipStreamDestroy(c->stream);
     delete c;
     return LV_OK;
@@ -1036,6 +1044,10 @@ extern "C" int lv_session_destroy(lv_session *s)
     if (!s) return LV_OK;
     (void)hipSetDevice(s->model->ctx->device);
     if (s->stream) (void)hipStreamSynchronize(s->stream);
+    {
+        std::lock_guard<std::mutex> lock(s->model->ctx->mega_mutex);
+        if (s->model->ctx->mega_last == s) s->model->ctx->mega_last = nullptr;   // its last launch has finished (stream synchronised)
+    }
     drop_graph(s);
     void *dev[] = {s->kv, s->trig, s->trig_abs, s->x, s->xn, s->q, s->k, s->v, s->vo, s->ff, s->logits, s->attn_part, s->attn_counters,
                    s->cfg, s->argmax_dev, s->trace_buf, s->pf_x, s->pf_xn, s->pf_q, s->pf_k, s->pf_v, s->pf_vo, s->pf_g1, s->pf_g2,
@@ -1207,12 +1219,19 @@ static int launch_mega(lv_session *s, uint32_t pos, uint32_t token)
     a.spin_limit = s->wait_limit ? s->wait_limit : kSpinLimit;
     s->xchg_turn++;
     void *params[] = {&a};
-    return mega_dispatch(m->mega_kind, [&](auto shape) -> int {
+    lv_ctx *c = m->ctx;
+    std::lock_guard<std::mutex> lock(c->mega_mutex);
+    if (c->mega_last && c->mega_last != s) HIP_TRY(hipStreamWaitEvent(s->stream, c->mega_done, 0));
+    LV_TRY(mega_dispatch(m->mega_kind, [&](auto shape) -> int {
         using S = decltype(shape);
         HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<const void *>(&mega_decode_kernel<S>), dim3(kMegaWGs), dim3(S::NW * 64), params, 0,
                                            s->stream));
         return LV_OK;
-    });
+    }));
+    if (!c->mega_done) HIP_TRY(hipEventCreateWithFlags(&c->mega_done, hipEventDisableTiming));
+    HIP_TRY(hipEventRecord(c->mega_done, s->stream));
+    c->mega_last = s;
+    return LV_OK;
 }
 
 // -----------------------------------------------------------------------------------------------------------

@@ -34,7 +34,10 @@ namespace lv {
 constexpr uint32_t kNotReady = 0xFFFFFFFFu;
 constexpr int kMegaWGs = 256;
 constexpr int kMegaVocabRows = 125;     // output-matrix rows per workgroup the head phase is laid out for (32000 / 256)
-constexpr uint32_t kSpinLimit = 1u << 20;   // default bound on the polls of one hand-over (MegaArgs::spin_limit)
+// Default bound on the polls of one hand-over (MegaArgs::spin_limit).  A hand-over normally takes one to three polls of
+// about 1.3 us; 16384 of them (20 ms) only run out when the workgroups are not all resident, and a token whose every
+// hand-over ran out still ends within seconds.
+constexpr uint32_t kSpinLimit = 1u << 14;
 constexpr int kStatusToken = 2;         // word of the status block that receives the index of the largest logit
 // A consumer reaches a hand-over about when its producers store: a load issued at once samples memory before the
 // stores are visible (0.6 us) yet comes back only after the prefetched tiles ahead of it on the CU's return path

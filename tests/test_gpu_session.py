@@ -258,3 +258,40 @@ def test_cli_prints_the_greedy_continuation(hl, orc, loaded):
     assert r.returncode != 0                       # the server mode is not part of this build
     r = subprocess.run([exe, "-m", path + ".absent", "hi"], capture_output=True, timeout=60)
     assert r.returncode != 0 and b"absent" in r.stderr
+
+
+def test_two_threads_two_sessions_one_model(lva, orc, ctx, tmp_path):
+    """the reference's threading contract (one session per thread, sessions share the context and the weights,
+    llava_context.h:47-49): two threads decode at the same time on the persistent kernel, whose launches must take
+    turns on the device; both must produce what a lone session produces"""
+    import threading
+    p = str(tmp_path / "two.ggml")
+    lva.write_model(p, wtype=lva.LV_Q4_0, seed=13, vocab=2048, layers=2, dim=4096, heads=32, ff=11008)
+    model = lva.Model(ctx, p)
+
+    def run(seed, out):
+        s = lva.Session(model, 128)
+        assert s.path() == lva.PATH_PERSISTENT
+        prompt = lva.synth_tokens(4, 3, 2048, seed=seed)
+        s.begin(prompt, 0)
+        toks, pos = [], 4
+        for _ in range(60):
+            t = s.argmax()
+            toks.append(t)
+            s.begin([t], pos)
+            pos += 1
+        toks.append(s.argmax())
+        s.close()
+        out.extend(toks)
+
+    alone = [[], []]
+    for i in range(2):
+        run(20 + i, alone[i])
+    together = [[], []]
+    threads = [threading.Thread(target=run, args=(20 + i, together[i])) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert together == alone
+    model.close()
