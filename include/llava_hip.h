@@ -62,7 +62,7 @@ typedef struct {
 } lv_tensor_desc;
 
 typedef struct {
-    uint32_t file_version;   /* only 3 (fp16 block scales) is accepted for quantised tensors */
+    uint32_t file_version;   /* 3 (fp16 block scales) or 1 (fp32 block scales, interleaved q4_0 nibbles) */
     uint32_t vocab, dim, heads, layers, rot, ff;
 } lv_hparams;
 
@@ -155,11 +155,13 @@ int lv_session_timer_stop(lv_session *s, float *ms);
 
 /* A quantised matrix in the device layout.  Built from GGML blocks by lv_matrix_upload; owns its memory. */
 typedef struct lv_matrix lv_matrix;
-/* replaces llava_buffer::load_from_disk for one tensor (llava_buffer.cpp:179-325) */
+/* replaces llava_buffer::load_from_disk for one tensor (llava_buffer.cpp:179-325).  file_version 3: 18 / 34-byte blocks
+ * with an fp16 scale; file_version 1 (llava_buffer.cpp:193-224, ggml_file.cpp:171-183): 20 / 36-byte blocks with an fp32
+ * scale, q4_0 byte j holding elements 2j and 2j+1; the device keeps an fp32 scale plane for such a matrix. */
 int lv_matrix_upload(lv_ctx *ctx, const void *ggml_blocks, uint32_t ftype, uint32_t file_version, uint32_t rows,
                      uint32_t cols, lv_matrix **out);
 int lv_matrix_destroy(lv_matrix *m);
-/* bytes the device layout occupies (equals the GGML payload size: 18 / 34 bytes per 32 weights) */
+/* bytes the device layout occupies (equals the GGML payload size: 18 / 34 bytes per 32 weights, 20 / 36 for file version 1) */
 int lv_matrix_bytes(const lv_matrix *m, uint64_t *bytes);
 
 /* ---- single kernels on the context's stream; all pointers are device pointers.  Asynchronous: follow with

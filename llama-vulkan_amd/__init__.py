@@ -269,8 +269,10 @@ def synth_tokens(n, lo, hi, seed):
 # GGJT table reader for Python callers of the C-ABI (the C++ ggml_file class is the product parser; this is
 # the same 40 lines of format knowledge for scripts that hand lv_model_upload a table)
 # ----------------------------------------------------------------------------------------------------------
-def _tensor_bytes(ftype, n):
-    return {LV_F32: n * 4, LV_F16: n * 2, LV_Q4_0: n // 32 * 18, LV_Q8_0: n // 32 * 34}[ftype]
+def _tensor_bytes(ftype, n, file_version=3):
+    """file version 1 stores fp32 block scales, later versions fp16 ones (reference: ggml_file.cpp:95-122)"""
+    wide = 2 if file_version == 1 else 0
+    return {LV_F32: n * 4, LV_F16: n * 2, LV_Q4_0: n // 32 * (18 + wide), LV_Q8_0: n // 32 * (34 + wide)}[ftype]
 
 
 def read_ggjt_table(path):
@@ -296,7 +298,7 @@ def read_ggjt_table(path):
         cur += name_len
         rows, cols = (ne[1], ne[0]) if n_dims == 2 else (ne[0], 1)
         offset = (cur + 31) & ~31
-        size = _tensor_bytes(ftype, rows * cols)
+        size = _tensor_bytes(ftype, rows * cols, header["file_version"])
         table.append((name, ftype, offset, rows, cols, size))
         cur = offset + size
     for name, _, _, rows, _, _ in table:

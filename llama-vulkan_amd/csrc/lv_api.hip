@@ -345,13 +345,15 @@ extern "C" int lv_dev_copy(lv_ctx *c, void *dst, const void *src, uint64_t bytes
 // -----------------------------------------------------------------------------------------------------------
 // matrices
 // -----------------------------------------------------------------------------------------------------------
-static uint64_t ggml_bytes(uint32_t ftype, uint64_t n)
+// bytes of n elements in the file (ggml_file.cpp:162-186): version-1 files carry fp32 block scales, 2 bytes more a block
+static uint64_t ggml_bytes(uint32_t ftype, uint64_t n, uint32_t file_version)
 {
+    const uint64_t wide = file_version == 1 ? 2 : 0;
     switch (ftype) {
     case LV_F32: return n * 4;
     case LV_F16: return n * 2;
-    case LV_Q4_0: return n / 32 * 18;
-    case LV_Q8_0: return n / 32 * 34;
+    case LV_Q4_0: return n / 32 * (18 + wide);
+    case LV_Q8_0: return n / 32 * (34 + wide);
     default: return 0;
     }
 }
@@ -363,30 +365,37 @@ static uint64_t align_up(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
 
 // Copies one GGML-format quantised tensor to `dst` (device, 256-byte aligned, matrix_device_bytes long)
 // through a device staging buffer and splits it there.
-static uint64_t matrix_device_bytes(uint32_t ftype, uint64_t rows, uint64_t cols)
+static uint64_t matrix_device_bytes(uint32_t ftype, uint64_t rows, uint64_t cols, uint32_t file_version)
 {
     const uint64_t nblk = rows * (cols / 32);
-    return align_up(codes_bytes(ftype, nblk), 256) + align_up(nblk * 2, 256);
+    return align_up(codes_bytes(ftype, nblk), 256) + align_up(nblk * (file_version == 1 ? 4 : 2), 256);
 }
 
 static int place_matrix(lv_ctx *c, lv_matrix *m, uint8_t *dst, const void *host_blocks, uint32_t ftype, uint32_t rows,
-                        uint32_t cols, uint8_t *staging)
+                        uint32_t cols, uint8_t *staging, uint32_t file_version)
 {
     const uint64_t nblk = (uint64_t)rows * (cols / 32);
-    const uint64_t raw = ggml_bytes(ftype, (uint64_t)rows * cols);
+    const uint64_t raw = ggml_bytes(ftype, (uint64_t)rows * cols, file_version);
     HIP_TRY(hipMemcpyAsync(staging, host_blocks, raw, hipMemcpyHostToDevice, c->stream));
     uint4 *codes = reinterpret_cast<uint4 *>(dst);
-    uint16_t *scales = reinterpret_cast<uint16_t *>(dst + align_up(codes_bytes(ftype, nblk), 256));
+    uint8_t *scale_plane = dst + align_up(codes_bytes(ftype, nblk), 256);
+    uint16_t *scales = file_version == 1 ? nullptr : reinterpret_cast<uint16_t *>(scale_plane);
+    float *scales_f32 = file_version == 1 ? reinterpret_cast<float *>(scale_plane) : nullptr;
     const unsigned grid = (unsigned)((nblk + 255) / 256);
-    if (ftype == LV_Q4_0)
+    if (file_version == 1) {
+        if (ftype == LV_Q4_0) repack_v1_kernel<4><<<dim3(grid), dim3(256), 0, c->stream>>>(staging, codes, scales_f32, nblk);
+        else repack_v1_kernel<8><<<dim3(grid), dim3(256), 0, c->stream>>>(staging, codes, scales_f32, nblk);
+    } else if (ftype == LV_Q4_0) {
         repack_kernel<4><<<dim3(grid), dim3(256), 0, c->stream>>>(staging, codes, scales, nblk);
-    else
+    } else {
         repack_kernel<8><<<dim3(grid), dim3(256), 0, c->stream>>>(staging, codes, scales, nblk);
+    }
     HIP_TRY(hipGetLastError());
     HIP_TRY(hipStreamSynchronize(c->stream));  // staging is reused by the next tensor
     m->ctx = c;
     m->view.codes = codes;
     m->view.scales = scales;
+    m->view.scales_f32 = scales_f32;
     m->view.rows = rows;
     m->view.cols = cols;
     m->ftype = ftype;
@@ -397,8 +406,8 @@ static int place_matrix(lv_ctx *c, lv_matrix *m, uint8_t *dst, const void *host_
 static int check_quant_shape(const char *who, uint32_t ftype, uint32_t file_version, uint32_t rows, uint32_t cols)
 {
     if (ftype != LV_Q4_0 && ftype != LV_Q8_0) return fail(LV_ERR_ARG, "%s: type %u is not q4_0/q8_0", who, ftype);
-    if (file_version != 3)
-        return fail(LV_ERR_ARG, "%s: file version %u (only version 3, fp16 block scales, is supported)", who, file_version);
+    if (file_version != 3 && file_version != 1)
+        return fail(LV_ERR_ARG, "%s: file version %u (1: fp32 block scales, 3: fp16 block scales)", who, file_version);
     if (rows == 0 || cols == 0 || cols % 32) return fail(LV_ERR_ARG, "%s: shape %u x %u", who, rows, cols);
     if (cols / 32 > 768) return fail(LV_ERR_ARG, "%s: %u columns exceed the 24576 the GEMV kernels cover", who, cols);
     return LV_OK;
@@ -414,12 +423,12 @@ extern "C" int lv_matrix_upload(lv_ctx *c, const void *blocks, uint32_t ftype, u
     lv_matrix *m = new (std::nothrow) lv_matrix;
     if (!m) return fail(LV_ERR_OOM, "lv_matrix_upload: host allocation");
     uint8_t *staging = nullptr;
-    const uint64_t raw = ggml_bytes(ftype, (uint64_t)rows * cols);
-    hipError_t e = hipMalloc(&m->owned, matrix_device_bytes(ftype, rows, cols));
+    const uint64_t raw = ggml_bytes(ftype, (uint64_t)rows * cols, file_version);
+    hipError_t e = hipMalloc(&m->owned, matrix_device_bytes(ftype, rows, cols, file_version));
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&staging), raw);
     int rc = LV_OK;
     if (e != hipSuccess) rc = fail(e == hipErrorOutOfMemory ? LV_ERR_OOM : LV_ERR_HIP, "lv_matrix_upload: %s", hipGetErrorString(e));
-    if (rc == LV_OK) rc = place_matrix(c, m, static_cast<uint8_t *>(m->owned), blocks, ftype, rows, cols, staging);
+    if (rc == LV_OK) rc = place_matrix(c, m, static_cast<uint8_t *>(m->owned), blocks, ftype, rows, cols, staging, file_version);
     (void)hipFree(staging);
     if (rc != LV_OK) {
         (void)hipFree(m->owned);
@@ -846,7 +855,7 @@ static int build_mega(lv_model *m)
 {
     const lv_hparams &hp = m->hp;
     const uint32_t ft = m->output.ftype;
-    bool uniform = ft == LV_Q4_0 || ft == LV_Q8_0;
+    bool uniform = (ft == LV_Q4_0 || ft == LV_Q8_0) && m->output.view.scales != nullptr;   // the tile stream carries fp16 scales
     for (const LayerWeights &lw : m->layers)
         for (const lv_matrix *x : {&lw.wq, &lw.wk, &lw.wv, &lw.wo, &lw.w1, &lw.w2, &lw.w3}) uniform = uniform && x->ftype == ft;
     if (!uniform || (int)m->ctx->props.multiProcessorCount < kMegaWGs) return LV_OK;
@@ -927,7 +936,7 @@ extern "C" int lv_model_upload(lv_ctx *c, const void *base, uint64_t base_size, 
         const lv_tensor_desc &d = *w.desc;
         if (d.rows != w.rows || d.cols != w.cols)
             return fail(LV_ERR_ARG, "lv_model_upload: %s is %u x %u, expected %u x %u", d.name, d.rows, d.cols, w.rows, w.cols);
-        const uint64_t raw = ggml_bytes(d.ftype, (uint64_t)d.rows * d.cols);
+        const uint64_t raw = ggml_bytes(d.ftype, (uint64_t)d.rows * d.cols, hp->file_version);
         if (raw == 0 || d.size != raw || d.offset + raw > base_size)
             return fail(LV_ERR_ARG, "lv_model_upload: %s has type %u / %llu bytes at %llu (file holds %llu)", d.name, d.ftype,
                         (unsigned long long)d.size, (unsigned long long)d.offset, (unsigned long long)base_size);
@@ -935,7 +944,7 @@ extern "C" int lv_model_upload(lv_ctx *c, const void *base, uint64_t base_size, 
         if (w.quant || (is_quant && w.cols > 1)) {
             LV_TRY(check_quant_shape(d.name, d.ftype, hp->file_version, d.rows, d.cols));
             w.arena_off = arena_bytes;
-            arena_bytes += matrix_device_bytes(d.ftype, d.rows, d.cols);
+            arena_bytes += matrix_device_bytes(d.ftype, d.rows, d.cols, hp->file_version);
             if (raw > staging_bytes) staging_bytes = raw;
         } else {
             if (d.ftype != LV_F32) return fail(LV_ERR_ARG, "lv_model_upload: %s must be f32 (type %u)", d.name, d.ftype);
@@ -963,7 +972,7 @@ extern "C" int lv_model_upload(lv_ctx *c, const void *base, uint64_t base_size, 
     int rc = LV_OK;
     const uint8_t *hb = static_cast<const uint8_t *>(base);
     auto put_matrix = [&](const Want &w, lv_matrix *dst) {
-        return place_matrix(c, dst, m->arena + w.arena_off, hb + w.desc->offset, w.desc->ftype, w.desc->rows, w.desc->cols, staging);
+        return place_matrix(c, dst, m->arena + w.arena_off, hb + w.desc->offset, w.desc->ftype, w.desc->rows, w.desc->cols, staging, hp->file_version);
     };
     auto put_f32 = [&](const Want &w, const float **dst) -> int {
         HIP_TRY(hipMemcpyAsync(m->arena + w.arena_off, hb + w.desc->offset, w.desc->size, hipMemcpyHostToDevice, c->stream));

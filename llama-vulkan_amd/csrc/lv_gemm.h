@@ -153,7 +153,7 @@ __global__ __launch_bounds__(NWV * 64) void gemm_kernel(GemmArgs a)
     // shorter than a trip to memory)
     struct Staged {
         uint4 c0, c1;
-        uint16_t dbits;
+        uint32_t dbits;     // raw scale word
         bool wvalid;
         uint4 gh[XP], gl[XP];
     } pre[2];
@@ -166,7 +166,7 @@ __global__ __launch_bounds__(NWV * 64) void gemm_kernel(GemmArgs a)
             const size_t sb = (size_t)(p.wvalid ? wrow : 0) * nb + (p.wvalid ? blk : 0);
             p.c0 = a.w.codes[sb * CPB];
             if constexpr (QT == 8) p.c1 = a.w.codes[sb * CPB + 1];
-            p.dbits = a.w.scales[sb];
+            p.dbits = mat_scale_raw(a.w, sb);
         }
         const uint32_t k = step * kGemmK + xc;
         const bool kok = k < K;
@@ -193,7 +193,7 @@ __global__ __launch_bounds__(NWV * 64) void gemm_kernel(GemmArgs a)
         // registers -> LDS
         if (has_w) {
             gemm_codes_block<QT>(sW + r_w * kGemmLd + b_w * 32, P.wvalid, P.c0, P.c1);
-            sD[b_w][r_w] = P.wvalid ? half_bits_to_float(P.dbits) : 0.f;
+            sD[b_w][r_w] = P.wvalid ? mat_scale_value(a.w, P.dbits) : 0.f;
         }
 #pragma unroll
         for (int i = 0; i < XP; i++) {

@@ -20,7 +20,7 @@ constexpr int kWideMaxK = 64 * 32 * kWideWaves;   // widest row: every wave one 
 
 struct WideTile {
     uint4 c, c2;
-    uint16_t d;
+    uint32_t d;     // raw scale word (fp16 bits, or fp32 bits for a version-1 file)
 };
 
 template <int QT>
@@ -33,14 +33,14 @@ __device__ __forceinline__ void wide_load(WideTile &t, const MatView &m, uint64_
         t.c = m.codes[2 * b];
         t.c2 = m.codes[2 * b + 1];
     }
-    t.d = m.scales[b];
+    t.d = mat_scale_raw(m, b);
 }
 
 template <int QT>
-__device__ __forceinline__ float wide_dot(const WideTile &t, const float (&x)[32], float xsum)
+__device__ __forceinline__ float wide_dot(const WideTile &t, const MatView &m, const float (&x)[32], float xsum)
 {
-    if constexpr (QT == 4) return (q4_block_dot(t.c, x) - 8.f * xsum) * half_bits_to_float(t.d);
-    else return (q8_block_dot(t.c, t.c2, x) - 128.f * xsum) * half_bits_to_float(t.d);
+    if constexpr (QT == 4) return (q4_block_dot(t.c, x) - 8.f * xsum) * mat_scale_value(m, t.d);
+    else return (q8_block_dot(t.c, t.c2, x) - 128.f * xsum) * mat_scale_value(m, t.d);
 }
 
 // Workgroup barrier that orders LDS traffic only: the weight loads in flight stay in flight.
@@ -138,7 +138,7 @@ __device__ __forceinline__ void gemv_wide_body(const GemvArgs &a, uint32_t rows_
 #pragma unroll
             for (int j = 0; j < 4; j++) {
 #pragma unroll
-                for (int mi = 0; mi < NMAT; mi++) p[mi][j] = wide_dot<QT>(q[mi][g + j], xr, xsum);
+                for (int mi = 0; mi < NMAT; mi++) p[mi][j] = wide_dot<QT>(q[mi][g + j], mi == 0 ? a.w : a.w1, xr, xsum);
                 fetch(g + j, i0 + g + j + DEPTH);
             }
 #pragma unroll

@@ -12,13 +12,53 @@ namespace lv {
 
 struct MatView {
     const uint4 *codes;     // 1 (q4_0) or 2 (q8_0) uint4 per block
-    const uint16_t *scales; // fp16 bits
+    const uint16_t *scales; // fp16 bits (file version 3)
     uint32_t rows, cols;
+    const float *scales_f32 = nullptr;   // fp32 block scales of a version-1 file (then `scales` is null)
 };
+
+// Scale of block b, raw (as loaded) and as a float.  Which plane a matrix has is uniform over a launch; keeping the
+// raw word lets a load queue run ahead and convert only when the block is used.
+__device__ __forceinline__ uint32_t mat_scale_raw(const MatView &m, uint64_t b)
+{
+    return m.scales_f32 ? __float_as_uint(m.scales_f32[b]) : (uint32_t)m.scales[b];
+}
+__device__ __forceinline__ float mat_scale_value(const MatView &m, uint32_t raw)
+{
+    return m.scales_f32 ? __uint_as_float(raw) : half_bits_to_float((uint16_t)raw);
+}
+__device__ __forceinline__ float mat_scale(const MatView &m, uint64_t b) { return mat_scale_value(m, mat_scale_raw(m, b)); }
 
 // ---------------------------------------------------------------------------------------------------------
 // GGML blocks -> device layout (runs once per tensor at upload; replaces llava_buffer.cpp:226-323)
 // ---------------------------------------------------------------------------------------------------------
+// Version-1 files (llava_buffer.cpp:66-71, 193-224): an fp32 scale in front of the codes (20 / 36 B blocks), and q4_0
+// nibbles interleaved (byte j carries elements 2j and 2j+1, llava_buffer.cpp:351-359) instead of split (j and j+16).
+// The codes are brought into the version-3 order, the scales kept as fp32: nothing is rounded.
+template <int QT>
+__global__ void repack_v1_kernel(const uint8_t *__restrict__ src, uint4 *__restrict__ codes, float *__restrict__ scales, uint64_t n_blocks)
+{
+    constexpr int kBlockBytes = QT == 4 ? 20 : 36;
+    const uint64_t b = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= n_blocks) return;
+    const uint32_t *p = reinterpret_cast<const uint32_t *>(src + b * kBlockBytes);  // blocks are 4-byte aligned
+    scales[b] = __uint_as_float(p[0]);
+    if constexpr (QT == 4) {
+        uint32_t out[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int e = 0; e < 32; e++) {
+            const uint32_t byte = (p[1 + (e >> 3)] >> (8 * ((e >> 1) & 3))) & 0xffu;      // v1: element e in byte e/2
+            const uint32_t nib = (e & 1) ? (byte >> 4) : (byte & 0xfu);
+            const int j = e & 15, hi = e >> 4;                                           // v3: byte e%16, nibble e/16
+            out[j >> 2] |= nib << (8 * (j & 3) + 4 * hi);
+        }
+        codes[b] = make_uint4(out[0], out[1], out[2], out[3]);
+    } else {
+        codes[2 * b] = make_uint4(p[1], p[2], p[3], p[4]);
+        codes[2 * b + 1] = make_uint4(p[5], p[6], p[7], p[8]);
+    }
+}
+
 template <int QT>  // 4: q4_0 (18 B blocks), 8: q8_0 (34 B blocks)
 __global__ void repack_kernel(const uint8_t *__restrict__ src, uint4 *__restrict__ codes, uint16_t *__restrict__ scales,
                               uint64_t n_blocks)
@@ -47,7 +87,7 @@ __global__ void dequant_kernel(MatView m, uint64_t first_block, uint64_t n_block
     const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n_blocks) return;
     const uint64_t b = first_block + i;
-    const float d = half_bits_to_float(m.scales[b]);
+    const float d = mat_scale(m, b);
     float4 *out = reinterpret_cast<float4 *>(dst + i * 32);
     if constexpr (QT == 4) {
         const uint4 q = m.codes[b];
@@ -103,7 +143,7 @@ struct GemvArgs {
 template <int QT>
 __device__ __forceinline__ float block_partial(const MatView &m, uint64_t blk, const float (&x)[32], float xoff)
 {
-    const float d = half_bits_to_float(m.scales[blk]);
+    const float d = mat_scale(m, blk);
     float s;
     if constexpr (QT == 4) {
         const uint4 q = m.codes[blk];
@@ -305,7 +345,7 @@ __global__ void embed_quant_kernel(float *__restrict__ x, MatView table, const u
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;  // block within the row
     if (i >= nb) return;
     const uint64_t b = (uint64_t)tokens[z] * nb + i;
-    const float d = half_bits_to_float(table.scales[b]);
+    const float d = mat_scale(table, b);
     float *dst = x + (size_t)z * table.cols + (size_t)i * 32;
     if constexpr (QT == 4) {
         const uint4 q = table.codes[b];

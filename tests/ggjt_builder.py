@@ -79,3 +79,47 @@ TOKENIZER_TEXTS = [
     "", "h", "hello", "hello world", "hellohello", " world", "world", "ab", "abab", "ababab", "aaaaaaa", "aaaa", "xyz", "xy",
     "é", "日本", "日本語", "héllo wörld", "\x00\x01\xff", "a" * 33, "llo", "lllo", "hell", "hel", "\xe6\x97",
 ]
+
+
+def blocks_to_v1(blocks, ftype):
+    """Re-encodes version-3 quantised blocks (fp16 scale; q4_0 byte j = elements j and j+16) as version-1 blocks
+    (fp32 scale of the same value; q4_0 byte j = elements 2j and 2j+1).  The element values are unchanged, so a
+    version-1 file made this way must give the same results as its version-3 source."""
+    stride = 18 if ftype == Q4_0 else 34
+    b = np.ascontiguousarray(blocks, dtype=np.uint8).reshape(-1, stride)
+    scale = b[:, :2].copy().view(np.float16).astype(np.float32)             # exact widening
+    codes = b[:, 2:]
+    if ftype == Q4_0:
+        elem = np.concatenate([codes & 15, codes >> 4], axis=1)             # elements 0..31 in order
+        codes = (elem[:, 0::2] | (elem[:, 1::2] << 4)).astype(np.uint8)
+    out = np.empty((b.shape[0], 4 + codes.shape[1]), dtype=np.uint8)
+    out[:, :4] = scale.view(np.uint8).reshape(-1, 4)
+    out[:, 4:] = codes
+    return out.reshape(-1)
+
+
+def convert_to_v1(src, dst):
+    """Rewrites a version-3 GGJT file as version 1, tensor by tensor, keeping names, shapes and vocabulary."""
+    data = np.fromfile(src, dtype=np.uint8)
+    hdr = np.frombuffer(data[:36].tobytes(), dtype=np.uint32).copy()
+    assert hdr[0] == MAGIC and hdr[1] == 3
+    cur = 36
+    for _ in range(int(hdr[2])):
+        ln = struct.unpack_from("<i", data, cur)[0]
+        cur += 8 + ln
+    hdr[1] = 1
+    out = bytearray(hdr.tobytes()) + bytearray(data[36:cur].tobytes())
+    while cur != data.shape[0]:
+        n_dims, name_len, ft = struct.unpack_from("<3I", data, cur)
+        head_len = 12 + 4 * n_dims + name_len
+        ne = struct.unpack_from(f"<{n_dims}I", data, cur + 12)
+        n = int(np.prod(ne))
+        out += data[cur:cur + head_len].tobytes()
+        out += b"\0" * ((-len(out)) % 32)
+        cur = (cur + head_len + 31) & ~31
+        size = payload_bytes(ft, n, 3)
+        payload = data[cur:cur + size]
+        out += (blocks_to_v1(payload, ft) if ft in (Q4_0, Q8_0) else payload).tobytes()
+        cur += size
+    with open(dst, "wb") as f:
+        f.write(out)

@@ -158,7 +158,8 @@ def test_errors_are_reported_not_fatal(lva, ctx):
     blocks = np.zeros(18 * 4, dtype=np.uint8)
     assert lib.lv_matrix_upload(ctx.h, blocks.ctypes.data_as(lva.C.c_void_p), lva.LV_Q4_0, 3, 4, 33, lva.C.byref(m)) == -1
     assert b"shape" in lib.lv_last_error()
-    assert lib.lv_matrix_upload(ctx.h, blocks.ctypes.data_as(lva.C.c_void_p), lva.LV_Q4_0, 1, 4, 32, lva.C.byref(m)) == -1
+    assert lib.lv_matrix_upload(ctx.h, blocks.ctypes.data_as(lva.C.c_void_p), lva.LV_Q4_0, 2, 4, 32, lva.C.byref(m)) == -1    # versions 1 and 3 only
+    assert b"version" in lib.lv_last_error()
     assert lib.lv_matrix_upload(ctx.h, blocks.ctypes.data_as(lva.C.c_void_p), 3, 3, 4, 32, lva.C.byref(m)) == -1
     assert lib.lv_kernel_normalize(ctx.h, None, None, None, 16, 1) == -1
     assert lib.lv_kernel_kv_append(ctx.h, lva.C.c_void_p(8), lva.C.c_void_p(8), 128, 16, 1, 128) == -5

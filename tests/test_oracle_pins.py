@@ -405,3 +405,21 @@ def test_prompt_as_one_batch_equals_token_by_token(lva, orc, tiny_models):
     again = b.eval(toks[4:], all_rows=True)
     assert np.array_equal(again, batched[4:])
     a.close(); b.close(); om.close()
+
+
+@pytest.mark.parametrize("name", ["tiny_q4", "tiny_q8"])
+def test_version_1_file_gives_the_logits_of_its_version_3_twin(lva, orc, tiny_models, tmp_path, name):
+    """the same element values stored as version-1 blocks (fp32 scale, interleaved nibbles; ggml_file.cpp:95-122):
+    the file is a different byte stream, the arithmetic on the decoded values is the same, bit for bit"""
+    import ggjt_builder as gb
+    p1 = str(tmp_path / "v1.ggml")
+    gb.convert_to_v1(tiny_models[name], p1)
+    toks = lva.synth_tokens(6, 3, 512, seed=4)
+    outs = []
+    for path, ver in ((tiny_models[name], 3), (p1, 1)):
+        om = orc.Model(path)
+        assert om.hp["file_version"] == ver
+        s = orc.Session(om, 128)
+        outs.append(s.eval(toks, all_rows=True).copy())
+        s.close(); om.close()
+    assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
