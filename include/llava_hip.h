@@ -131,7 +131,9 @@ enum {
     LV_TRACE_POST_ATTN_NORM = 2, /* post_attn_norm_logit    [dim] */
     LV_TRACE_FF = 3,             /* ff_result               [ff]  */
     LV_TRACE_OUT = 4,            /* output_logit            [dim] */
-    LV_TRACE_COUNT = 5
+    LV_TRACE_ATTN = 5,           /* attn_result             [backlog][heads]: softmax weights, 0 behind the row's position
+                                    (mhsa.comp + softmax.comp; the reference's [BACKLOG][HEAD_COUNT] layout) */
+    LV_TRACE_COUNT = 6
 };
 int lv_trace_enable(lv_session *s, int enable);
 int lv_trace_read(lv_session *s, uint32_t layer, int which, float *dst, uint32_t count);

@@ -21,7 +21,7 @@ ROOT_DIR = os.path.dirname(PKG_DIR)
 
 LV_F32, LV_F16, LV_Q4_0, LV_Q8_0 = 0, 1, 2, 8
 PATH_AUTO, PATH_KERNELS, PATH_GRAPH, PATH_PERSISTENT = range(4)
-TRACE_NORM_IN, TRACE_POST_ATTN, TRACE_POST_ATTN_NORM, TRACE_FF, TRACE_OUT = range(5)
+TRACE_NORM_IN, TRACE_POST_ATTN, TRACE_POST_ATTN_NORM, TRACE_FF, TRACE_OUT, TRACE_ATTN = range(6)
 
 
 class LvError(RuntimeError):
@@ -403,6 +403,10 @@ class Session:
 
     def trace(self, layer, which):
         n = self.model.header["ff"] if which == TRACE_FF else self.model.header["dim"]
+        if which == TRACE_ATTN:
+            rows = C.c_uint32()
+            check(self.lib.lv_session_backlog(self.h, C.byref(rows)))
+            n = rows.value * self.model.header["heads"]
         out = np.empty(n, dtype=np.float32)
         check(self.lib.lv_trace_read(self.h, layer, which, _ptr(out), n))
         return out

@@ -165,7 +165,8 @@ struct lv_session {
     bool in_flight = false;
     bool have_logits = false;
     bool trace = false;
-    float *trace_buf = nullptr;  // [layers][LV_TRACE_COUNT][max(dim, ff)]
+    float *trace_buf = nullptr;  // [layers][LV_TRACE_ATTN][max(dim, ff)]: the five vector buffers
+    float *trace_attn = nullptr; // [layers][backlog][heads]: LV_TRACE_ATTN; follows the backlog
     hipEvent_t ev_start = nullptr, ev_stop = nullptr;
 };
 
@@ -1059,7 +1060,7 @@ extern "C" int lv_session_destroy(lv_session *s)
     }
     drop_graph(s);
     void *dev[] = {s->kv, s->trig, s->trig_abs, s->x, s->xn, s->q, s->k, s->v, s->vo, s->ff, s->logits, s->attn_part, s->attn_counters,
-                   s->cfg, s->argmax_dev, s->trace_buf, s->pf_x, s->pf_xn, s->pf_q, s->pf_k, s->pf_v, s->pf_vo, s->pf_g1, s->pf_g2,
+                   s->cfg, s->argmax_dev, s->trace_buf, s->trace_attn, s->pf_x, s->pf_xn, s->pf_q, s->pf_k, s->pf_v, s->pf_vo, s->pf_g1, s->pf_g2,
                    s->pf_xh, s->pf_xl};
     for (void *p : dev) (void)hipFree(p);
     (void)hipFree(s->xchg[0]);
@@ -1125,6 +1126,20 @@ extern "C" int lv_session_create(lv_model *m, lv_session **out)
     return LV_OK;
 }
 
+// record mode's attention weights: one [backlog][heads] buffer per layer, zero until a traced step fills it
+static int make_trace_attn(lv_session *s, uint32_t backlog)
+{
+    const lv_hparams &hp = s->model->hp;
+    const size_t bytes = (size_t)hp.layers * backlog * hp.heads * 4;
+    if (bytes == 0) return LV_OK;
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&s->trace_attn), bytes);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(e == hipErrorOutOfMemory ? LV_ERR_OOM : LV_ERR_HIP, "record mode: attention weights of %u rows: %s", backlog, hipGetErrorString(e));
+    }
+    return zero_async(s->trace_attn, bytes, s->stream);
+}
+
 extern "C" int lv_session_reserve(lv_session *s, uint32_t backlog)
 {
     if (!s) return fail(LV_ERR_ARG, "lv_session_reserve: session is null");
@@ -1164,6 +1179,8 @@ extern "C" int lv_session_reserve(lv_session *s, uint32_t backlog)
     s->attn_part = nullptr;
     (void)hipFree(s->attn_counters);
     s->attn_counters = nullptr;
+    (void)hipFree(s->trace_attn);
+    s->trace_attn = nullptr;
     s->backlog = 0;
     LV_TRY(upload_trig(&s->trig, backlog, hp.rot, s->stream));
     LV_TRY(upload_trig(&s->trig_abs, backlog, hp.rot, s->stream, true));
@@ -1171,6 +1188,7 @@ extern "C" int lv_session_reserve(lv_session *s, uint32_t backlog)
     HIP_TRY(hipMalloc(reinterpret_cast<void **>(&s->attn_part), attn_part_floats(1, hp.heads, splits, hp.rot) * sizeof(float)));
     HIP_TRY(hipMalloc(reinterpret_cast<void **>(&s->attn_counters), (size_t)hp.heads * 4));
     LV_TRY(zero_async(s->attn_counters, (size_t)hp.heads * 4, s->stream));
+    if (s->trace_buf) LV_TRY(make_trace_attn(s, backlog));
     HIP_TRY(hipStreamSynchronize(s->stream));
     s->backlog = backlog;
     return LV_OK;
@@ -1251,7 +1269,7 @@ static int trace_copy(lv_session *s, uint32_t layer, int which, const float *src
     if (!s->trace) return LV_OK;
     const lv_hparams &hp = s->model->hp;
     const size_t slot = hp.dim > hp.ff ? hp.dim : hp.ff;
-    float *dst = s->trace_buf + ((size_t)layer * LV_TRACE_COUNT + which) * slot;
+    float *dst = s->trace_buf + ((size_t)layer * LV_TRACE_ATTN + which) * slot;
     HIP_TRY(hipMemcpyAsync(dst, src, count * 4, hipMemcpyDeviceToDevice, s->stream));
     return LV_OK;
 }
@@ -1298,6 +1316,11 @@ static int record_token(lv_session *s, uint32_t idx, bool with_head)
         }
         LV_TRY(launch_attention(st, s->vo, kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->q, s->trig, s->attn_part, s->attn_counters,
                                 pos_ptr, idx, s->backlog, hp.heads, hp.rot, 1));
+        if (s->trace) {
+            attn_weights_kernel<<<dim3(hp.heads), dim3(256), 0, st>>>(s->trace_attn + (size_t)li * s->backlog * hp.heads, kv_ptr(s, li, 0), s->q,
+                                                                       s->trig, pos_ptr, idx, hp.heads, hp.rot, s->backlog);
+            HIP_TRY(hipGetLastError());
+        }
         LV_TRY(launch_gemv(st, s->x, lw.wo, nullptr, s->vo, 1, kGemvAdd));
         LV_TRY(trace_copy(s, li, LV_TRACE_POST_ATTN, s->x, D));
         if (fused) {
@@ -1563,7 +1586,9 @@ extern "C" int lv_trace_enable(lv_session *s, int enable)
     if (enable && !s->trace_buf) {
         const size_t slot = hp.dim > hp.ff ? hp.dim : hp.ff;
         HIP_TRY(hipSetDevice(s->model->ctx->device));
-        HIP_TRY(hipMalloc(reinterpret_cast<void **>(&s->trace_buf), (size_t)hp.layers * LV_TRACE_COUNT * slot * 4));
+        HIP_TRY(hipMalloc(reinterpret_cast<void **>(&s->trace_buf), (size_t)hp.layers * LV_TRACE_ATTN * slot * 4));
+        LV_TRY(make_trace_attn(s, s->backlog));
+        HIP_TRY(hipStreamSynchronize(s->stream));
     }
     s->trace = enable != 0;
     return LV_OK;
@@ -1575,10 +1600,11 @@ extern "C" int lv_trace_read(lv_session *s, uint32_t layer, int which, float *ds
     if (!s->trace || !s->trace_buf) return fail(LV_ERR_STATE, "lv_trace_read: record mode is off");
     const lv_hparams &hp = s->model->hp;
     if (layer >= hp.layers || which < 0 || which >= LV_TRACE_COUNT) return fail(LV_ERR_RANGE, "lv_trace_read: layer %u / buffer %d", layer, which);
-    const uint32_t have = which == LV_TRACE_FF ? hp.ff : hp.dim;
+    const uint32_t have = which == LV_TRACE_FF ? hp.ff : which == LV_TRACE_ATTN ? s->backlog * hp.heads : hp.dim;
     if (count != have) return fail(LV_ERR_ARG, "lv_trace_read: buffer %d holds %u floats, %u asked", which, have, count);
     const size_t slot = hp.dim > hp.ff ? hp.dim : hp.ff;
-    HIP_TRY(hipMemcpyAsync(dst, s->trace_buf + ((size_t)layer * LV_TRACE_COUNT + which) * slot, (size_t)count * 4, hipMemcpyDeviceToHost, s->stream));
+    const float *src = which == LV_TRACE_ATTN ? s->trace_attn + (size_t)layer * have : s->trace_buf + ((size_t)layer * LV_TRACE_ATTN + which) * slot;
+    HIP_TRY(hipMemcpyAsync(dst, src, (size_t)count * 4, hipMemcpyDeviceToHost, s->stream));
     HIP_TRY(hipStreamSynchronize(s->stream));
     s->in_flight = false;
     return LV_OK;

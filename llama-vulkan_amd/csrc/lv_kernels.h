@@ -528,6 +528,47 @@ __global__ __launch_bounds__(256) void attention_kernel(AttnArgs a)
 }
 
 // ---------------------------------------------------------------------------------------------------------
+// Record mode only: the attention weights of one query as a buffer, which the fused kernel above never holds
+// (mhsa.comp + softmax.comp leave them in attn_result, laid out [backlog][heads]; slots behind the query's position
+// hold 0, softmax.comp:33-35).  One workgroup per head; scores with the per-pair rotation of the shader, no max
+// subtraction, the sum taken over the workgroup in a fixed order.  Not on the decode path.
+// ---------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void attn_weights_kernel(float *__restrict__ out, const uint16_t *__restrict__ kcache,
+                                                           const float *__restrict__ q, const float2 *__restrict__ trig,
+                                                           const uint32_t *pos_ptr, uint32_t pos_add, uint32_t heads, uint32_t rot,
+                                                           uint32_t backlog)
+{
+    __shared__ float red[4];
+    const uint32_t h = blockIdx.x, half = rot / 2, dim = heads * rot;
+    const uint32_t cur = *pos_ptr + pos_add;
+    const float factor = 1.0f / sqrtf((float)rot);
+    const float *qr = q + (size_t)h * rot;
+    float sum = 0.f;
+    for (uint32_t p = threadIdx.x; p < backlog; p += 256) {
+        float e = 0.f;
+        if (p <= cur) {
+            const uint16_t *kr = kcache + (size_t)p * dim + (size_t)h * rot;
+            const float2 *t = trig + (size_t)(cur - p) * half;
+            float score = 0.f;
+            for (uint32_t i = 0; i < half; i++) {
+                const float kx = half_bits_to_float(kr[2 * i]), ky = half_bits_to_float(kr[2 * i + 1]);
+                const float2 cs = t[i];
+                const float rx = cs.x * kx + cs.y * ky, ry = -cs.y * kx + cs.x * ky;
+                score += qr[2 * i] * rx + qr[2 * i + 1] * ry;
+            }
+            e = expf(score * factor);
+        }
+        out[(size_t)p * heads + h] = e;       // un-normalised for now; this thread re-reads its own slots below
+        sum += e;
+    }
+    for (int off = 32; off; off >>= 1) sum += __shfl_xor(sum, off);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = sum;
+    __syncthreads();
+    const float total = (red[0] + red[1]) + (red[2] + red[3]);
+    for (uint32_t p = threadIdx.x; p < backlog; p += 256) out[(size_t)p * heads + h] /= total;
+}
+
+// ---------------------------------------------------------------------------------------------------------
 // Greedy pick (llava_session.cpp:144-152): index of the first strict maximum.  One workgroup.
 // ---------------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ logits, uint32_t n, uint32_t *out)

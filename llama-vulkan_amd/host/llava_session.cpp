@@ -24,14 +24,16 @@ constexpr u32 kMinBacklog = 128;
 constexpr u32 kMaxBacklog = 2048;
 
 // record-mode buffers in the order they are dumped, with the names the reference gives them
-// (llava_layer_session_data.cpp:80-85).  attn_result is not materialised by the fused attention kernel.
-struct TraceSlot { int which; const char *name; bool is_ff; };
+// (llava_layer_session_data.cpp:80-85)
+enum class TraceShape { dim, ff, attn };
+struct TraceSlot { int which; const char *name; TraceShape shape; };
 constexpr TraceSlot kTraceSlots[] = {
-    {LV_TRACE_FF, "ff_result", true},
-    {LV_TRACE_NORM_IN, "normalized_input_logit", false},
-    {LV_TRACE_POST_ATTN, "post_attn_logit", false},
-    {LV_TRACE_POST_ATTN_NORM, "post_attn_norm_logit", false},
-    {LV_TRACE_OUT, "output_logit", false},
+    {LV_TRACE_ATTN, "attn_result", TraceShape::attn},
+    {LV_TRACE_FF, "ff_result", TraceShape::ff},
+    {LV_TRACE_NORM_IN, "normalized_input_logit", TraceShape::dim},
+    {LV_TRACE_POST_ATTN, "post_attn_logit", TraceShape::dim},
+    {LV_TRACE_POST_ATTN_NORM, "post_attn_norm_logit", TraceShape::dim},
+    {LV_TRACE_OUT, "output_logit", TraceShape::dim},
 };
 
 // RAII for a file descriptor
@@ -70,9 +72,12 @@ void llava_layer_session_data::restore_kv_cache(const u8 *src, u32 token_count)
 // multiple of 32 bytes, then the raw fp32 values.
 void llava_layer_session_data::dump_tracing_layers(int out_fd, const std::string &name)
 {
-    const u32 dim = session->model->get_header().dim, ff = session->model->get_ff_size();
+    const u32 dim = session->model->get_header().dim, ff = session->model->get_ff_size(), heads = session->model->get_header().n_heads;
     for (const TraceSlot &slot : kTraceSlots) {
-        const u32 count = slot.is_ff ? ff : dim;
+        // shape as the reference's buffers have it: (values per row, rows); attn_result is (backlog, heads x rows)
+        const u32 shape0 = slot.shape == TraceShape::ff ? ff : slot.shape == TraceShape::attn ? session->backlog_size : dim;
+        const u32 shape1 = slot.shape == TraceShape::attn ? heads : 1u;      // the last row of the step
+        const u32 count = shape0 * shape1;
         std::vector<float> values(count);
         if (lv_trace_read(session->device_session, layer, slot.which, values.data(), count) != LV_OK) {
             std::cerr << "dump_tracing_layers: " << lv_last_error() << std::endl;
@@ -81,7 +86,7 @@ void llava_layer_session_data::dump_tracing_layers(int out_fd, const std::string
         const std::string full = name + "." + slot.name;
         const u32 header_size = static_cast<u32>((12 + full.size() + 1 + 31) & ~static_cast<std::size_t>(31));
         std::vector<u8> head(header_size, 0);
-        const u32 fields[3] = {count, 1u /* the last row of the step */, static_cast<u32>(ggml_value_type::f32)};
+        const u32 fields[3] = {shape0, shape1, static_cast<u32>(ggml_value_type::f32)};
         std::memcpy(head.data(), fields, sizeof fields);
         std::memcpy(head.data() + 12, full.data(), full.size());
         if (write_noshort(out_fd, head.data(), head.size()) != head.size() ||

@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(HERE, "liboracle.so")
 REF_PATH = os.path.join(HERE, "_ref", "libref_ggml.so")
 
 F32, F16, Q4_0, Q8_0 = 0, 1, 2, 8
-TR_NORM_IN, TR_POST_ATTN, TR_POST_ATTN_NORM, TR_FF, TR_OUT = range(5)
+TR_NORM_IN, TR_POST_ATTN, TR_POST_ATTN_NORM, TR_FF, TR_OUT, TR_ATTN = range(6)
 
 
 class HParams(C.Structure):

@@ -623,7 +623,7 @@ typedef struct {
     const orc_tensor *wq, *wk, *wv, *wo, *w1, *w2, *w3, *attn_norm, *ffn_norm;
 } orc_layer;
 
-enum { TR_NORM_IN = 0, TR_POST_ATTN, TR_POST_ATTN_NORM, TR_FF, TR_OUT, TR_COUNT };
+enum { TR_NORM_IN = 0, TR_POST_ATTN, TR_POST_ATTN_NORM, TR_FF, TR_OUT, TR_ATTN, TR_COUNT };
 
 struct orc_session {
     const orc_model *m;
@@ -670,7 +670,7 @@ orc_session *orc_session_new(const orc_model *m, uint32_t backlog)
         s->kc[i] = (uint16_t *)calloc((size_t)backlog * D, 2);
         s->vc[i] = (uint16_t *)calloc((size_t)backlog * D, 2);
         for (int t = 0; t < TR_COUNT; t++)
-            s->trace[i * TR_COUNT + t] = (float *)calloc(t == TR_FF ? F : D, sizeof(float));
+            s->trace[i * TR_COUNT + t] = (float *)calloc(t == TR_FF ? F : t == TR_ATTN ? (size_t)backlog * m->hp.heads : D, sizeof(float));
     }
     s->tok = find_tensor(m, "tok_embeddings");
     s->norm = find_tensor(m, "norm");
@@ -743,7 +743,7 @@ const float *orc_session_trace(const orc_session *s, uint32_t layer, int which, 
     if (layer >= s->m->hp.layers || which < 0 || which >= TR_COUNT)
         return NULL;
     if (count)
-        *count = (which == TR_FF) ? s->m->hp.ff : s->m->hp.dim;
+        *count = (which == TR_FF) ? s->m->hp.ff : (which == TR_ATTN) ? s->backlog * s->m->hp.heads : s->m->hp.dim;
     return s->trace[layer * TR_COUNT + which];
 }
 
@@ -791,6 +791,7 @@ int orc_session_eval(orc_session *s, const uint32_t *tokens, uint32_t n, float *
         orc_kv_append(s->vc[li], v, pos, D, n);
         orc_mhsa(att, s->kc[li], q, pos, L, H, R, n);
         orc_softmax(att, pos, L, H, R, n);
+        memcpy(tr[TR_ATTN], att + last * L * H, sizeof(float) * L * H); /* attn_result of the last row, [backlog][heads] */
         orc_kqv(vo, s->vc[li], att, L, H, R, n);
         rc |= orc_gemv(x, tdata(m, l->wo), l->wo->ftype, ver, D, D, vo, n, 1, 0);
         memcpy(tr[TR_POST_ATTN], x + last * D, sizeof(float) * D);

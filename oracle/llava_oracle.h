@@ -93,7 +93,8 @@ int orc_session_kv_load(orc_session *s, uint32_t layer, int which, const uint16_
 int orc_session_set_pos(orc_session *s, uint32_t pos);
 /* threads the checker's row loops run on */
 int orc_num_threads(void);
-/* per-layer intermediates of the LAST row of the last eval (trace); returns dim or ff floats */
+/* per-layer intermediates of the LAST row of the last eval (trace); dim, ff or (which 5, the softmax weights
+ * attn_result laid out [backlog][heads], llava_layer.cpp:60-61) backlog*heads floats */
 const float *orc_session_trace(const orc_session *s, uint32_t layer, int which, uint32_t *count);
 
 #ifdef __cplusplus

@@ -124,6 +124,22 @@ def test_trace_buffers_match_oracle(lva, orc, ctx, tiny_models):
             got, want = s.trace(layer, which), osess.trace(layer, which)
             assert got.shape == want.shape
             assert np.max(np.abs(got - want)) <= 1e-4 * max(1.0, np.max(np.abs(want))), (layer, which)
+        # attn_result: the softmax weights of the last row, [backlog][heads]; rows behind its position hold exact zeros
+        got, want = s.trace(layer, lva.TRACE_ATTN).reshape(128, -1), osess.trace(layer, orc.TR_ATTN).reshape(128, -1)
+        assert got.shape == want.shape == (128, om.hp["heads"])
+        assert np.all(got[5:] == 0.0) and np.all(want[5:] == 0.0)
+        assert np.max(np.abs(got - want)) <= 1e-5 and np.allclose(got.sum(axis=0), 1.0, atol=1e-5)
+    # one more token: the weights now cover six rows; a larger backlog keeps the layout [backlog][heads]
+    tok = orc.greedy(osess.eval([7]))
+    s.begin([7], 5); s.wait()
+    s.reserve(256)
+    assert np.all(s.trace(0, lva.TRACE_ATTN) == 0.0)          # a fresh buffer of the new size
+    s.begin([tok], 6); s.wait()
+    o2 = orc.Session(om, 256)
+    o2.eval(list(prompt) + [7, tok])
+    got, want = s.trace(1, lva.TRACE_ATTN).reshape(256, -1), o2.trace(1, orc.TR_ATTN).reshape(256, -1)
+    assert np.all(got[7:] == 0.0) and np.max(np.abs(got - want)) <= 1e-5
+    o2.close()
     s.close(); model.close(); osess.close(); om.close()
 
 

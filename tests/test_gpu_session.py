@@ -197,7 +197,7 @@ def test_save_frame_needs_tracing_and_writes_named_buffers(hl, orc, loaded, tmp_
     om = orc.Model(path)
     o = orc.Session(om, 128)
     o.eval(np.array(s.tokens(), dtype=np.uint32))
-    which = {"normalized_input_logit": 0, "post_attn_logit": 1, "post_attn_norm_logit": 2, "ff_result": 3, "output_logit": 4}
+    which = {"normalized_input_logit": 0, "post_attn_logit": 1, "post_attn_norm_logit": 2, "ff_result": 3, "output_logit": 4, "attn_result": 5}
     cur, seen = 0, []
     while cur < len(raw):
         # llava_buffer.cpp:497-522: two shape words, the type, the name, zeros up to a multiple of 32, the values
@@ -206,12 +206,13 @@ def test_save_frame_needs_tracing_and_writes_named_buffers(hl, orc, loaded, tmp_
         head = (12 + len(name) + 1 + 31) // 32 * 32
         vals = np.frombuffer(raw, dtype=np.float32, count=count * rows, offset=cur + head)
         cur += head + 4 * count * rows
-        assert ftype == 0 and rows == 1
         _, layer, slot = name.split(".")
+        # attn_result is (backlog, heads) as in llava_layer_session_data.cpp:80; the vectors are (length, 1 row)
+        assert ftype == 0 and (count, rows) == ((128, om.hp["heads"]) if slot == "attn_result" else (count, 1))
         want = o.trace(int(layer), which[slot])
         assert vals.shape == want.shape and np.max(np.abs(vals - want)) <= 1e-4 * max(1.0, np.max(np.abs(want))), name
         seen.append(name)
-    assert cur == len(raw) and len(seen) == 2 * 5 and seen[0] == "layer.0.ff_result"
+    assert cur == len(raw) and len(seen) == 2 * 6 and seen[:2] == ["layer.0.attn_result", "layer.0.ff_result"]
     o.close(); om.close()
     assert s.set_options(0) == hl.RC_OK and not s.is_tracing()
     s.close()
