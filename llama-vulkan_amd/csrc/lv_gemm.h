@@ -88,9 +88,9 @@ __host__ __device__ constexpr int gemm_k_position(int e)
 
 // 32 codes of one block -> 32 halfs at w, in gemm_k_position order, as the integers they are (q4_0: q - 8, q8_0: q):
 // 1024 + u has the fp16 bit pattern 0x6400 | u, and subtracting 1024 + offset is exact.  A block outside the matrix
-// becomes zeros.
+// is given the scale 0 by the caller, which removes it from the sum whatever codes were unpacked for it.
 template <int QT>
-__device__ __forceinline__ void gemm_codes_block(uint16_t *w, bool valid, const uint4 &c0, const uint4 &c1)
+__device__ __forceinline__ void gemm_codes_block(uint16_t *w, const uint4 &c0, const uint4 &c1)
 {
     uint32_t ph[16];
     auto emit = [&](int slot, uint32_t packed_codes, _Float16 bias) {
@@ -99,7 +99,7 @@ __device__ __forceinline__ void gemm_codes_block(uint16_t *w, bool valid, const 
         c.u = packed_codes;
         const lv_h2 bb = {bias, bias};
         v.h = c.h - bb;                              // exact: small integers
-        ph[slot] = valid ? v.u : 0u;
+        ph[slot] = v.u;
     };
     if constexpr (QT == 4) {
         const uint32_t q[4] = {c0.x, c0.y, c0.z, c0.w};
@@ -112,8 +112,9 @@ __device__ __forceinline__ void gemm_codes_block(uint16_t *w, bool valid, const 
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             const uint32_t u = q[i] ^ 0x80808080u;   // int8 -> biased unsigned
-            emit(2 * i, ((u & 0xffu) | ((u & 0xff00u) << 8)) | 0x64006400u, (_Float16)1152.f);
-            emit(2 * i + 1, (((u >> 16) & 0xffu) | ((u >> 8) & 0xff0000u)) | 0x64006400u, (_Float16)1152.f);
+            // one byte permute per pair: bytes (u.b0, 0x64, u.b1, 0x64) and (u.b2, 0x64, u.b3, 0x64)
+            emit(2 * i, __builtin_amdgcn_perm(u, 0x64646464u, 0x00050004u), (_Float16)1152.f);
+            emit(2 * i + 1, __builtin_amdgcn_perm(u, 0x64646464u, 0x00070006u), (_Float16)1152.f);
         }
     }
 #pragma unroll
@@ -192,7 +193,7 @@ __global__ __launch_bounds__(NWV * 64) void gemm_kernel(GemmArgs a)
     auto one_step = [&](Staged &P, uint32_t step) {
         // registers -> LDS
         if (has_w) {
-            gemm_codes_block<QT>(sW + r_w * kGemmLd + b_w * 32, P.wvalid, P.c0, P.c1);
+            gemm_codes_block<QT>(sW + r_w * kGemmLd + b_w * 32, P.c0, P.c1);
             sD[b_w][r_w] = P.wvalid ? mat_scale_value(a.w, P.dbits) : 0.f;
         }
 #pragma unroll
