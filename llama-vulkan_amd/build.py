@@ -55,6 +55,8 @@ def build_mkggml():
 def build_host():
     host = os.path.join(PKG, "host")
     srcs = [os.path.join(host, f) for f in sorted(os.listdir(host)) if f.endswith(".cpp") and f != "main.cpp"]
+    server = os.path.join(host, "server")
+    srcs += [os.path.join(server, f) for f in sorted(os.listdir(server)) if f.endswith(".cpp")]
     if not srcs:
         return None
     common = ["g++", "-std=c++17", "-O2", "-fPIC", "-Wall", "-Wextra", "-pthread", "-I", os.path.join(ROOT, "include")]

@@ -3,11 +3,13 @@
 // llava_session and adds nothing.
 #include <cstring>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "ggml_file.h"
 #include "llava_context.h"
 #include "llava_session.h"
+#include "server/server.h"
 
 namespace {
 unsigned copy_out(const std::string &s, char *out, unsigned cap)
@@ -76,6 +78,33 @@ void llh_context_free(void *c) { delete static_cast<llava_context *>(c); }
 int llh_context_load(void *c, const char *path, int device) { return static_cast<llava_context *>(c)->load_model(path, device) ? 0 : -1; }
 unsigned llh_context_error(void *c, char *out, unsigned cap) { return copy_out(static_cast<llava_context *>(c)->last_error(), out, cap); }
 int llh_context_run(void *c, int argc, char **argv) { return static_cast<llava_context *>(c)->run(argc, argv); }
+int llh_context_open_file(void *c, const char *path) { return static_cast<llava_context *>(c)->open_model_file(path) ? 0 : -1; }
+
+// ---- lsrv::llava_server: open() + serve_forever() on a thread of its own ----------------------------------
+struct llh_server {
+    lsrv::llava_server server;
+    std::thread loop;
+    llh_server(llava_context *c, unsigned short port, const char *bind) : server(c, port, bind) {}
+};
+// null when the socket cannot be opened
+void *llh_server_start(void *c, unsigned short port, const char *bind_address)
+{
+    llh_server *s = new llh_server(static_cast<llava_context *>(c), port, bind_address);
+    if (!s->server.open()) {
+        delete s;
+        return nullptr;
+    }
+    s->loop = std::thread([s] { s->server.serve_forever(); });
+    return s;
+}
+unsigned llh_server_port(void *s) { return static_cast<llh_server *>(s)->server.bound_port(); }
+void llh_server_stop(void *h)
+{
+    llh_server *s = static_cast<llh_server *>(h);
+    s->server.request_stop();
+    s->loop.join();
+    delete s;
+}
 
 // ---- llava_session ----------------------------------------------------------------------------------------
 void *llh_session_new(void *c) { return new llava_session(static_cast<llava_context *>(c)); }

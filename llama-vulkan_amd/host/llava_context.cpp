@@ -1,6 +1,6 @@
 // llava_context.cpp — model load onto the device and the command line front end.
-// The reference's run() (llava_context.cpp:151-380) also brings up Vulkan and starts the TCP server; here
-// device bring-up is lv_ctx_create + lv_model_upload and the server is not part of this build.
+// The reference's run() (llava_context.cpp:151-380) also brings up Vulkan; here device bring-up is lv_ctx_create +
+// lv_model_upload.  With -s the loaded model is handed to the token server (server/server.h).
 #include "llava_context.h"
 
 #include <cstdlib>
@@ -10,6 +10,7 @@
 
 #include "llava_hip.h"
 #include "llava_session.h"
+#include "server/server.h"
 
 llava_context::llava_context() = default;
 
@@ -18,6 +19,22 @@ llava_context::~llava_context()
     if (device_model) lv_model_destroy(device_model);
     if (device_ctx) lv_ctx_destroy(device_ctx);
     delete model;
+}
+
+bool llava_context::open_model_file(const std::string &path)
+{
+    if (model) {
+        problem = "a model is already loaded";
+        return false;
+    }
+    ggml_file *file = new ggml_file(path.c_str());
+    if (!file->is_open()) {
+        problem = file->error();
+        delete file;
+        return false;
+    }
+    model = file;
+    return true;
 }
 
 bool llava_context::load_model(const std::string &path, int device)
@@ -60,17 +77,20 @@ bool llava_context::load_model(const std::string &path, int device)
 static void print_usage(const char *argv0)
 {
     std::cerr << "usage: " << argv0 << " [-m|--model FILE] [--print_header] [--greedy] [--seed N] [-n TOKENS] [-d DEVICE] [-v] [-h] [PROMPT]\n"
+              << "       " << argv0 << " [-m|--model FILE] -s|--server [--port N] [--bind ADDRESS]\n"
               << "       the model path may also come from the LLAVA_MODEL environment variable\n";
 }
 
 // Flags of the reference kept: -m/--model, --print_header, -h, -v, trailing positional prompt, LLAVA_MODEL
 // (llava_context.cpp:163-212).  --use-prebuilt, --debug and --sigdebug concern Vulkan shader builds, the
-// validation layer and signalfd debugging and are accepted and ignored; -s/--server is refused (no server here).
+// validation layer and signalfd debugging and are accepted and ignored.  -s/--server starts the token server after
+// the model is loaded (llava_context.cpp:333-336); --port and --bind are additions (the reference listens on 0.0.0.0:1337).
 int llava_context::run(int argc, char **argv)
 {
     std::string path, prompt;
-    bool print_header = false, greedy = false, have_seed = false;
-    u32 seed = 0, max_new = ~0u;
+    bool print_header = false, greedy = false, have_seed = false, server_mode = false;
+    u32 seed = 0, max_new = ~0u, port = 1337;
+    std::string bind_address = "0.0.0.0";
     int device = 0;
     for (int i = 1; i < argc; ++i) {
         const std::string a = argv[i];
@@ -86,7 +106,9 @@ int llava_context::run(int argc, char **argv)
         else if (a == "--print_header") print_header = true;
         else if (a == "--greedy") greedy = true;
         else if (a == "--use-prebuilt" || a == "--debug" || a == "--sigdebug") continue;
-        else if (a == "-s" || a == "--server") { std::cerr << "the TCP server is not part of this build" << std::endl; return 1; }
+        else if (a == "-s" || a == "--server") server_mode = true;
+        else if (a == "--port") { const char *v = value("--port"); if (!v) return 1; port = static_cast<u32>(std::strtoul(v, nullptr, 0)); }
+        else if (a == "--bind") { const char *v = value("--bind"); if (!v) return 1; bind_address = v; }
         else if (a == "-m" || a == "--model") { const char *v = value("--model"); if (!v) return 1; path = v; }
         else if (a == "--seed") { const char *v = value("--seed"); if (!v) return 1; seed = static_cast<u32>(std::strtoul(v, nullptr, 0)); have_seed = true; }
         else if (a == "-n") { const char *v = value("-n"); if (!v) return 1; max_new = static_cast<u32>(std::strtoul(v, nullptr, 0)); }
@@ -102,6 +124,9 @@ int llava_context::run(int argc, char **argv)
         }
         path = env;
     }
+    // before the device runtime starts its threads: they inherit the mask (llava_context.cpp:284-287 sets up its
+    // signalfd at the same point)
+    if (server_mode) lsrv::llava_server::block_termination_signals();
     if (!load_model(path, device)) return 1;
     if (print_header) model->print_info();
     if (verbosity) {
@@ -110,6 +135,14 @@ int llava_context::run(int argc, char **argv)
         uint64_t hbm = 0;
         if (lv_ctx_info(device_ctx, name, sizeof name, &cus, &hbm) == LV_OK)
             std::cout << "Selected device: " << name << ", " << cus << " compute units, " << (hbm >> 30) << " GiB" << std::endl;
+    }
+    if (server_mode) {
+        if (port > 65535) {
+            std::cerr << "--port " << port << " is not a TCP port" << std::endl;
+            return 1;
+        }
+        lsrv::llava_server server(this, static_cast<u16>(port), bind_address);
+        return server.serve_forever() ? 0 : 1;
     }
     if (prompt.empty()) return 0;
 

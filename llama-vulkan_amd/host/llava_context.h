@@ -24,6 +24,9 @@ public:
 
     // Opens and uploads a model without going through argv.  False + message on stderr when anything fails.
     bool load_model(const std::string &path, int device = 0);
+    // Opens and parses the file only: vocabulary and tensor table are available, sessions are not (for tools that
+    // run without a device).
+    bool open_model_file(const std::string &path);
 
     [[nodiscard]] const ggml_file *get_model() const { return model; }
     [[nodiscard]] lv_ctx *get_device_context() const { return device_ctx; }

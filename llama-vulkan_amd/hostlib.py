@@ -31,6 +31,8 @@ def lib():
             "llh_file_tokenize": (u, [vp, cp, u, C.c_int, C.POINTER(u), u]), "llh_file_detokenize": (u, [vp, C.POINTER(u), u, cp, u]),
             "llh_context_new": (vp, []), "llh_context_free": (None, [vp]), "llh_context_load": (C.c_int, [vp, cp, C.c_int]),
             "llh_context_error": (u, [vp, cp, u]), "llh_context_run": (C.c_int, [vp, C.c_int, C.POINTER(cp)]),
+            "llh_context_open_file": (C.c_int, [vp, cp]),
+            "llh_server_start": (vp, [vp, C.c_ushort, cp]), "llh_server_port": (u, [vp]), "llh_server_stop": (None, [vp]),
             "llh_session_new": (vp, [vp]), "llh_session_free": (None, [vp]), "llh_session_good": (C.c_int, [vp]),
             "llh_session_set_text": (C.c_int, [vp, cp, u]), "llh_session_add_text": (C.c_int, [vp, cp, u]),
             "llh_session_push_token": (C.c_int, [vp, u]), "llh_session_token_count": (u, [vp]), "llh_session_tokens": (u, [vp, C.POINTER(u), u]),
@@ -120,12 +122,32 @@ class LlavaContext:
     def load_model(self, path, device=0):
         return lib().llh_context_load(self.h, os.fsencode(path), device) == 0
 
+    def open_model_file(self, path):
+        """parse only: vocabulary and tensor table, no device"""
+        return lib().llh_context_open_file(self.h, os.fsencode(path)) == 0
+
     def error(self):
         return _text(lib().llh_context_error, self.h)
 
     def close(self):
         if self.h:
             lib().llh_context_free(self.h)
+            self.h = None
+
+
+class LlavaServer:
+    """lsrv::llava_server running its poll loop on a thread of its own; port 0 takes a free port"""
+
+    def __init__(self, ctx, port=0, bind_address="127.0.0.1"):
+        self.h = lib().llh_server_start(ctx.h, port, bind_address.encode())
+        if not self.h:
+            raise OSError("the server socket could not be opened")
+        self.port = lib().llh_server_port(self.h)
+
+    def stop(self):
+        """kills the sessions, waits for their threads, closes the connections"""
+        if self.h:
+            lib().llh_server_stop(self.h)
             self.h = None
 
 

@@ -255,8 +255,8 @@ def test_cli_prints_the_greedy_continuation(hl, orc, loaded):
     r = subprocess.run([exe, "-m", path, "--greedy", "-n", "12", PROMPT.decode()], capture_output=True, timeout=120)
     assert r.returncode == 0, r.stderr.decode(errors="replace")
     assert r.stdout.rstrip(b"\n") == text.rstrip(b"\n")
-    r = subprocess.run([exe, "-m", path, "-s", "x"], capture_output=True, timeout=60)
-    assert r.returncode != 0                       # the server mode is not part of this build
+    r = subprocess.run([exe, "-m", path, "-s", "--port", "70000"], capture_output=True, timeout=60)
+    assert r.returncode != 0 and b"port" in r.stderr
     r = subprocess.run([exe, "-m", path + ".absent", "hi"], capture_output=True, timeout=60)
     assert r.returncode != 0 and b"absent" in r.stderr
 
