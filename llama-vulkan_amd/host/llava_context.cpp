@@ -3,6 +3,7 @@
 // lv_model_upload.  With -s the loaded model is handed to the token server (server/server.h).
 #include "llava_context.h"
 
+#include <csignal>
 #include <cstdlib>
 #include <cstring>
 #include <iostream>
@@ -73,6 +74,11 @@ bool llava_context::load_model(const std::string &path, int device)
     model = file;
     return true;
 }
+
+// SIGINT / SIGTERM during the token loop end the generation after the current token (llava_context.cpp:352 polls its
+// signalfd at the same place)
+static volatile std::sig_atomic_t g_interrupted = 0;
+static void note_interrupt(int) { g_interrupted = 1; }
 
 static void print_usage(const char *argv0)
 {
@@ -154,6 +160,9 @@ int llava_context::run(int argc, char **argv)
         std::cerr << "[!] System prompt overflows backlog buffer !" << std::endl;
         return 1;
     }
+    g_interrupted = 0;
+    auto old_int = std::signal(SIGINT, note_interrupt);
+    auto old_term = std::signal(SIGTERM, note_interrupt);
     std::cout << prompt << std::flush;
     u32 next = session.predict_next_token(greedy);
     u32 produced = 0;
@@ -162,7 +171,7 @@ int llava_context::run(int argc, char **argv)
             std::cerr << "Unknown error" << std::endl;
             break;
         }
-        if (next == eos_id || produced >= max_new) break;
+        if (g_interrupted || next == eos_id || produced >= max_new) break;
         if (!session.push_token(next)) break;  // context full
         if (!session.start_next_token_prediction()) {
             std::cerr << "Cannot start processing, unknown error" << std::endl;
@@ -174,5 +183,7 @@ int llava_context::run(int argc, char **argv)
     }
     if (~next != 0 && next != eos_id && produced < max_new) std::cout << model->get_tokens()[next].text;
     std::cout << std::endl;
+    std::signal(SIGINT, old_int);
+    std::signal(SIGTERM, old_term);
     return 0;
 }

@@ -296,3 +296,22 @@ def test_two_threads_two_sessions_one_model(lva, orc, ctx, tmp_path):
         t.join()
     assert together == alone
     model.close()
+
+
+def test_command_line_stops_at_a_signal(tiny_models):
+    """an interrupt ends the token loop after the current token and the program exits normally (llava_context.cpp:352)"""
+    import signal
+    import time
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "llama-vulkan_amd", "bin", "llava")
+    # the context holds 2048 tokens at most; without the signal the run would go on to that limit
+    p = subprocess.Popen([exe, "-m", tiny_models["tiny_q4"], "--greedy", PROMPT.decode()], stdout=subprocess.PIPE, stderr=subprocess.PIPE)
+    try:
+        time.sleep(1.0)
+        if p.poll() is None:
+            p.send_signal(signal.SIGINT)
+        assert p.wait(timeout=60) == 0
+        assert p.stdout.read().startswith(PROMPT)
+    finally:
+        if p.poll() is None:
+            p.kill()
+            p.wait()
