@@ -157,3 +157,51 @@ def test_7b_q8_0_long_context_steps_match_oracle(lva, orc, ctx):
         assert s.argmax() == tok, step
         pos += 1
     s.close(); model.close(); osess.close(); om.close()
+
+
+def test_13b_q8_0_prompt_of_512_as_one_batch(lva, orc, ctx):
+    """the prompt case at full size: 512 tokens through the matrix-core GEMM and the batched attention of a 40-layer 13B
+    q8_0 model.  The oracle would need minutes for this on the CPU, so the check is in two steps that together reach
+    it: (1) the same 512 tokens evaluated one by one by the persistent kernel, whose steps are pinned against the
+    oracle (above, and at every tile shape in tests/test_gpu_model.py), must leave the same cache rows and logits
+    within TWICE the tolerance (two paths that each round fp16 cache rows their own way, 40 layers deep: if each is
+    within the tolerance of the exact result they are within twice of each other; measured: 0.004 typical, 0.018 the
+    worst of 32000 logits of magnitude 5); (2) from a copy of that cache the oracle itself evaluates the next token,
+    at the tolerance itself."""
+    path = _model_file(lva, "13b_q8_0", lva.LV_Q8_0, 3, SHAPE_13B)
+    model = lva.Model(ctx, path)
+    n = 512
+    prompt = lva.synth_tokens(n, 3, SHAPE_13B["vocab"], seed=3)
+    batch, single = lva.Session(model, 1024), lva.Session(model, 1024)
+    assert single.path() == lva.PATH_PERSISTENT
+    batch.begin(prompt, 0)
+    got = batch.logits().copy()
+    for i in range(n):
+        single.begin(prompt[i:i + 1], i)
+        single.wait()
+    want = single.logits().copy()
+    assert np.all(np.abs(got - want) <= 2 * (1e-2 + 1e-3 * np.abs(want))), float(np.max(np.abs(got - want)))
+    assert batch.argmax() == single.argmax()
+    # cache rows: fp16 values of fp32 sums taken in two different orders; they may differ by an fp16 ulp where a sum
+    # falls near a rounding boundary, and by more only through error carried from layer to layer
+    for layer, bound in ((0, 2.0 ** -10), (19, 1e-2), (39, 1e-2)):
+        for which in (0, 1):
+            a = batch.kv(layer, which, n).view(np.float16).astype(np.float32)
+            b = single.kv(layer, which, n).view(np.float16).astype(np.float32)
+            worst = float(np.max(np.abs(a - b))) / float(np.max(np.abs(b)))
+            assert worst <= bound, (layer, which, worst)
+    # the oracle continues from the batch path's cache
+    om = orc.Model(path)
+    osess = orc.Session(om, 1024)
+    for layer in range(SHAPE_13B["layers"]):
+        for which in (0, 1):
+            osess.kv_load(layer, which, batch.kv(layer, which, n))
+    osess.set_pos(n)
+    tok = batch.argmax()
+    ref = osess.eval(np.array([tok], dtype=np.uint32))
+    batch.begin([tok], n)
+    nxt = batch.logits()
+    assert np.all(np.abs(nxt - ref) <= 1e-2 + 1e-3 * np.abs(ref)), float(np.max(np.abs(nxt - ref)))
+    assert batch.argmax() == orc.greedy(ref)
+    for h in (batch, single, model, osess, om):
+        h.close()
