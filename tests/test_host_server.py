@@ -124,3 +124,37 @@ def test_stop_with_live_sessions_and_clients(hl, tmp_path):
         for _ in range(16):
             c.read_packet()
     c.close(); ctx.close()
+
+
+def test_random_bytes_do_not_hurt_the_server(served):
+    """whatever one client sends, the others are served: random packets with plausible headers, then pure noise"""
+    import random
+    server, _ = served
+    rng = random.Random(5)
+    good = sc.Client(server.port)
+    sid = good.new_session()
+    for round_ in range(20):
+        bad = sc.Client(server.port, timeout=0.2)
+        blob = b""
+        for _ in range(50):
+            command = rng.choice([0, 1, 2, 3, 15, 16, 17, 19, 20, 22, 23, 31, 32, 33, 34, 35, 36, 37, 38, 39, 1 << 31])
+            length = rng.choice([0, 1, 3, 4, 5, 8, 9, 64])
+            body = bytes(rng.getrandbits(8) for _ in range(length))
+            if length >= 4 and rng.random() < 0.5:
+                body = struct.pack("<I", rng.choice([sid, sid + 1, 0])) + body[4:]
+            if command in (36, 37, 38) and len(body) > 4:
+                body = body[:4] + b"/nonexistent-dir/" + bytes(b % 26 + 97 for b in body[4:])     # never a real path
+            blob += struct.pack("<3I", command, rng.getrandbits(32), len(body)) + body
+        if round_ % 2:
+            blob += bytes(rng.getrandbits(8) for _ in range(rng.randrange(1, 4000)))
+        try:
+            bad.send_raw(blob)
+        except OSError:
+            pass
+        bad.close()
+        listed = good.sessions()
+        assert listed == sorted(listed) and all(s >= sid for s in listed)     # random cmdNewSession packets may have added some
+        if sid not in listed:                                                  # ... and a random cmdKillSession may have hit ours
+            sid = good.new_session()
+    assert good.ack(sc.SUBSCRIBE, sid) == sc.RC_OK
+    good.close()
