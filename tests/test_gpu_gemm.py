@@ -18,7 +18,7 @@ def _abs_dot_bound(orc, blocks, ftype, rows, cols, x):
     (256, 4096, 130, False),     # a second, almost empty token tile
     (704, 256, 17, True),        # rows not a multiple of the tile, residual add
     (96, 1376, 200, False),      # K = 43 blocks: a half K step at the end, fewer rows than a tile
-    (4096, 4096, 512, True),     # the 7B attention shape at the batch of BASELINE's prompt case
+    (4096, 4096, 512, True),     # the 7B attention shape at a 512-token prompt batch
 ])
 def test_gemm_matches_oracle(lva, orc, ctx, ftype_name, rows, cols, batch, accumulate):
     ftype = lva.LV_Q4_0 if ftype_name == "q4_0" else lva.LV_Q8_0
