@@ -481,7 +481,9 @@ static void launch_gemv_mode(const GemvArgs &a, uint32_t batch, hipStream_t st)
         const uint32_t rows_per_wg = (a.w.rows + 255) / 256;
         const uint32_t ns = (nb + 63) / 64, nr = kWideWaves / ns, per_set = (rows_per_wg + nr - 1) / nr;
         const size_t red_bytes = (size_t)per_set * nr * (MODE == kGemvSilu ? 2 : 1) * ns * sizeof(float);
-        gemv_wide_kernel<QT, MODE><<<dim3((a.w.rows + rows_per_wg - 1) / rows_per_wg, batch), dim3(kWideWaves * 64), red_bytes, st>>>(a, rows_per_wg);
+        const dim3 grid((a.w.rows + rows_per_wg - 1) / rows_per_wg, batch);
+        if (a.w.scales_f32) gemv_wide_kernel<QT, MODE, true><<<grid, dim3(kWideWaves * 64), red_bytes, st>>>(a, rows_per_wg);
+        else gemv_wide_kernel<QT, MODE, false><<<grid, dim3(kWideWaves * 64), red_bytes, st>>>(a, rows_per_wg);
         return;
     }
     if (nb <= 64) launch_gemv_cfg<QT, MODE, 1, 1>(a, batch, st);
@@ -498,6 +500,8 @@ static int launch_gemv(hipStream_t st, float *out, const lv_matrix &w, const lv_
     GemvArgs a{};
     a.w = w.view;
     if (w1) a.w1 = w1->view;
+    if (w1 && (w1->view.scales_f32 != nullptr) != (w.view.scales_f32 != nullptr))
+        return fail(LV_ERR_ARG, "gemv: the two matrices come from different file versions (fp16 and fp32 block scales)");
     a.x = x;
     a.out = out;
     a.norm_w = norm_w;
@@ -524,7 +528,9 @@ static bool gemv3_streams(const lv_matrix *const w[3])
 {
     const lv_matrix &w0 = *w[0];
     bool same = true;
-    for (int i = 1; i < 3; i++) same = same && w[i]->ftype == w0.ftype && w[i]->view.rows == w0.view.rows && w[i]->view.cols == w0.view.cols;
+    for (int i = 1; i < 3; i++)
+        same = same && w[i]->ftype == w0.ftype && w[i]->view.rows == w0.view.rows && w[i]->view.cols == w0.view.cols &&
+               (w[i]->view.scales_f32 != nullptr) == (w0.view.scales_f32 != nullptr);
     return same && gemv_streams(w0.view, 1);
 }
 static int launch_gemv3(hipStream_t st, float *const out[3], const lv_matrix *const w[3], const float *x, const Gemv3Extras *ex = nullptr)
@@ -544,8 +550,14 @@ static int launch_gemv3(hipStream_t st, float *const out[3], const lv_matrix *co
         const uint32_t ns = (nb + 63) / 64, nr = kWideWaves / ns, per_set = (rows_per_wg + nr - 1) / nr;
         const size_t red_bytes = (size_t)per_set * nr * ns * sizeof(float);
         const dim3 grid((rows + rows_per_wg - 1) / rows_per_wg, 3);
-        if (w0.ftype == LV_Q4_0) gemv_wide3_kernel<4><<<grid, dim3(kWideWaves * 64), red_bytes, st>>>(a, rows_per_wg);
-        else gemv_wide3_kernel<8><<<grid, dim3(kWideWaves * 64), red_bytes, st>>>(a, rows_per_wg);
+        const bool sf32 = w0.view.scales_f32 != nullptr;
+        if (w0.ftype == LV_Q4_0) {
+            if (sf32) gemv_wide3_kernel<4, true><<<grid, dim3(kWideWaves * 64), red_bytes, st>>>(a, rows_per_wg);
+            else gemv_wide3_kernel<4, false><<<grid, dim3(kWideWaves * 64), red_bytes, st>>>(a, rows_per_wg);
+        } else {
+            if (sf32) gemv_wide3_kernel<8, true><<<grid, dim3(kWideWaves * 64), red_bytes, st>>>(a, rows_per_wg);
+            else gemv_wide3_kernel<8, false><<<grid, dim3(kWideWaves * 64), red_bytes, st>>>(a, rows_per_wg);
+        }
         HIP_TRY(hipGetLastError());
         return LV_OK;
     }
@@ -709,12 +721,13 @@ static int launch_gemm_presplit(hipStream_t st, float *out, uint32_t ldo, const 
     const uint32_t token_tiles = n_pad / kGemmTile;
     const bool narrow = (uint64_t)((w.view.rows + 127) / 128) * token_tiles < 128;
     const dim3 grid((w.view.rows + (narrow ? 63 : 127)) / (narrow ? 64 : 128), token_tiles);
+    const bool sf32 = w.view.scales_f32 != nullptr;
     if (w.ftype == LV_Q4_0) {
-        if (narrow) gemm_kernel<4, 64><<<grid, dim3(256), 0, st>>>(a);
-        else gemm_kernel<4, 128, 8><<<grid, dim3(512), 0, st>>>(a);
+        if (narrow) { if (sf32) gemm_kernel<4, 64, 4, true><<<grid, dim3(256), 0, st>>>(a); else gemm_kernel<4, 64, 4, false><<<grid, dim3(256), 0, st>>>(a); }
+        else { if (sf32) gemm_kernel<4, 128, 8, true><<<grid, dim3(512), 0, st>>>(a); else gemm_kernel<4, 128, 8, false><<<grid, dim3(512), 0, st>>>(a); }
     } else if (w.ftype == LV_Q8_0) {
-        if (narrow) gemm_kernel<8, 64><<<grid, dim3(256), 0, st>>>(a);
-        else gemm_kernel<8, 128, 8><<<grid, dim3(512), 0, st>>>(a);
+        if (narrow) { if (sf32) gemm_kernel<8, 64, 4, true><<<grid, dim3(256), 0, st>>>(a); else gemm_kernel<8, 64, 4, false><<<grid, dim3(256), 0, st>>>(a); }
+        else { if (sf32) gemm_kernel<8, 128, 8, true><<<grid, dim3(512), 0, st>>>(a); else gemm_kernel<8, 128, 8, false><<<grid, dim3(512), 0, st>>>(a); }
     }
     else return fail(LV_ERR_ARG, "gemm: matrix type %u", w.ftype);
     HIP_TRY(hipGetLastError());

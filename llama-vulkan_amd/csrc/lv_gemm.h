@@ -124,7 +124,7 @@ __device__ __forceinline__ void gemm_codes_block(uint16_t *w, const uint4 &c0, c
 // RM = weight rows per workgroup (128 or 64); tokens per workgroup: 128.  The four waves split the tile 2 x 2
 // (RM = 128: 64 tokens x 64 rows each) or 4 x 1 (RM = 64: 32 tokens x 64 rows each).  The narrow form doubles the
 // number of workgroups for matrices that would otherwise not fill 256 CUs.
-template <int QT, int RM, int NWV = 4>
+template <int QT, int RM, int NWV = 4, bool SF32 = false /* fp32 scale plane (file version 1) */>
 __global__ __launch_bounds__(NWV * 64) void gemm_kernel(GemmArgs a)
 {
     constexpr int CPB = QT == 4 ? 1 : 2;          // uint4 of codes per block
@@ -167,7 +167,8 @@ __global__ __launch_bounds__(NWV * 64) void gemm_kernel(GemmArgs a)
             const size_t sb = (size_t)(p.wvalid ? wrow : 0) * nb + (p.wvalid ? blk : 0);
             p.c0 = a.w.codes[sb * CPB];
             if constexpr (QT == 8) p.c1 = a.w.codes[sb * CPB + 1];
-            p.dbits = mat_scale_raw(a.w, sb);
+            if constexpr (SF32) p.dbits = __float_as_uint(a.w.scales_f32[sb]);
+            else p.dbits = a.w.scales[sb];
         }
         const uint32_t k = step * kGemmK + xc;
         const bool kok = k < K;
@@ -194,7 +195,7 @@ __global__ __launch_bounds__(NWV * 64) void gemm_kernel(GemmArgs a)
         // registers -> LDS
         if (has_w) {
             gemm_codes_block<QT>(sW + r_w * kGemmLd + b_w * 32, P.c0, P.c1);
-            sD[b_w][r_w] = P.wvalid ? mat_scale_value(a.w, P.dbits) : 0.f;
+            sD[b_w][r_w] = !P.wvalid ? 0.f : SF32 ? __uint_as_float(P.dbits) : half_bits_to_float((uint16_t)P.dbits);
         }
 #pragma unroll
         for (int i = 0; i < XP; i++) {

@@ -23,7 +23,9 @@ struct WideTile {
     uint32_t d;     // raw scale word (fp16 bits, or fp32 bits for a version-1 file)
 };
 
-template <int QT>
+// SF32: the matrix has an fp32 scale plane (file version 1).  A template parameter, not a test of the view: a branch
+// per tile would stand between the loads of the queue, and the queue only runs ahead through straight-line code.
+template <int QT, bool SF32>
 __device__ __forceinline__ void wide_load(WideTile &t, const MatView &m, uint64_t blk, bool ok)
 {
     const uint64_t b = ok ? blk : 0;     // rows / lanes without a block read block 0 and are discarded
@@ -33,14 +35,16 @@ __device__ __forceinline__ void wide_load(WideTile &t, const MatView &m, uint64_
         t.c = m.codes[2 * b];
         t.c2 = m.codes[2 * b + 1];
     }
-    t.d = mat_scale_raw(m, b);
+    if constexpr (SF32) t.d = __float_as_uint(m.scales_f32[b]);
+    else t.d = m.scales[b];
 }
 
-template <int QT>
-__device__ __forceinline__ float wide_dot(const WideTile &t, const MatView &m, const float (&x)[32], float xsum)
+template <int QT, bool SF32>
+__device__ __forceinline__ float wide_dot(const WideTile &t, const float (&x)[32], float xsum)
 {
-    if constexpr (QT == 4) return (q4_block_dot(t.c, x) - 8.f * xsum) * mat_scale_value(m, t.d);
-    else return (q8_block_dot(t.c, t.c2, x) - 128.f * xsum) * mat_scale_value(m, t.d);
+    const float d = SF32 ? __uint_as_float(t.d) : half_bits_to_float((uint16_t)t.d);
+    if constexpr (QT == 4) return (q4_block_dot(t.c, x) - 8.f * xsum) * d;
+    else return (q8_block_dot(t.c, t.c2, x) - 128.f * xsum) * d;
 }
 
 // Workgroup barrier that orders LDS traffic only: the weight loads in flight stay in flight.
@@ -64,7 +68,7 @@ __device__ __forceinline__ float wide_block_sum(float v, float *scratch, int w, 
 }
 
 // NMAT = 2: the SiLU form, rows of w (W3) and w1 (W1) with the same index are walked together.
-template <int QT, int MODE>
+template <int QT, int MODE, bool SF32>
 __device__ __forceinline__ void gemv_wide_body(const GemvArgs &a, uint32_t rows_per_wg, uint32_t z /* batch row */, float *xs, float *red,
                                                float *stat /* 32 floats */)
 {
@@ -88,8 +92,8 @@ __device__ __forceinline__ void gemv_wide_body(const GemvArgs &a, uint32_t rows_
         const uint32_t r = (uint32_t)rset * per_set + i;
         const bool ok = lane_ok && i < per_set && r < n_rows;
         const uint64_t blk = (uint64_t)(row0 + r) * nb + blk_col;
-        wide_load<QT>(q[0][slot], a.w, blk, ok);
-        if constexpr (NMAT == 2) wide_load<QT>(q[1][slot], a.w1, blk, ok);
+        wide_load<QT, SF32>(q[0][slot], a.w, blk, ok);
+        if constexpr (NMAT == 2) wide_load<QT, SF32>(q[1][slot], a.w1, blk, ok);
     };
 #pragma unroll
     for (int i = 0; i < DEPTH; i++) fetch(i, i);
@@ -138,7 +142,7 @@ __device__ __forceinline__ void gemv_wide_body(const GemvArgs &a, uint32_t rows_
 #pragma unroll
             for (int j = 0; j < 4; j++) {
 #pragma unroll
-                for (int mi = 0; mi < NMAT; mi++) p[mi][j] = wide_dot<QT>(q[mi][g + j], mi == 0 ? a.w : a.w1, xr, xsum);
+                for (int mi = 0; mi < NMAT; mi++) p[mi][j] = wide_dot<QT, SF32>(q[mi][g + j], xr, xsum);
                 fetch(g + j, i0 + g + j + DEPTH);
             }
 #pragma unroll
@@ -178,26 +182,26 @@ __device__ __forceinline__ void gemv_wide_body(const GemvArgs &a, uint32_t rows_
     }
 }
 
-template <int QT, int MODE>
+template <int QT, int MODE, bool SF32 = false>
 __global__ __launch_bounds__(kWideWaves * 64) void gemv_wide_kernel(GemvArgs a, uint32_t rows_per_wg)
 {
     __shared__ __attribute__((aligned(16))) float xs[kWideMaxK];
     __shared__ float stat[32];
     extern __shared__ float red[];       // [rows_per_wg rounded up to 4*NR][NMAT][NS]
-    gemv_wide_body<QT, MODE>(a, rows_per_wg, blockIdx.y, xs, red, stat);
+    gemv_wide_body<QT, MODE, SF32>(a, rows_per_wg, blockIdx.y, xs, red, stat);
 }
 
 // Three matrices with the same input vector in one launch (Wq, Wk, Wv of a layer): blockIdx.y selects the matrix.
 struct GemvArgs3 {
     GemvArgs m[3];
 };
-template <int QT>
+template <int QT, bool SF32 = false>
 __global__ __launch_bounds__(kWideWaves * 64) void gemv_wide3_kernel(GemvArgs3 a, uint32_t rows_per_wg)
 {
     __shared__ __attribute__((aligned(16))) float xs[kWideMaxK];
     __shared__ float stat[32];
     extern __shared__ float red[];
-    gemv_wide_body<QT, kGemvStore>(a.m[blockIdx.y], rows_per_wg, 0, xs, red, stat);
+    gemv_wide_body<QT, kGemvStore, SF32>(a.m[blockIdx.y], rows_per_wg, 0, xs, red, stat);
 }
 
 }  // namespace lv
