@@ -5,6 +5,7 @@
     python llama-vulkan_amd/measure.py decode-q8     7B q8_0, cache positions 1920..2047 (128 greedy steps)
     python llama-vulkan_amd/measure.py decode-13b    13B q4_0, 32-token prompt + 256 greedy steps
     python llama-vulkan_amd/measure.py prefill-13b   13B q8_0, 512-token prompt evaluated in one lv_step_begin
+    python llama-vulkan_amd/measure.py gemm          isolated 512-token GEMMs at the 13B shapes, q8_0 (for kernel traces and counters)
     python llama-vulkan_amd/measure.py copy          1 GiB device-to-device copy: achievable bandwidth, counter calibration
     python llama-vulkan_amd/measure.py all
 
@@ -145,6 +146,25 @@ def prefill_case(ctx):
     model.close()
 
 
+def gemm_cases(ctx):
+    """lv_kernel_gemm allocates its workspace and splits the activations in every call, so the time of a call is not the
+    kernel's: this case exists to put gemm_kernel launches of known shape under rocprofv3 (kernel trace, counters)"""
+    n, wtype = 512, lva.LV_Q8_0
+    for rows, cols in ((5120, 5120), (13824, 5120), (5120, 13824)):
+        m = ctx.matrix(lva.synth_quant(wtype, rows, cols, seed=1), wtype, rows, cols)
+        x = ctx.to_device(lva.synth_normal(n, cols, seed=2))
+        out = ctx.zeros(n * rows * 4)
+        reps = 6
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            lva.check(ctx.lib.lv_kernel_gemm(ctx.h, out, m, x, n, 0))
+        ctx.sync()
+        emit(case="gemm", wtype="q8_0", rows=rows, cols=cols, tokens=n, launches=reps, us_per_call_with_workspace=round((time.perf_counter() - t0) / reps * 1e6, 1))
+        ctx.matrix_free(m)
+        ctx.free(x)
+        ctx.free(out)
+
+
 def main():
     which = sys.argv[1] if len(sys.argv) > 1 else "all"
     ctx = lva.Context(0)
@@ -154,6 +174,8 @@ def main():
         copy_case(ctx)
     if which in ("gemv", "all"):
         gemv_cases(ctx)
+    if which == "gemm":
+        gemm_cases(ctx)
     if which in ("decode-q8", "all"):
         decode_case(ctx, "decode-q8", "7b", lva.LV_Q8_0, 1, 2048, 1916, 128)
     if which in ("decode-13b", "all"):
