@@ -10,9 +10,9 @@
 // lane: in the MFMA result a lane holds one weight row) and added to the fp32 result.  The batched path therefore
 // agrees with the one-token fp32 path to fp32 rounding, not to fp16 rounding.
 //
-// Tiling: workgroup = 256 threads = 4 waves, output tile 128 tokens x 128 (or 64) weight rows, K step 64 (two quant
-// blocks).  One thread unpacks one (row, block) pair per step; every wave owns a 64 x 64 (or 32 x 64) sub-tile of
-// v_mfma_f32_32x32x16_f16 tiles.  Global loads of step s+1 are issued before the MFMAs of step s.
+// Tiling: workgroup = 8 (or 4) waves, output tile 128 tokens x 128 (or 64) weight rows, K step 64 (two quant blocks).
+// Two threads unpack one (row, block) pair per step; every wave owns a 32-token x 64-row sub-tile of
+// v_mfma_f32_32x32x16_f16 tiles.  The global loads of step s+2 are issued before the MFMAs of step s.
 #pragma once
 
 #include "lv_kernels.h"
@@ -86,31 +86,32 @@ __host__ __device__ constexpr int gemm_k_position(int e)
     return 8 * i + 2 * j + (b >> 1);
 }
 
-// 32 codes of one block -> 32 halfs at w, in gemm_k_position order, as the integers they are (q4_0: q - 8, q8_0: q):
+// 16 codes of half a block (q8_0: 16 bytes; q4_0: 8 bytes, the two dwords whose nibbles unpack to positions
+// 16*half .. 16*half+15 of gemm_k_position order) -> 16 halfs at w, as the integers they are (q4_0: q - 8, q8_0: q):
 // 1024 + u has the fp16 bit pattern 0x6400 | u, and subtracting 1024 + offset is exact.  A block outside the matrix
 // is given the scale 0 by the caller, which removes it from the sum whatever codes were unpacked for it.
 template <int QT>
-__device__ __forceinline__ void gemm_codes_block(uint16_t *w, const uint4 &c0, const uint4 &c1)
+__device__ __forceinline__ void gemm_codes_half(uint16_t *w, const uint4 &c)
 {
-    uint32_t ph[16];
+    uint32_t ph[8];
     auto emit = [&](int slot, uint32_t packed_codes, _Float16 bias) {
         // packed_codes: two halfs 0x6400 | u
-        union { uint32_t u; lv_h2 h; } c, v;
-        c.u = packed_codes;
+        union { uint32_t u; lv_h2 h; } cc, v;
+        cc.u = packed_codes;
         const lv_h2 bb = {bias, bias};
-        v.h = c.h - bb;                              // exact: small integers
+        v.h = cc.h - bb;                             // exact: small integers
         ph[slot] = v.u;
     };
     if constexpr (QT == 4) {
-        const uint32_t q[4] = {c0.x, c0.y, c0.z, c0.w};
+        const uint32_t q[2] = {c.x, c.y};
 #pragma unroll
-        for (int i = 0; i < 4; i++)
+        for (int i = 0; i < 2; i++)
 #pragma unroll
             for (int j = 0; j < 4; j++) emit(4 * i + j, ((q[i] >> (4 * j)) & 0x000f000fu) | 0x64006400u, (_Float16)1032.f);
     } else {
-        const uint32_t q[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+        const uint32_t q[4] = {c.x, c.y, c.z, c.w};
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
+        for (int i = 0; i < 4; i++) {
             const uint32_t u = q[i] ^ 0x80808080u;   // int8 -> biased unsigned
             // one byte permute per pair: bytes (u.b0, 0x64, u.b1, 0x64) and (u.b2, 0x64, u.b3, 0x64)
             emit(2 * i, __builtin_amdgcn_perm(u, 0x64646464u, 0x00050004u), (_Float16)1152.f);
@@ -118,7 +119,7 @@ __device__ __forceinline__ void gemm_codes_block(uint16_t *w, const uint4 &c0, c
         }
     }
 #pragma unroll
-    for (int g = 0; g < 4; g++) *reinterpret_cast<uint4 *>(w + 8 * g) = make_uint4(ph[4 * g], ph[4 * g + 1], ph[4 * g + 2], ph[4 * g + 3]);
+    for (int g = 0; g < 2; g++) *reinterpret_cast<uint4 *>(w + 8 * g) = make_uint4(ph[4 * g], ph[4 * g + 1], ph[4 * g + 2], ph[4 * g + 3]);
 }
 
 // RM = weight rows per workgroup (128 or 64); tokens per workgroup: 128.  The four waves split the tile 2 x 2
@@ -127,7 +128,6 @@ __device__ __forceinline__ void gemm_codes_block(uint16_t *w, const uint4 &c0, c
 template <int QT, int RM, int NWV = 4, bool SF32 = false /* fp32 scale plane (file version 1) */>
 __global__ __launch_bounds__(NWV * 64) void gemm_kernel(GemmArgs a)
 {
-    constexpr int CPB = QT == 4 ? 1 : 2;          // uint4 of codes per block
     constexpr int TN = kGemmTile;                 // tokens per workgroup
     constexpr int WN = RM / 64;                   // waves along the rows
     constexpr int WM = NWV / WN;                  // waves along the tokens
@@ -141,37 +141,43 @@ __global__ __launch_bounds__(NWV * 64) void gemm_kernel(GemmArgs a)
     const uint32_t tok0 = blockIdx.y * TN, row0 = blockIdx.x * RM;
     const uint32_t K = a.w.cols, nb = K / 32, steps = (K + kGemmK - 1) / kGemmK;
 
-    // this thread's weight block of a step: row r_w, block (2*step + b_w); with RM = 64 half of the threads have none
-    const int r_w = tid >> 1, b_w = tid & 1;
-    const bool has_w = r_w < RM;
+    // this thread's share of the weights of a step: half h_w of block (2*step + b_w) of row r_w.  Every thread has one,
+    // and every load below is issued by every thread at every step (addresses are clamped, results discarded where
+    // there is nothing to load): the compiler can then count the loads in flight exactly and wait for the oldest set
+    // only, which a load under a condition would force it to give up.
+    static_assert(NT == RM * 4, "two threads per (row, block)");
+    const int r_w = tid >> 2, b_w = (tid >> 1) & 1, h_w = tid & 1;
     const uint32_t wrow = row0 + r_w;
-    const bool wrow_ok = has_w && wrow < a.w.rows;
-    // this thread's four 16-byte pieces of the activation tile of a step: token rows tid/8 + 32*i, halfs (tid%8)*8..+7
+    const bool wrow_ok = wrow < a.w.rows;
+    // this thread's 16-byte pieces of the activation tile of a step: token rows tid/8 + XR*i, halfs (tid%8)*8..+7
     const int xr = tid >> 3, xc = (tid & 7) * 8;
     constexpr int XR = NT / 8;                    // token rows covered per piece index
+    const uint32_t steps2 = (steps + 1) & ~1u;    // the loop takes two steps at a time; a step past the end multiplies zeros
 
     // two register sets: the loads of step s + 2 are in flight while step s is multiplied (one step of MFMAs is
     // shorter than a trip to memory)
     struct Staged {
-        uint4 c0, c1;
+        uint4 c;
         uint32_t dbits;     // raw scale word
         bool wvalid;
         uint4 gh[XP], gl[XP];
     } pre[2];
     auto fetch = [&](Staged &p, uint32_t step) {
-        const uint32_t blk = 2 * step + b_w;
-        p.wvalid = wrow_ok && blk < nb;
-        p.c0 = p.c1 = make_uint4(0, 0, 0, 0);
-        p.dbits = 0;
-        if (has_w) {
-            const size_t sb = (size_t)(p.wvalid ? wrow : 0) * nb + (p.wvalid ? blk : 0);
-            p.c0 = a.w.codes[sb * CPB];
-            if constexpr (QT == 8) p.c1 = a.w.codes[sb * CPB + 1];
-            if constexpr (SF32) p.dbits = __float_as_uint(a.w.scales_f32[sb]);
-            else p.dbits = a.w.scales[sb];
+        const bool real = step < steps;
+        const uint32_t sc = real ? step : steps - 1;
+        const uint32_t blk = 2 * sc + b_w;
+        p.wvalid = real && wrow_ok && blk < nb;
+        const size_t sb = (size_t)(p.wvalid ? wrow : 0) * nb + (p.wvalid ? blk : 0);
+        if constexpr (QT == 8) {
+            p.c = a.w.codes[sb * 2 + h_w];
+        } else {
+            const uint2 half = reinterpret_cast<const uint2 *>(a.w.codes)[sb * 2 + h_w];
+            p.c = make_uint4(half.x, half.y, 0, 0);
         }
-        const uint32_t k = step * kGemmK + xc;
-        const bool kok = k < K;
+        if constexpr (SF32) p.dbits = __float_as_uint(a.w.scales_f32[sb]);
+        else p.dbits = a.w.scales[sb];
+        const uint32_t k = sc * kGemmK + xc;
+        const bool kok = real && k < K;
 #pragma unroll
         for (int i = 0; i < XP; i++) {
             const size_t off = (size_t)(tok0 + xr + XR * i) * K + (kok ? k : 0);
@@ -190,20 +196,18 @@ __global__ __launch_bounds__(NWV * 64) void gemm_kernel(GemmArgs a)
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
     fetch(pre[0], 0);
-    if (steps > 1) fetch(pre[1], 1);
+    fetch(pre[1], 1);
     auto one_step = [&](Staged &P, uint32_t step) {
         // registers -> LDS
-        if (has_w) {
-            gemm_codes_block<QT>(sW + r_w * kGemmLd + b_w * 32, P.c0, P.c1);
-            sD[b_w][r_w] = !P.wvalid ? 0.f : SF32 ? __uint_as_float(P.dbits) : half_bits_to_float((uint16_t)P.dbits);
-        }
+        gemm_codes_half<QT>(sW + r_w * kGemmLd + b_w * 32 + h_w * 16, P.c);
+        if (h_w == 0) sD[b_w][r_w] = !P.wvalid ? 0.f : SF32 ? __uint_as_float(P.dbits) : half_bits_to_float((uint16_t)P.dbits);
 #pragma unroll
         for (int i = 0; i < XP; i++) {
             *reinterpret_cast<uint4 *>(sXh + (xr + XR * i) * kGemmLd + xc) = P.gh[i];
             *reinterpret_cast<uint4 *>(sXl + (xr + XR * i) * kGemmLd + xc) = P.gl[i];
         }
         __syncthreads();
-        if (step + 2 < steps) fetch(P, step + 2);
+        fetch(P, step + 2);
 #pragma unroll
         for (int b = 0; b < kGemmK / 32; b++) {          // the two quant blocks of the step
             lv_f16v blk[MT][2];
@@ -250,9 +254,9 @@ __global__ __launch_bounds__(NWV * 64) void gemm_kernel(GemmArgs a)
         }
         __syncthreads();
     };
-    for (uint32_t step = 0; step < steps; step += 2) {
+    for (uint32_t step = 0; step < steps2; step += 2) {
         one_step(pre[0], step);
-        if (step + 1 < steps) one_step(pre[1], step + 1);
+        one_step(pre[1], step + 1);
     }
 
     // D[i][j]: i = token within the 32-tile, j = weight row; lane l holds j = l%32 and, in register r,
