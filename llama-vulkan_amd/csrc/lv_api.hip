@@ -715,19 +715,19 @@ static int launch_gemm_presplit(hipStream_t st, float *out, uint32_t ldo, const 
     const uint32_t n_pad = (n + kGemmTile - 1) / kGemmTile * kGemmTile;
     GemmArgs a{};
     a.out = out; a.xh = xh; a.xl = xl; a.w = w.view; a.n = n; a.ldo = ldo; a.accumulate = accumulate ? 1 : 0;
-    // 128-row workgroups of eight waves (one per CU: an activation tile brought into the CU then serves twice as many
-    // rows) unless fewer than 128 of them exist: then 64-row ones of four waves, twice as many.  Measured at 512 tokens,
-    // q8_0, 5120 x 5120 / 13824 x 5120 / 5120 x 13824: 109 / 250 / 308 us against 131 / 287 / 367 us.
+    // 128-row workgroups of eight waves with two LDS buffers (one workgroup per CU) unless fewer than 128 of them
+    // exist: then 64-row ones of four waves, twice as many.  Measured at 512 tokens, q8_0, 5120 x 5120 / 13824 x 5120 /
+    // 5120 x 13824: 103 / 216 / 263 us; with one LDS buffer 106 / 224 / 280; the 64-row form at those sizes 135 / - / 355.
     const uint32_t token_tiles = n_pad / kGemmTile;
     const bool narrow = (uint64_t)((w.view.rows + 127) / 128) * token_tiles < 128;
     const dim3 grid((w.view.rows + (narrow ? 63 : 127)) / (narrow ? 64 : 128), token_tiles);
     const bool sf32 = w.view.scales_f32 != nullptr;
     if (w.ftype == LV_Q4_0) {
         if (narrow) { if (sf32) gemm_kernel<4, 64, 4, true><<<grid, dim3(256), 0, st>>>(a); else gemm_kernel<4, 64, 4, false><<<grid, dim3(256), 0, st>>>(a); }
-        else { if (sf32) gemm_kernel<4, 128, 8, true><<<grid, dim3(512), 0, st>>>(a); else gemm_kernel<4, 128, 8, false><<<grid, dim3(512), 0, st>>>(a); }
+        else { if (sf32) gemm_kernel<4, 128, 8, true, true><<<grid, dim3(512), 0, st>>>(a); else gemm_kernel<4, 128, 8, false, true><<<grid, dim3(512), 0, st>>>(a); }
     } else if (w.ftype == LV_Q8_0) {
         if (narrow) { if (sf32) gemm_kernel<8, 64, 4, true><<<grid, dim3(256), 0, st>>>(a); else gemm_kernel<8, 64, 4, false><<<grid, dim3(256), 0, st>>>(a); }
-        else { if (sf32) gemm_kernel<8, 128, 8, true><<<grid, dim3(512), 0, st>>>(a); else gemm_kernel<8, 128, 8, false><<<grid, dim3(512), 0, st>>>(a); }
+        else { if (sf32) gemm_kernel<8, 128, 8, true, true><<<grid, dim3(512), 0, st>>>(a); else gemm_kernel<8, 128, 8, false, true><<<grid, dim3(512), 0, st>>>(a); }
     }
     else return fail(LV_ERR_ARG, "gemm: matrix type %u", w.ftype);
     HIP_TRY(hipGetLastError());

@@ -125,7 +125,7 @@ __device__ __forceinline__ void gemm_codes_half(uint16_t *w, const uint4 &c)
 // RM = weight rows per workgroup (128 or 64); tokens per workgroup: 128.  The four waves split the tile 2 x 2
 // (RM = 128: 64 tokens x 64 rows each) or 4 x 1 (RM = 64: 32 tokens x 64 rows each).  The narrow form doubles the
 // number of workgroups for matrices that would otherwise not fill 256 CUs.
-template <int QT, int RM, int NWV = 4, bool SF32 = false /* fp32 scale plane (file version 1) */>
+template <int QT, int RM, int NWV = 4, bool SF32 = false /* fp32 scale plane (file version 1) */, bool DB = false /* two LDS buffers */>
 __global__ __launch_bounds__(NWV * 64) void gemm_kernel(GemmArgs a)
 {
     constexpr int TN = kGemmTile;                 // tokens per workgroup
@@ -134,8 +134,9 @@ __global__ __launch_bounds__(NWV * 64) void gemm_kernel(GemmArgs a)
     constexpr int NT = NWV * 64;                  // threads
     constexpr int XP = TN * 8 / NT;               // 16-byte pieces of an activation half-tile per thread
     constexpr int MT = TN / WM / 32;              // 32-token tiles per wave
-    __shared__ __attribute__((aligned(16))) uint16_t sXh[TN * kGemmLd], sXl[TN * kGemmLd], sW[RM * kGemmLd];
-    __shared__ float sD[2][RM];                   // scale of (block of the step, row)
+    constexpr int NBUF = DB ? 2 : 1;
+    __shared__ __attribute__((aligned(16))) uint16_t sXh_[NBUF][TN * kGemmLd], sXl_[NBUF][TN * kGemmLd], sW_[NBUF][RM * kGemmLd];
+    __shared__ float sD_[NBUF][2][RM];            // scale of (block of the step, row)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
     const uint32_t tok0 = blockIdx.y * TN, row0 = blockIdx.x * RM;
@@ -161,7 +162,7 @@ __global__ __launch_bounds__(NWV * 64) void gemm_kernel(GemmArgs a)
         uint32_t dbits;     // raw scale word
         bool wvalid;
         uint4 gh[XP], gl[XP];
-    } pre[2];
+    } pre[DB ? 3 : 2];
     auto fetch = [&](Staged &p, uint32_t step) {
         const bool real = step < steps;
         const uint32_t sc = real ? step : steps - 1;
@@ -196,18 +197,20 @@ __global__ __launch_bounds__(NWV * 64) void gemm_kernel(GemmArgs a)
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
     fetch(pre[0], 0);
-    fetch(pre[1], 1);
-    auto one_step = [&](Staged &P, uint32_t step) {
-        // registers -> LDS
+    // registers -> LDS buffer `buf`
+    auto stage = [&](const Staged &P, int buf) {
+        uint16_t *sXh = sXh_[buf], *sXl = sXl_[buf], *sW = sW_[buf];
         gemm_codes_half<QT>(sW + r_w * kGemmLd + b_w * 32 + h_w * 16, P.c);
-        if (h_w == 0) sD[b_w][r_w] = !P.wvalid ? 0.f : SF32 ? __uint_as_float(P.dbits) : half_bits_to_float((uint16_t)P.dbits);
+        if (h_w == 0) sD_[buf][b_w][r_w] = !P.wvalid ? 0.f : SF32 ? __uint_as_float(P.dbits) : half_bits_to_float((uint16_t)P.dbits);
 #pragma unroll
         for (int i = 0; i < XP; i++) {
             *reinterpret_cast<uint4 *>(sXh + (xr + XR * i) * kGemmLd + xc) = P.gh[i];
             *reinterpret_cast<uint4 *>(sXl + (xr + XR * i) * kGemmLd + xc) = P.gl[i];
         }
-        __syncthreads();
-        fetch(P, step + 2);
+    };
+    // the step held by LDS buffer `buf` into the accumulators
+    auto multiply = [&](int buf) {
+        const uint16_t *sXh = sXh_[buf], *sXl = sXl_[buf], *sW = sW_[buf];
 #pragma unroll
         for (int b = 0; b < kGemmK / 32; b++) {          // the two quant blocks of the step
             lv_f16v blk[MT][2];
@@ -245,18 +248,57 @@ __global__ __launch_bounds__(NWV * 64) void gemm_kernel(GemmArgs a)
             // times the block's scale: a lane's sixteen results of a tile belong to one weight row
 #pragma unroll
             for (int j = 0; j < 2; j++) {
-                const float d = sD[b][wn * 64 + j * 32 + (lane & 31)];
+                const float d = sD_[buf][b][wn * 64 + j * 32 + (lane & 31)];
 #pragma unroll
                 for (int i = 0; i < MT; i++)
 #pragma unroll
                     for (int r = 0; r < 16; r++) acc[i][j][r] = fmaf(blk[i][j][r], d, acc[i][j][r]);
             }
         }
-        __syncthreads();
     };
-    for (uint32_t step = 0; step < steps2; step += 2) {
-        one_step(pre[0], step);
-        one_step(pre[1], step + 1);
+    if constexpr (!DB) {
+        // one buffer: unpack, barrier, multiply, barrier; two register sets, the loads of step s + 2 in flight
+        fetch(pre[1], 1);
+        auto one_step = [&](Staged &P, uint32_t step) {
+            stage(P, 0);
+            __syncthreads();
+            fetch(P, step + 2);
+            multiply(0);
+            __syncthreads();
+        };
+        for (uint32_t step = 0; step < steps2; step += 2) {
+            one_step(pre[0], step);
+            one_step(pre[1], step + 1);
+        }
+    } else {
+        // two buffers, one barrier per step: step s + 1 is unpacked into one buffer while step s is multiplied out of
+        // the other, so a wave's unpacking sits between its MFMAs; three register sets, the loads of steps s + 2 and
+        // s + 3 in flight
+        fetch(pre[1], 1);
+        fetch(pre[2], 2);
+        stage(pre[0], 0);
+        __syncthreads();
+        // mine: the set that held step s (in LDS since the iteration before), reloaded with step s + 3;
+        // next: the set holding step s + 1
+        auto iteration = [&](uint32_t s, Staged &mine, const Staged &next) {
+            fetch(mine, s + 3);
+            stage(next, (s + 1) & 1);
+            multiply(s & 1);
+            __syncthreads();
+        };
+        for (uint32_t s = 0; s < steps; s += 6) {
+            iteration(s, pre[0], pre[1]);
+            if (s + 1 >= steps) break;
+            iteration(s + 1, pre[1], pre[2]);
+            if (s + 2 >= steps) break;
+            iteration(s + 2, pre[2], pre[0]);
+            if (s + 3 >= steps) break;
+            iteration(s + 3, pre[0], pre[1]);
+            if (s + 4 >= steps) break;
+            iteration(s + 4, pre[1], pre[2]);
+            if (s + 5 >= steps) break;
+            iteration(s + 5, pre[2], pre[0]);
+        }
     }
 
     // D[i][j]: i = token within the 32-tile, j = weight row; lane l holds j = l%32 and, in register r,
