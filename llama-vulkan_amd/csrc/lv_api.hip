@@ -708,19 +708,22 @@ static int launch_gemm(hipStream_t st, float *out, uint32_t ldo, const lv_matrix
     return launch_gemm_presplit(st, out, ldo, w, n, xh, xl, accumulate);
 }
 
-// the same with the activations already split (one split serves wq, wk, wv or w3, w1)
-static int launch_gemm_presplit(hipStream_t st, float *out, uint32_t ldo, const lv_matrix &w, uint32_t n, const uint16_t *xh, const uint16_t *xl,
-                                bool accumulate)
+// the same with the activations already split (one split serves wq, wk, wv or w3, w1); nmat matrices of one shape,
+// type and scale plane as one launch
+static int launch_gemm_multi(hipStream_t st, float *const outs[], uint32_t ldo, const lv_matrix *const ws[], int nmat, uint32_t n,
+                             const uint16_t *xh, const uint16_t *xl, bool accumulate)
 {
+    const lv_matrix &w = *ws[0];
     const uint32_t n_pad = (n + kGemmTile - 1) / kGemmTile * kGemmTile;
     GemmArgs a{};
-    a.out = out; a.xh = xh; a.xl = xl; a.w = w.view; a.n = n; a.ldo = ldo; a.accumulate = accumulate ? 1 : 0;
+    for (int i = 0; i < nmat; i++) { a.outs[i] = outs[i]; a.ws[i] = ws[i]->view; }
+    a.xh = xh; a.xl = xl; a.n = n; a.ldo = ldo; a.accumulate = accumulate ? 1 : 0;
     // 128-row workgroups of eight waves with two LDS buffers (one workgroup per CU) unless fewer than 128 of them
     // exist: then 64-row ones of four waves, twice as many.  Measured at 512 tokens, q8_0, 5120 x 5120 / 13824 x 5120 /
     // 5120 x 13824: 103 / 216 / 263 us; with one LDS buffer 106 / 224 / 280; the 64-row form at those sizes 135 / - / 355.
     const uint32_t token_tiles = n_pad / kGemmTile;
-    const bool narrow = (uint64_t)((w.view.rows + 127) / 128) * token_tiles < 128;
-    const dim3 grid((w.view.rows + (narrow ? 63 : 127)) / (narrow ? 64 : 128), token_tiles);
+    const bool narrow = (uint64_t)((w.view.rows + 127) / 128) * token_tiles * nmat < 128;
+    const dim3 grid((w.view.rows + (narrow ? 63 : 127)) / (narrow ? 64 : 128), token_tiles, nmat);
     const bool sf32 = w.view.scales_f32 != nullptr;
     if (w.ftype == LV_Q4_0) {
         if (narrow) { if (sf32) gemm_kernel<4, 64, 4, true><<<grid, dim3(256), 0, st>>>(a); else gemm_kernel<4, 64, 4, false><<<grid, dim3(256), 0, st>>>(a); }
@@ -732,6 +735,20 @@ static int launch_gemm_presplit(hipStream_t st, float *out, uint32_t ldo, const 
     else return fail(LV_ERR_ARG, "gemm: matrix type %u", w.ftype);
     HIP_TRY(hipGetLastError());
     return LV_OK;
+}
+
+static int launch_gemm_presplit(hipStream_t st, float *out, uint32_t ldo, const lv_matrix &w, uint32_t n, const uint16_t *xh, const uint16_t *xl,
+                                bool accumulate)
+{
+    float *const outs[1] = {out};
+    const lv_matrix *const ws[1] = {&w};
+    return launch_gemm_multi(st, outs, ldo, ws, 1, n, xh, xl, accumulate);
+}
+
+// can these matrices share a launch?  (one shape, one type, one kind of scale plane)
+static bool gemm_same(const lv_matrix &a, const lv_matrix &b)
+{
+    return a.ftype == b.ftype && a.view.rows == b.view.rows && a.view.cols == b.view.cols && (a.view.scales_f32 != nullptr) == (b.view.scales_f32 != nullptr);
 }
 
 extern "C" int lv_kernel_gemm(lv_ctx *c, float *out, const lv_matrix *w, const float *x, uint32_t batch, int accumulate)
@@ -1411,12 +1428,17 @@ static int record_prefill(lv_session *s, uint32_t idx0, uint32_t n, bool with_he
         normalize_kernel<<<dim3(n), dim3(256), 0, st>>>(s->pf_xn, s->pf_x, lw.attn_norm, D);
         HIP_TRY(hipGetLastError());
         LV_TRY(launch_split(st, s->pf_xh, s->pf_xl, s->pf_xn, n, D, lw.wq.ftype));
-        LV_TRY(launch_gemm_presplit(st, s->pf_q, D, lw.wq, n, s->pf_xh, s->pf_xl, false));
-        // one split serves all three when they share a weight type (the element order depends on it)
-        if (lw.wk.ftype == lw.wq.ftype) LV_TRY(launch_gemm_presplit(st, s->pf_k, D, lw.wk, n, s->pf_xh, s->pf_xl, false));
-        else LV_TRY(launch_gemm(st, s->pf_k, D, lw.wk, s->pf_xn, n, s->pf_xh, s->pf_xl, false));
-        if (lw.wv.ftype == lw.wk.ftype) LV_TRY(launch_gemm_presplit(st, s->pf_v, D, lw.wv, n, s->pf_xh, s->pf_xl, false));
-        else LV_TRY(launch_gemm(st, s->pf_v, D, lw.wv, s->pf_xn, n, s->pf_xh, s->pf_xl, false));
+        if (gemm_same(lw.wq, lw.wk) && gemm_same(lw.wq, lw.wv)) {
+            float *const outs[3] = {s->pf_q, s->pf_k, s->pf_v};
+            const lv_matrix *const ws[3] = {&lw.wq, &lw.wk, &lw.wv};
+            LV_TRY(launch_gemm_multi(st, outs, D, ws, 3, n, s->pf_xh, s->pf_xl, false));
+        } else {
+            LV_TRY(launch_gemm_presplit(st, s->pf_q, D, lw.wq, n, s->pf_xh, s->pf_xl, false));
+            if (lw.wk.ftype == lw.wq.ftype) LV_TRY(launch_gemm_presplit(st, s->pf_k, D, lw.wk, n, s->pf_xh, s->pf_xl, false));
+            else LV_TRY(launch_gemm(st, s->pf_k, D, lw.wk, s->pf_xn, n, s->pf_xh, s->pf_xl, false));
+            if (lw.wv.ftype == lw.wk.ftype) LV_TRY(launch_gemm_presplit(st, s->pf_v, D, lw.wv, n, s->pf_xh, s->pf_xl, false));
+            else LV_TRY(launch_gemm(st, s->pf_v, D, lw.wv, s->pf_xn, n, s->pf_xh, s->pf_xl, false));
+        }
         kv_append2_kernel<<<dim3(kv_grid.x, kv_grid.y, 2), dim3(256), 0, st>>>(kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->pf_k, s->pf_v, pos_ptr, idx0, D, s->backlog);
         HIP_TRY(hipGetLastError());
         LV_TRY(launch_attention_batch(st, s->pf_vo, kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->pf_q, s->trig_abs, pos_ptr, idx0, n, s->backlog,
@@ -1425,9 +1447,15 @@ static int record_prefill(lv_session *s, uint32_t idx0, uint32_t n, bool with_he
         normalize_kernel<<<dim3(n), dim3(256), 0, st>>>(s->pf_xn, s->pf_x, lw.ffn_norm, D);
         HIP_TRY(hipGetLastError());
         LV_TRY(launch_split(st, s->pf_xh, s->pf_xl, s->pf_xn, n, D, lw.w3.ftype));
-        LV_TRY(launch_gemm_presplit(st, s->pf_g1, F, lw.w3, n, s->pf_xh, s->pf_xl, false));
-        if (lw.w1.ftype == lw.w3.ftype) LV_TRY(launch_gemm_presplit(st, s->pf_g2, F, lw.w1, n, s->pf_xh, s->pf_xl, false));
-        else LV_TRY(launch_gemm(st, s->pf_g2, F, lw.w1, s->pf_xn, n, s->pf_xh, s->pf_xl, false));
+        if (gemm_same(lw.w3, lw.w1)) {
+            float *const outs[2] = {s->pf_g1, s->pf_g2};
+            const lv_matrix *const ws[2] = {&lw.w3, &lw.w1};
+            LV_TRY(launch_gemm_multi(st, outs, F, ws, 2, n, s->pf_xh, s->pf_xl, false));
+        } else {
+            LV_TRY(launch_gemm_presplit(st, s->pf_g1, F, lw.w3, n, s->pf_xh, s->pf_xl, false));
+            if (lw.w1.ftype == lw.w3.ftype) LV_TRY(launch_gemm_presplit(st, s->pf_g2, F, lw.w1, n, s->pf_xh, s->pf_xl, false));
+            else LV_TRY(launch_gemm(st, s->pf_g2, F, lw.w1, s->pf_xn, n, s->pf_xh, s->pf_xl, false));
+        }
         const size_t count = (size_t)n * F;
         silu_mul_kernel<<<dim3((unsigned)((count + 255) / 256)), dim3(256), 0, st>>>(s->pf_g1, s->pf_g1, s->pf_g2, count);
         HIP_TRY(hipGetLastError());

@@ -62,10 +62,13 @@ __global__ void silu_mul_kernel(float *__restrict__ out, const float *__restrict
     }
 }
 
+constexpr int kGemmMaxMats = 3;
 struct GemmArgs {
-    float *out;             // [n][ldo]
+    // up to three matrices of one shape and type applied to the same activations in one launch (blockIdx.z picks the
+    // matrix): q, k and v of a layer together fill the CUs that each alone leaves idle
+    float *outs[kGemmMaxMats];  // [n][ldo] each
     const uint16_t *xh, *xl;  // [n_pad][K] fp16 halves of the activations, n_pad a multiple of 128
-    MatView w;              // rows x K
+    MatView ws[kGemmMaxMats];   // rows x K each
     uint32_t n;             // tokens
     uint32_t ldo;           // floats between output rows
     int accumulate;         // out += instead of out =
@@ -140,7 +143,9 @@ __global__ __launch_bounds__(NWV * 64) void gemm_kernel(GemmArgs a)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
     const uint32_t tok0 = blockIdx.y * TN, row0 = blockIdx.x * RM;
-    const uint32_t K = a.w.cols, nb = K / 32, steps = (K + kGemmK - 1) / kGemmK;
+    const MatView w = a.ws[blockIdx.z];
+    float *const out = a.outs[blockIdx.z];
+    const uint32_t K = w.cols, nb = K / 32, steps = (K + kGemmK - 1) / kGemmK;
 
     // this thread's share of the weights of a step: half h_w of block (2*step + b_w) of row r_w.  Every thread has one,
     // and every load below is issued by every thread at every step (addresses are clamped, results discarded where
@@ -149,7 +154,7 @@ __global__ __launch_bounds__(NWV * 64) void gemm_kernel(GemmArgs a)
     static_assert(NT == RM * 4, "two threads per (row, block)");
     const int r_w = tid >> 2, b_w = (tid >> 1) & 1, h_w = tid & 1;
     const uint32_t wrow = row0 + r_w;
-    const bool wrow_ok = wrow < a.w.rows;
+    const bool wrow_ok = wrow < w.rows;
     // this thread's 16-byte pieces of the activation tile of a step: token rows tid/8 + XR*i, halfs (tid%8)*8..+7
     const int xr = tid >> 3, xc = (tid & 7) * 8;
     constexpr int XR = NT / 8;                    // token rows covered per piece index
@@ -170,13 +175,13 @@ __global__ __launch_bounds__(NWV * 64) void gemm_kernel(GemmArgs a)
         p.wvalid = real && wrow_ok && blk < nb;
         const size_t sb = (size_t)(p.wvalid ? wrow : 0) * nb + (p.wvalid ? blk : 0);
         if constexpr (QT == 8) {
-            p.c = a.w.codes[sb * 2 + h_w];
+            p.c = w.codes[sb * 2 + h_w];
         } else {
-            const uint2 half = reinterpret_cast<const uint2 *>(a.w.codes)[sb * 2 + h_w];
+            const uint2 half = reinterpret_cast<const uint2 *>(w.codes)[sb * 2 + h_w];
             p.c = make_uint4(half.x, half.y, 0, 0);
         }
-        if constexpr (SF32) p.dbits = __float_as_uint(a.w.scales_f32[sb]);
-        else p.dbits = a.w.scales[sb];
+        if constexpr (SF32) p.dbits = __float_as_uint(w.scales_f32[sb]);
+        else p.dbits = w.scales[sb];
         const uint32_t k = sc * kGemmK + xc;
         const bool kok = real && k < K;
 #pragma unroll
@@ -311,8 +316,8 @@ __global__ __launch_bounds__(NWV * 64) void gemm_kernel(GemmArgs a)
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const uint32_t n = tok0 + (wm * MT + ti) * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
-                if (n < a.n && m < a.w.rows) {
-                    float *dst = a.out + (size_t)n * a.ldo + m;
+                if (n < a.n && m < w.rows) {
+                    float *dst = out + (size_t)n * a.ldo + m;
                     *dst = a.accumulate ? *dst + acc[ti][tj][r] : acc[ti][tj][r];
                 }
             }
