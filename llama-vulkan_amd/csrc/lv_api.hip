@@ -708,22 +708,15 @@ static int launch_gemm(hipStream_t st, float *out, uint32_t ldo, const lv_matrix
     return launch_gemm_presplit(st, out, ldo, w, n, xh, xl, accumulate);
 }
 
-// the same with the activations already split (one split serves wq, wk, wv or w3, w1); nmat matrices of one shape,
-// type and scale plane as one launch
-static int launch_gemm_multi(hipStream_t st, float *const outs[], uint32_t ldo, const lv_matrix *const ws[], int nmat, uint32_t n,
-                             const uint16_t *xh, const uint16_t *xl, bool accumulate)
+// launches gemm_kernel for args whose ws[0..nz-1] are set: nz matrices, or nz K slices of one
+static int dispatch_gemm(hipStream_t st, const GemmArgs &a, const lv_matrix &w, uint32_t nz)
 {
-    const lv_matrix &w = *ws[0];
-    const uint32_t n_pad = (n + kGemmTile - 1) / kGemmTile * kGemmTile;
-    GemmArgs a{};
-    for (int i = 0; i < nmat; i++) { a.outs[i] = outs[i]; a.ws[i] = ws[i]->view; }
-    a.xh = xh; a.xl = xl; a.n = n; a.ldo = ldo; a.accumulate = accumulate ? 1 : 0;
     // 128-row workgroups of eight waves with two LDS buffers (one workgroup per CU) unless fewer than 128 of them
     // exist: then 64-row ones of four waves, twice as many.  Measured at 512 tokens, q8_0, 5120 x 5120 / 13824 x 5120 /
     // 5120 x 13824: 103 / 216 / 263 us; with one LDS buffer 106 / 224 / 280; the 64-row form at those sizes 135 / - / 355.
-    const uint32_t token_tiles = n_pad / kGemmTile;
-    const bool narrow = (uint64_t)((w.view.rows + 127) / 128) * token_tiles * nmat < 128;
-    const dim3 grid((w.view.rows + (narrow ? 63 : 127)) / (narrow ? 64 : 128), token_tiles, nmat);
+    const uint32_t token_tiles = (a.n + kGemmTile - 1) / kGemmTile;
+    const bool narrow = (uint64_t)((w.view.rows + 127) / 128) * token_tiles * nz < 128;
+    const dim3 grid((w.view.rows + (narrow ? 63 : 127)) / (narrow ? 64 : 128), token_tiles, nz);
     const bool sf32 = w.view.scales_f32 != nullptr;
     if (w.ftype == LV_Q4_0) {
         if (narrow) { if (sf32) gemm_kernel<4, 64, 4, true><<<grid, dim3(256), 0, st>>>(a); else gemm_kernel<4, 64, 4, false><<<grid, dim3(256), 0, st>>>(a); }
@@ -733,6 +726,60 @@ static int launch_gemm_multi(hipStream_t st, float *const outs[], uint32_t ldo, 
         else { if (sf32) gemm_kernel<8, 128, 8, true, true><<<grid, dim3(512), 0, st>>>(a); else gemm_kernel<8, 128, 8, false, true><<<grid, dim3(512), 0, st>>>(a); }
     }
     else return fail(LV_ERR_ARG, "gemm: matrix type %u", w.ftype);
+    HIP_TRY(hipGetLastError());
+    return LV_OK;
+}
+
+// the same with the activations already split (one split serves wq, wk, wv or w3, w1); nmat matrices of one shape,
+// type and scale plane as one launch
+static int launch_gemm_multi(hipStream_t st, float *const outs[], uint32_t ldo, const lv_matrix *const ws[], int nmat, uint32_t n,
+                             const uint16_t *xh, const uint16_t *xl, bool accumulate)
+{
+    GemmArgs a{};
+    for (int i = 0; i < nmat; i++) { a.outs[i] = outs[i]; a.ws[i] = ws[i]->view; }
+    a.xh = xh; a.xl = xl; a.n = n; a.ldo = ldo; a.accumulate = accumulate ? 1 : 0;
+    return dispatch_gemm(st, a, *ws[0], (uint32_t)nmat);
+}
+
+// Into how many K slices to cut a product whose 128 x 128 output tiles alone number `tiles`: the count (1..3) that
+// leaves the fewest CU-rounds idle, the smaller count unless a larger one fills them clearly better.  A slice keeps
+// at least 16 K steps.
+static uint32_t gemm_k_slices(uint32_t tiles, uint32_t k_steps)
+{
+    constexpr uint32_t cus = 256;
+    uint32_t best = 1;
+    double best_fill = 0;
+    for (uint32_t s = 1; s <= (uint32_t)kGemmMaxMats; s++) {
+        if (s > 1 && k_steps / s < 16) break;
+        const uint32_t wgs = tiles * s, rounds = (wgs + cus - 1) / cus;
+        const double fill = (double)wgs / ((double)rounds * cus);
+        if (fill > best_fill + 0.05) { best_fill = fill; best = s; }
+    }
+    return best;
+}
+
+// one matrix, activations already split, K cut in slices when that fills the CUs better: the slices go to parts[]
+// ([n][rows] floats each, scratch of the caller) and gemm_reduce_kernel adds them to out in a fixed order
+static int launch_gemm_sliced(hipStream_t st, float *out, uint32_t ldo, const lv_matrix &w, uint32_t n, const uint16_t *xh, const uint16_t *xl,
+                              bool accumulate, float *const parts[kGemmMaxMats])
+{
+    const uint32_t rows = w.view.rows, k_steps = (w.view.cols + kGemmK - 1) / kGemmK;
+    const uint32_t token_tiles = (n + kGemmTile - 1) / kGemmTile;
+    const uint32_t slices = (rows % 4 || ldo % 4) ? 1 : gemm_k_slices((rows + 127) / 128 * token_tiles, k_steps);
+    GemmArgs a{};
+    a.xh = xh; a.xl = xl; a.n = n;
+    if (slices == 1) {
+        a.outs[0] = out; a.ws[0] = w.view; a.ldo = ldo; a.accumulate = accumulate ? 1 : 0;
+        return dispatch_gemm(st, a, w, 1);
+    }
+    a.slice_steps = (k_steps + slices - 1) / slices;
+    const uint32_t used = (k_steps + a.slice_steps - 1) / a.slice_steps;      // every slice launched has a step
+    GemmReduceArgs r{};
+    for (uint32_t i = 0; i < used; i++) { a.outs[i] = parts[i]; a.ws[i] = w.view; r.parts[i] = parts[i]; }
+    a.ldo = rows;
+    LV_TRY(dispatch_gemm(st, a, w, used));
+    r.out = out; r.nparts = used; r.rows = rows; r.ldo = ldo; r.n = n; r.accumulate = accumulate ? 1 : 0;
+    gemm_reduce_kernel<<<dim3((rows / 4 + 255) / 256, n), dim3(256), 0, st>>>(r);
     HIP_TRY(hipGetLastError());
     return LV_OK;
 }
@@ -1443,7 +1490,11 @@ static int record_prefill(lv_session *s, uint32_t idx0, uint32_t n, bool with_he
         HIP_TRY(hipGetLastError());
         LV_TRY(launch_attention_batch(st, s->pf_vo, kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->pf_q, s->trig_abs, pos_ptr, idx0, n, s->backlog,
                                       hp.heads, hp.rot));
-        LV_TRY(launch_gemm(st, s->pf_x, D, lw.wo, s->pf_vo, n, s->pf_xh, s->pf_xl, true));
+        // q, k and v have been consumed: their buffers take the K slices of the output projection, and of the down
+        // projection further on
+        float *const parts[kGemmMaxMats] = {s->pf_q, s->pf_k, s->pf_v};
+        LV_TRY(launch_split(st, s->pf_xh, s->pf_xl, s->pf_vo, n, D, lw.wo.ftype));
+        LV_TRY(launch_gemm_sliced(st, s->pf_x, D, lw.wo, n, s->pf_xh, s->pf_xl, true, parts));
         normalize_kernel<<<dim3(n), dim3(256), 0, st>>>(s->pf_xn, s->pf_x, lw.ffn_norm, D);
         HIP_TRY(hipGetLastError());
         LV_TRY(launch_split(st, s->pf_xh, s->pf_xl, s->pf_xn, n, D, lw.w3.ftype));
@@ -1459,7 +1510,8 @@ static int record_prefill(lv_session *s, uint32_t idx0, uint32_t n, bool with_he
         const size_t count = (size_t)n * F;
         silu_mul_kernel<<<dim3((unsigned)((count + 255) / 256)), dim3(256), 0, st>>>(s->pf_g1, s->pf_g1, s->pf_g2, count);
         HIP_TRY(hipGetLastError());
-        LV_TRY(launch_gemm(st, s->pf_x, D, lw.w2, s->pf_g1, n, s->pf_xh, s->pf_xl, true));
+        LV_TRY(launch_split(st, s->pf_xh, s->pf_xl, s->pf_g1, n, F, lw.w2.ftype));
+        LV_TRY(launch_gemm_sliced(st, s->pf_x, D, lw.w2, n, s->pf_xh, s->pf_xl, true, parts));
     }
     if (with_head) {
         // only the last row's logits are ever read (llava_session.cpp:131-139)

@@ -72,7 +72,36 @@ struct GemmArgs {
     uint32_t n;             // tokens
     uint32_t ldo;           // floats between output rows
     int accumulate;         // out += instead of out =
+    // 0: blockIdx.z picks the matrix.  Otherwise the launch splits K: ws[] all name one matrix, slice z multiplies the
+    // K steps z*slice_steps .. (z+1)*slice_steps-1 into outs[z], and gemm_reduce_kernel adds the slices up (a matrix
+    // with few rows and a long K, like the down projection, fills the CUs that way)
+    uint32_t slice_steps;
 };
+
+// out[n][ldo] (+)= p[0] + p[1] (+ p[2]), the K slices of one product, each [n][rows]; always summed in this order
+struct GemmReduceArgs {
+    float *out;
+    const float *parts[kGemmMaxMats];
+    uint32_t nparts, rows, ldo, n;
+    int accumulate;
+};
+__global__ void gemm_reduce_kernel(GemmReduceArgs a)
+{
+    const uint32_t row = blockIdx.y, c = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    if (c >= a.rows) return;
+    const size_t src = (size_t)row * a.rows + c;
+    float4 s = *reinterpret_cast<const float4 *>(a.parts[0] + src);
+    for (uint32_t i = 1; i < a.nparts; i++) {
+        const float4 v = *reinterpret_cast<const float4 *>(a.parts[i] + src);
+        s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    }
+    float4 *dst = reinterpret_cast<float4 *>(a.out + (size_t)row * a.ldo + c);
+    if (a.accumulate) {
+        const float4 o = *dst;
+        s.x += o.x; s.y += o.y; s.z += o.z; s.w += o.w;
+    }
+    *dst = s;
+}
 
 typedef _Float16 lv_h2 __attribute__((ext_vector_type(2)));
 
@@ -145,7 +174,10 @@ __global__ __launch_bounds__(NWV * 64) void gemm_kernel(GemmArgs a)
     const uint32_t tok0 = blockIdx.y * TN, row0 = blockIdx.x * RM;
     const MatView w = a.ws[blockIdx.z];
     float *const out = a.outs[blockIdx.z];
-    const uint32_t K = w.cols, nb = K / 32, steps = (K + kGemmK - 1) / kGemmK;
+    const uint32_t K = w.cols, nb = K / 32, all_steps = (K + kGemmK - 1) / kGemmK;
+    // this workgroup's K steps: step0 .. step0 + steps - 1 (the host gives every slice at least one)
+    const uint32_t step0 = a.slice_steps ? blockIdx.z * a.slice_steps : 0;
+    const uint32_t steps = a.slice_steps ? min(a.slice_steps, all_steps - step0) : all_steps;
 
     // this thread's share of the weights of a step: half h_w of block (2*step + b_w) of row r_w.  Every thread has one,
     // and every load below is issued by every thread at every step (addresses are clamped, results discarded where
@@ -170,7 +202,7 @@ __global__ __launch_bounds__(NWV * 64) void gemm_kernel(GemmArgs a)
     } pre[DB ? 3 : 2];
     auto fetch = [&](Staged &p, uint32_t step) {
         const bool real = step < steps;
-        const uint32_t sc = real ? step : steps - 1;
+        const uint32_t sc = step0 + (real ? step : steps - 1);
         const uint32_t blk = 2 * sc + b_w;
         p.wvalid = real && wrow_ok && blk < nb;
         const size_t sb = (size_t)(p.wvalid ? wrow : 0) * nb + (p.wvalid ? blk : 0);
