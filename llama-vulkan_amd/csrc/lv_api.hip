@@ -711,18 +711,27 @@ static int launch_gemm(hipStream_t st, float *out, uint32_t ldo, const lv_matrix
 // launches gemm_kernel for args whose ws[0..nz-1] are set: nz matrices, or nz K slices of one
 static int dispatch_gemm(hipStream_t st, const GemmArgs &a, const lv_matrix &w, uint32_t nz)
 {
-    // 128-row workgroups of eight waves with two LDS buffers (one workgroup per CU) unless fewer than 128 of them
-    // exist: then 64-row ones of four waves, twice as many.  Measured at 512 tokens, q8_0, 5120 x 5120 / 13824 x 5120 /
-    // 5120 x 13824: 103 / 216 / 263 us; with one LDS buffer 106 / 224 / 280; the 64-row form at those sizes 135 / - / 355.
+    // Three forms.  128 tokens x 128 rows with eight waves and two LDS buffers (one workgroup per CU) is the base.
+    // 128 x 256 (every wave 64 x 64: a quarter fewer operand reads from LDS per MFMA) does the same work about 8 %
+    // faster per CU, so it is taken when its coarser rounds of 256 workgroups do not cost more than that.  Fewer than
+    // 128 workgroups of the base form: 64-row ones of four waves, twice as many.  Measured at 512 tokens, q8_0,
+    // 5120 x 5120 / 13824 x 5120 / 5120 x 13824: base 103 / 216 / 263 us; with one LDS buffer 106 / 224 / 280; the
+    // 64-row form at those sizes 135 / - / 355.
     const uint32_t token_tiles = (a.n + kGemmTile - 1) / kGemmTile;
-    const bool narrow = (uint64_t)((w.view.rows + 127) / 128) * token_tiles * nz < 128;
-    const dim3 grid((w.view.rows + (narrow ? 63 : 127)) / (narrow ? 64 : 128), token_tiles, nz);
+    constexpr uint32_t cus = 256;
+    const uint32_t t128 = (w.view.rows + 127) / 128 * token_tiles * nz, t256 = (w.view.rows + 255) / 256 * token_tiles * nz;
+    const bool narrow = t128 < 128;
+    // (q8_0 only: the q4_0 instantiation of the 256-row form spills registers and is 4 % slower than the base form)
+    const bool wide = !narrow && w.ftype == LV_Q8_0 && (double)((t256 + cus - 1) / cus) * 1.84 < (double)((t128 + cus - 1) / cus);
+    const uint32_t rm = narrow ? 64 : wide ? 256 : 128;
+    const dim3 grid((w.view.rows + rm - 1) / rm, token_tiles, nz);
     const bool sf32 = w.view.scales_f32 != nullptr;
     if (w.ftype == LV_Q4_0) {
         if (narrow) { if (sf32) gemm_kernel<4, 64, 4, true><<<grid, dim3(256), 0, st>>>(a); else gemm_kernel<4, 64, 4, false><<<grid, dim3(256), 0, st>>>(a); }
         else { if (sf32) gemm_kernel<4, 128, 8, true, true><<<grid, dim3(512), 0, st>>>(a); else gemm_kernel<4, 128, 8, false, true><<<grid, dim3(512), 0, st>>>(a); }
     } else if (w.ftype == LV_Q8_0) {
         if (narrow) { if (sf32) gemm_kernel<8, 64, 4, true><<<grid, dim3(256), 0, st>>>(a); else gemm_kernel<8, 64, 4, false><<<grid, dim3(256), 0, st>>>(a); }
+        else if (wide) { if (sf32) gemm_kernel<8, 256, 8, true, true><<<grid, dim3(512), 0, st>>>(a); else gemm_kernel<8, 256, 8, false, true><<<grid, dim3(512), 0, st>>>(a); }
         else { if (sf32) gemm_kernel<8, 128, 8, true, true><<<grid, dim3(512), 0, st>>>(a); else gemm_kernel<8, 128, 8, false, true><<<grid, dim3(512), 0, st>>>(a); }
     }
     else return fail(LV_ERR_ARG, "gemm: matrix type %u", w.ftype);
@@ -758,14 +767,21 @@ static uint32_t gemm_k_slices(uint32_t tiles, uint32_t k_steps)
     return best;
 }
 
+// the slice count launch_gemm_sliced uses for n tokens of w into rows of ldo floats (the reduce works on float4)
+static uint32_t gemm_slices_for(const lv_matrix &w, uint32_t n, uint32_t ldo)
+{
+    const uint32_t rows = w.view.rows, k_steps = (w.view.cols + kGemmK - 1) / kGemmK;
+    const uint32_t token_tiles = (n + kGemmTile - 1) / kGemmTile;
+    return (rows % 4 || ldo % 4) ? 1 : gemm_k_slices((rows + 127) / 128 * token_tiles, k_steps);
+}
+
 // one matrix, activations already split, K cut in slices when that fills the CUs better: the slices go to parts[]
 // ([n][rows] floats each, scratch of the caller) and gemm_reduce_kernel adds them to out in a fixed order
 static int launch_gemm_sliced(hipStream_t st, float *out, uint32_t ldo, const lv_matrix &w, uint32_t n, const uint16_t *xh, const uint16_t *xl,
                               bool accumulate, float *const parts[kGemmMaxMats])
 {
     const uint32_t rows = w.view.rows, k_steps = (w.view.cols + kGemmK - 1) / kGemmK;
-    const uint32_t token_tiles = (n + kGemmTile - 1) / kGemmTile;
-    const uint32_t slices = (rows % 4 || ldo % 4) ? 1 : gemm_k_slices((rows + 127) / 128 * token_tiles, k_steps);
+    const uint32_t slices = parts ? gemm_slices_for(w, n, ldo) : 1;
     GemmArgs a{};
     a.xh = xh; a.xl = xl; a.n = n;
     if (slices == 1) {
@@ -805,13 +821,20 @@ extern "C" int lv_kernel_gemm(lv_ctx *c, float *out, const lv_matrix *w, const f
     if (batch > kMaxStepTokens) return fail(LV_ERR_RANGE, "lv_kernel_gemm: batch %u (limit %u)", batch, kMaxStepTokens);
     HIP_TRY(hipSetDevice(c->device));
     const size_t n_pad = (batch + kGemmTile - 1) / kGemmTile * kGemmTile, halfs = n_pad * w->view.cols;
-    uint16_t *xh = nullptr, *xl = nullptr;
-    HIP_TRY(hipMalloc(reinterpret_cast<void **>(&xh), halfs * 2));
-    hipError_t e = hipMalloc(reinterpret_cast<void **>(&xl), halfs * 2);
-    int rc = e == hipSuccess ? launch_gemm(c->stream, out, w->view.rows, *w, x, batch, xh, xl, accumulate != 0) : fail(LV_ERR_OOM, "lv_kernel_gemm: workspace");
+    if (w->view.cols % 32) return fail(LV_ERR_ARG, "gemm: %u columns", w->view.cols);
+    // workspace: the two fp16 halves of the activations and, where K is cut in slices, their partial results
+    const uint32_t slices = gemm_slices_for(*w, batch, w->view.rows);
+    const size_t part = slices > 1 ? (size_t)batch * w->view.rows : 0;
+    uint16_t *xh = nullptr;
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&xh), halfs * 4 + part * slices * 4);
+    if (e != hipSuccess) return fail(LV_ERR_OOM, "lv_kernel_gemm: workspace");
+    uint16_t *xl = xh + halfs;
+    float *p0 = reinterpret_cast<float *>(xl + halfs);
+    float *const parts[kGemmMaxMats] = {p0, p0 + part, p0 + 2 * part};
+    int rc = launch_split(c->stream, xh, xl, x, batch, w->view.cols, w->ftype);
+    if (rc == LV_OK) rc = launch_gemm_sliced(c->stream, out, w->view.rows, *w, batch, xh, xl, accumulate != 0, slices > 1 ? parts : nullptr);
     (void)hipStreamSynchronize(c->stream);
     (void)hipFree(xh);
-    (void)hipFree(xl);
     return rc;
 }
 

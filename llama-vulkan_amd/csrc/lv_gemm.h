@@ -122,8 +122,8 @@ __host__ __device__ constexpr int gemm_k_position(int e)
 // 16*half .. 16*half+15 of gemm_k_position order) -> 16 halfs at w, as the integers they are (q4_0: q - 8, q8_0: q):
 // 1024 + u has the fp16 bit pattern 0x6400 | u, and subtracting 1024 + offset is exact.  A block outside the matrix
 // is given the scale 0 by the caller, which removes it from the sum whatever codes were unpacked for it.
-template <int QT>
-__device__ __forceinline__ void gemm_codes_half(uint16_t *w, const uint4 &c)
+template <int QT, typename CW>
+__device__ __forceinline__ void gemm_codes_half(uint16_t *w, const CW &c)
 {
     uint32_t ph[8];
     auto emit = [&](int slot, uint32_t packed_codes, _Float16 bias) {
@@ -141,7 +141,7 @@ __device__ __forceinline__ void gemm_codes_half(uint16_t *w, const uint4 &c)
 #pragma unroll
             for (int j = 0; j < 4; j++) emit(4 * i + j, ((q[i] >> (4 * j)) & 0x000f000fu) | 0x64006400u, (_Float16)1032.f);
     } else {
-        const uint32_t q[4] = {c.x, c.y, c.z, c.w};
+        const uint32_t q[4] = {c.x, c.y, c.z, c.w};      // CW = uint4
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const uint32_t u = q[i] ^ 0x80808080u;   // int8 -> biased unsigned
@@ -183,10 +183,9 @@ __global__ __launch_bounds__(NWV * 64) void gemm_kernel(GemmArgs a)
     // and every load below is issued by every thread at every step (addresses are clamped, results discarded where
     // there is nothing to load): the compiler can then count the loads in flight exactly and wait for the oldest set
     // only, which a load under a condition would force it to give up.
-    static_assert(NT == RM * 4, "two threads per (row, block)");
+    static_assert(RM * 4 % NT == 0, "two threads per (row, block)");
+    constexpr int WP = RM * 4 / NT;               // (row, block, half) pieces per thread: rows r_w + (NT/4)*i
     const int r_w = tid >> 2, b_w = (tid >> 1) & 1, h_w = tid & 1;
-    const uint32_t wrow = row0 + r_w;
-    const bool wrow_ok = wrow < w.rows;
     // this thread's 16-byte pieces of the activation tile of a step: token rows tid/8 + XR*i, halfs (tid%8)*8..+7
     const int xr = tid >> 3, xc = (tid & 7) * 8;
     constexpr int XR = NT / 8;                    // token rows covered per piece index
@@ -194,26 +193,30 @@ __global__ __launch_bounds__(NWV * 64) void gemm_kernel(GemmArgs a)
 
     // two register sets: the loads of step s + 2 are in flight while step s is multiplied (one step of MFMAs is
     // shorter than a trip to memory)
+    using CodeWords = typename std::conditional<QT == 8, uint4, uint2>::type;     // 16 codes
     struct Staged {
-        uint4 c;
-        uint32_t dbits;     // raw scale word
-        bool wvalid;
+        CodeWords c[WP];
+        uint32_t dbits[WP]; // raw scale word
+        bool wvalid[WP];
         uint4 gh[XP], gl[XP];
     } pre[DB ? 3 : 2];
     auto fetch = [&](Staged &p, uint32_t step) {
         const bool real = step < steps;
         const uint32_t sc = step0 + (real ? step : steps - 1);
         const uint32_t blk = 2 * sc + b_w;
-        p.wvalid = real && wrow_ok && blk < nb;
-        const size_t sb = (size_t)(p.wvalid ? wrow : 0) * nb + (p.wvalid ? blk : 0);
-        if constexpr (QT == 8) {
-            p.c = w.codes[sb * 2 + h_w];
-        } else {
-            const uint2 half = reinterpret_cast<const uint2 *>(w.codes)[sb * 2 + h_w];
-            p.c = make_uint4(half.x, half.y, 0, 0);
+#pragma unroll
+        for (int i = 0; i < WP; i++) {
+            const uint32_t wrow = row0 + r_w + (NT / 4) * i;
+            p.wvalid[i] = real && wrow < w.rows && blk < nb;
+            const size_t sb = (size_t)(p.wvalid[i] ? wrow : 0) * nb + (p.wvalid[i] ? blk : 0);
+            if constexpr (QT == 8) {
+                p.c[i] = w.codes[sb * 2 + h_w];
+            } else {
+                p.c[i] = reinterpret_cast<const uint2 *>(w.codes)[sb * 2 + h_w];
+            }
+            if constexpr (SF32) p.dbits[i] = __float_as_uint(w.scales_f32[sb]);
+            else p.dbits[i] = w.scales[sb];
         }
-        if constexpr (SF32) p.dbits = __float_as_uint(w.scales_f32[sb]);
-        else p.dbits = w.scales[sb];
         const uint32_t k = sc * kGemmK + xc;
         const bool kok = real && k < K;
 #pragma unroll
@@ -237,8 +240,12 @@ __global__ __launch_bounds__(NWV * 64) void gemm_kernel(GemmArgs a)
     // registers -> LDS buffer `buf`
     auto stage = [&](const Staged &P, int buf) {
         uint16_t *sXh = sXh_[buf], *sXl = sXl_[buf], *sW = sW_[buf];
-        gemm_codes_half<QT>(sW + r_w * kGemmLd + b_w * 32 + h_w * 16, P.c);
-        if (h_w == 0) sD_[buf][b_w][r_w] = !P.wvalid ? 0.f : SF32 ? __uint_as_float(P.dbits) : half_bits_to_float((uint16_t)P.dbits);
+#pragma unroll
+        for (int i = 0; i < WP; i++) {
+            const int r = r_w + (NT / 4) * i;
+            gemm_codes_half<QT>(sW + r * kGemmLd + b_w * 32 + h_w * 16, P.c[i]);
+            if (h_w == 0) sD_[buf][b_w][r] = !P.wvalid[i] ? 0.f : SF32 ? __uint_as_float(P.dbits[i]) : half_bits_to_float((uint16_t)P.dbits[i]);
+        }
 #pragma unroll
         for (int i = 0; i < XP; i++) {
             *reinterpret_cast<uint4 *>(sXh + (xr + XR * i) * kGemmLd + xc) = P.gh[i];

@@ -5,6 +5,7 @@
     python llama-vulkan_amd/measure.py decode-q8     7B q8_0, cache positions 1920..2047 (128 greedy steps)
     python llama-vulkan_amd/measure.py decode-13b    13B q4_0, 32-token prompt + 256 greedy steps
     python llama-vulkan_amd/measure.py prefill-13b   13B q8_0, 512-token prompt evaluated in one lv_step_begin
+    python llama-vulkan_amd/measure.py prefill-7b    7B q4_0, the same
     python llama-vulkan_amd/measure.py gemm          isolated 512-token GEMMs at the 13B shapes, q8_0 (for kernel traces and counters)
     python llama-vulkan_amd/measure.py copy          1 GiB device-to-device copy: achievable bandwidth, counter calibration
     python llama-vulkan_amd/measure.py all
@@ -128,9 +129,9 @@ def decode_case(ctx, name, preset, wtype, seed, backlog, first, steps):
     model.close()
 
 
-def prefill_case(ctx):
-    shape, wtype = SHAPES["13b"], lva.LV_Q8_0
-    path = model_file("13b", wtype, 3)
+def prefill_case(ctx, case, name, wtype):
+    shape = SHAPES[name]
+    path = model_file(name, wtype, 3)
     model = lva.Model(ctx, path)
     s = lva.Session(model, 512)
     prompt = lva.synth_tokens(512, 3, shape["vocab"], seed=3)
@@ -140,8 +141,9 @@ def prefill_case(ctx):
     s.begin(prompt, 0)
     ms = s.timer_stop()
     D, F, V, L = shape["dim"], shape["ff"], shape["vocab"], shape["layers"]
-    flops = 2.0 * 512 * (L * (4 * D * D + 3 * D * F) + V * D)
-    emit(case="prefill-13b", model="13b", wtype="q8_0", tokens=512, ms=round(ms, 2), tok_s=round(512 / ms * 1e3, 1), TFLOPs=round(flops / ms / 1e9, 2))
+    flops = 2.0 * 512 * L * (4 * D * D + 3 * D * F) + 2.0 * V * D      # the output matrix sees the last row only
+    emit(case=case, model=name, wtype="q4_0" if wtype == lva.LV_Q4_0 else "q8_0", tokens=512, ms=round(ms, 2),
+         tok_s=round(512 / ms * 1e3, 1), TFLOPs=round(flops / ms / 1e9, 2))
     s.close()
     model.close()
 
@@ -181,7 +183,9 @@ def main():
     if which in ("decode-13b", "all"):
         decode_case(ctx, "decode-13b", "13b", lva.LV_Q4_0, 2, 512, 32, 256)
     if which in ("prefill-13b", "all"):
-        prefill_case(ctx)
+        prefill_case(ctx, "prefill-13b", "13b", lva.LV_Q8_0)
+    if which in ("prefill-7b", "all"):
+        prefill_case(ctx, "prefill-7b", "7b", lva.LV_Q4_0)
 
 
 if __name__ == "__main__":

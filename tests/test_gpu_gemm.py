@@ -18,7 +18,9 @@ def _abs_dot_bound(orc, blocks, ftype, rows, cols, x):
     (256, 4096, 130, False),     # a second, almost empty token tile
     (704, 256, 17, True),        # rows not a multiple of the tile, residual add
     (96, 1376, 200, False),      # K = 43 blocks: a half K step at the end, fewer rows than a tile
-    (4096, 4096, 512, True),     # the 7B attention shape at a 512-token prompt batch
+    (4096, 4096, 512, True),     # the 7B attention shape at a 512-token prompt batch (K cut in two slices)
+    (5120, 3168, 512, True),     # 160 tiles for 256 CUs: K cut in three slices of 17, 17 and 15.5 steps, then reduced
+    (8264, 160, 400, True),      # more 128-row tiles than CUs: the 256-row form (q8_0), ragged in rows, K and tokens
 ])
 def test_gemm_matches_oracle(lva, orc, ctx, ftype_name, rows, cols, batch, accumulate):
     ftype = lva.LV_Q4_0 if ftype_name == "q4_0" else lva.LV_Q8_0
