@@ -16,7 +16,8 @@
 //
 // One workgroup = one head x 64 query rows, four waves = 2 query tiles x 2 position tiles of 32; the cache is walked
 // in tiles of 64 positions staged through LDS (K rotated, as fp32, x and y components apart; V transposed, fp16, even
-// and odd positions apart: both so that an MFMA operand is a run of consecutive LDS words per lane).
+// and odd positions apart: both so that an MFMA operand is a run of consecutive LDS words per lane; the 8-byte units
+// of a V row are permuted so that the stores of the staging spread over the banks).
 #pragma once
 
 #include "lv_kernels.h"
@@ -45,7 +46,9 @@ struct AttnBatchLds {
     static constexpr int VP = kAttnBatchK / 2 + 8;   // row stride of vt in halfs
     static constexpr int PP = 16 + 4;        // row stride of the probability tiles in floats
     float kx[kAttnBatchK][KP], ky[kAttnBatchK][KP];   // rotated K: components 2i and 2i+1 of the pairs
-    uint16_t vt[2][R][VP];                   // V transposed: [position parity][dim][position / 2]
+    uint16_t vt[2][R][VP];                   // V transposed: [position parity][dim][position / 2], 8-byte units permuted:
+    // unit u (positions / 2 = 4u .. 4u+3) of the row of a dim in group c8 = dim / 8 is stored at unit u ^ (c8 & 7)
+    __device__ static constexpr int vt_unit(int u, int c8) { return u ^ (c8 & 7); }
     float ps[4][2][32][PP];                  // per wave: exp(score) [position parity][query row][position / 2]
     float den[2][2][32];                     // [position tile][query tile][query row]
 };
@@ -58,7 +61,8 @@ __global__ __launch_bounds__(256) void attention_batch_kernel(AttnBatchArgs a)
     constexpr int DT = R / 32;    // 32-wide tiles of the head dimension
     using L = AttnBatchLds<R>;
     __shared__ __attribute__((aligned(16))) L l;
-    const uint32_t h = blockIdx.x, z0 = blockIdx.y * TQ;
+    // the last query tile walks the most cache tiles: it is dispatched first, so the short ones fill the tail
+    const uint32_t h = blockIdx.x, z0 = (gridDim.y - 1 - blockIdx.y) * TQ;
     const uint32_t H = a.heads, D = H * R;
     const uint32_t pos0 = (a.pos_ptr ? *a.pos_ptr : 0u) + a.pos_add;  // cache position of batch row 0
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
@@ -99,29 +103,46 @@ __global__ __launch_bounds__(256) void attention_batch_kernel(AttnBatchArgs a)
     for (uint32_t k0 = 0; k0 <= last_pos; k0 += TK) {
         __syncthreads();  // the previous tile is consumed
         // ---- stage K (rotated, fp32) and V (transposed, fp16) of this tile ------------------------------------------
-        for (int i = t; i < TK * R / 8; i += 256) {
-            const int row = i / (R / 8), c8 = i % (R / 8);
-            const uint32_t p = min(k0 + row, a.backlog - 1);
-            const uint4 kraw = *reinterpret_cast<const uint4 *>(a.kcache + (size_t)p * D + (size_t)h * R + c8 * 8);
-            const uint4 vraw = *reinterpret_cast<const uint4 *>(a.vcache + (size_t)p * D + (size_t)h * R + c8 * 8);
-            const float4 cs0 = *reinterpret_cast<const float4 *>(a.trig_abs + (size_t)p * (R / 2) + c8 * 4);
-            const float4 cs1 = *reinterpret_cast<const float4 *>(a.trig_abs + (size_t)p * (R / 2) + c8 * 4 + 2);
-            const uint32_t kw[4] = {kraw.x, kraw.y, kraw.z, kraw.w};
-            const float c[4] = {cs0.x, cs0.z, cs1.x, cs1.z}, s[4] = {cs0.y, cs0.w, cs1.y, cs1.w};
-            float xr[4], yr[4];
+        // a thread takes eight dims (c8) of four positions of one parity, base + par + 2m: their V halfs are neighbours
+        // in the transposed tile and go out as one 8-byte store per dim.  The 8-byte units of a vt row are permuted by
+        // the row's c8 (vt_unit), which spreads the stores of a wave's sixteen c8 over the banks.
+        for (int g = t; g < (R / 8) * 16; g += 256) {
+            const int c8 = g % (R / 8), rg = g / (R / 8), par = rg & 1, base = (rg >> 1) * 8;
+            uint4 kraw[4], vraw[4];
+            float4 cs0[4], cs1[4];
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const float x = half_bits_to_float((uint16_t)(kw[j] & 0xffffu)), y = half_bits_to_float((uint16_t)(kw[j] >> 16));
-                xr[j] = x * c[j] - y * s[j];
-                yr[j] = x * s[j] + y * c[j];
+            for (int m = 0; m < 4; m++) {
+                const uint32_t p = min(k0 + base + par + 2 * m, a.backlog - 1);
+                kraw[m] = *reinterpret_cast<const uint4 *>(a.kcache + (size_t)p * D + (size_t)h * R + c8 * 8);
+                vraw[m] = *reinterpret_cast<const uint4 *>(a.vcache + (size_t)p * D + (size_t)h * R + c8 * 8);
+                cs0[m] = *reinterpret_cast<const float4 *>(a.trig_abs + (size_t)p * (R / 2) + c8 * 4);
+                cs1[m] = *reinterpret_cast<const float4 *>(a.trig_abs + (size_t)p * (R / 2) + c8 * 4 + 2);
             }
-            *reinterpret_cast<float4 *>(&l.kx[row][c8 * 4]) = make_float4(xr[0], xr[1], xr[2], xr[3]);
-            *reinterpret_cast<float4 *>(&l.ky[row][c8 * 4]) = make_float4(yr[0], yr[1], yr[2], yr[3]);
-            const uint32_t vw[4] = {vraw.x, vraw.y, vraw.z, vraw.w};
+#pragma unroll
+            for (int m = 0; m < 4; m++) {
+                const int row = base + par + 2 * m;
+                const uint32_t kw[4] = {kraw[m].x, kraw[m].y, kraw[m].z, kraw[m].w};
+                const float c[4] = {cs0[m].x, cs0[m].z, cs1[m].x, cs1[m].z}, s[4] = {cs0[m].y, cs0[m].w, cs1[m].y, cs1[m].w};
+                float xr[4], yr[4];
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const float x = half_bits_to_float((uint16_t)(kw[j] & 0xffffu)), y = half_bits_to_float((uint16_t)(kw[j] >> 16));
+                    xr[j] = x * c[j] - y * s[j];
+                    yr[j] = x * s[j] + y * c[j];
+                }
+                *reinterpret_cast<float4 *>(&l.kx[row][c8 * 4]) = make_float4(xr[0], xr[1], xr[2], xr[3]);
+                *reinterpret_cast<float4 *>(&l.ky[row][c8 * 4]) = make_float4(yr[0], yr[1], yr[2], yr[3]);
+            }
+            const uint32_t vw[4][4] = {{vraw[0].x, vraw[0].y, vraw[0].z, vraw[0].w}, {vraw[1].x, vraw[1].y, vraw[1].z, vraw[1].w},
+                                       {vraw[2].x, vraw[2].y, vraw[2].z, vraw[2].w}, {vraw[3].x, vraw[3].y, vraw[3].z, vraw[3].w}};
+            const int unit = L::vt_unit(rg >> 1, c8);
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                l.vt[row & 1][c8 * 8 + 2 * j][row >> 1] = (uint16_t)(vw[j] & 0xffffu);
-                l.vt[row & 1][c8 * 8 + 2 * j + 1][row >> 1] = (uint16_t)(vw[j] >> 16);
+                // dims c8*8 + 2j (low halfs) and + 2j + 1 (high halfs) at positions m = 0..3
+                const uint2 lo = make_uint2((vw[0][j] & 0xffffu) | (vw[1][j] << 16), (vw[2][j] & 0xffffu) | (vw[3][j] << 16));
+                const uint2 hi = make_uint2((vw[0][j] >> 16) | (vw[1][j] & 0xffff0000u), (vw[2][j] >> 16) | (vw[3][j] & 0xffff0000u));
+                *reinterpret_cast<uint2 *>(&l.vt[par][c8 * 8 + 2 * j][unit * 4]) = lo;
+                *reinterpret_cast<uint2 *>(&l.vt[par][c8 * 8 + 2 * j + 1][unit * 4]) = hi;
             }
         }
         __syncthreads();
@@ -167,9 +188,14 @@ __global__ __launch_bounds__(256) void attention_batch_kernel(AttnBatchArgs a)
 #pragma unroll
         for (int d = 0; d < DT; d++) {
             // B operand: V[position 32 pt + 2j + hh][dim 32 d + n32], sixteen consecutive halfs of the transposed tile
-            const uint16_t *vr = &l.vt[hh][32 * d + n32][16 * pt];
-            const uint4 va = *reinterpret_cast<const uint4 *>(vr), vb = *reinterpret_cast<const uint4 *>(vr + 8);
-            const uint32_t vw[8] = {va.x, va.y, va.z, va.w, vb.x, vb.y, vb.z, vb.w};
+            const int dim = 32 * d + n32;
+            uint32_t vw[8];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const uint2 v2 = *reinterpret_cast<const uint2 *>(&l.vt[hh][dim][L::vt_unit(4 * pt + u, dim >> 3) * 4]);
+                vw[2 * u] = v2.x;
+                vw[2 * u + 1] = v2.y;
+            }
 #pragma unroll
             for (int j = 0; j < 8; j++) {
                 acc[d] = __builtin_amdgcn_mfma_f32_32x32x2f32(pf[2 * j], half_bits_to_float((uint16_t)(vw[j] & 0xffffu)), acc[d], 0, 0, 0);
