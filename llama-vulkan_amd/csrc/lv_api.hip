@@ -767,6 +767,18 @@ static uint32_t gemm_k_slices(uint32_t tiles, uint32_t k_steps)
     return best;
 }
 
+// out[n][ldo] (+)= the sum of `count` K slices [n][rows]
+static int launch_gemm_reduce(hipStream_t st, float *out, uint32_t ldo, float *const parts[kGemmMaxMats], uint32_t count, uint32_t rows, uint32_t n,
+                              bool accumulate)
+{
+    GemmReduceArgs r{};
+    for (uint32_t i = 0; i < count; i++) r.parts[i] = parts[i];
+    r.out = out; r.nparts = count; r.rows = rows; r.ldo = ldo; r.n = n; r.accumulate = accumulate ? 1 : 0;
+    gemm_reduce_kernel<<<dim3((rows / 4 + 255) / 256, n), dim3(256), 0, st>>>(r);
+    HIP_TRY(hipGetLastError());
+    return LV_OK;
+}
+
 // the slice count launch_gemm_sliced uses for n tokens of w into rows of ldo floats (the reduce works on float4)
 static uint32_t gemm_slices_for(const lv_matrix &w, uint32_t n, uint32_t ldo)
 {
@@ -777,9 +789,12 @@ static uint32_t gemm_slices_for(const lv_matrix &w, uint32_t n, uint32_t ldo)
 
 // one matrix, activations already split, K cut in slices when that fills the CUs better: the slices go to parts[]
 // ([n][rows] floats each, scratch of the caller) and gemm_reduce_kernel adds them to out in a fixed order
+// With `pending` given, the slices are left unsummed and *pending says how many there are (0: out is complete): the
+// caller adds them to out itself (prefill_norm_kernel does, on its way through the row).
 static int launch_gemm_sliced(hipStream_t st, float *out, uint32_t ldo, const lv_matrix &w, uint32_t n, const uint16_t *xh, const uint16_t *xl,
-                              bool accumulate, float *const parts[kGemmMaxMats])
+                              bool accumulate, float *const parts[kGemmMaxMats], uint32_t *pending = nullptr)
 {
+    if (pending) *pending = 0;
     const uint32_t rows = w.view.rows, k_steps = (w.view.cols + kGemmK - 1) / kGemmK;
     const uint32_t slices = parts ? gemm_slices_for(w, n, ldo) : 1;
     GemmArgs a{};
@@ -790,14 +805,11 @@ static int launch_gemm_sliced(hipStream_t st, float *out, uint32_t ldo, const lv
     }
     a.slice_steps = (k_steps + slices - 1) / slices;
     const uint32_t used = (k_steps + a.slice_steps - 1) / a.slice_steps;      // every slice launched has a step
-    GemmReduceArgs r{};
-    for (uint32_t i = 0; i < used; i++) { a.outs[i] = parts[i]; a.ws[i] = w.view; r.parts[i] = parts[i]; }
+    for (uint32_t i = 0; i < used; i++) { a.outs[i] = parts[i]; a.ws[i] = w.view; }
     a.ldo = rows;
     LV_TRY(dispatch_gemm(st, a, w, used));
-    r.out = out; r.nparts = used; r.rows = rows; r.ldo = ldo; r.n = n; r.accumulate = accumulate ? 1 : 0;
-    gemm_reduce_kernel<<<dim3((rows / 4 + 255) / 256, n), dim3(256), 0, st>>>(r);
-    HIP_TRY(hipGetLastError());
-    return LV_OK;
+    if (pending && accumulate) { *pending = used; return LV_OK; }
+    return launch_gemm_reduce(st, out, ldo, parts, used, rows, n, accumulate);
 }
 
 static int launch_gemm_presplit(hipStream_t st, float *out, uint32_t ldo, const lv_matrix &w, uint32_t n, const uint16_t *xh, const uint16_t *xl,
@@ -1473,6 +1485,27 @@ static int prefill_reserve(lv_session *s, uint32_t n)
     return LV_OK;
 }
 
+// x += pending K slices, xn = normalize(x) * w, halves of xn for a GEMM on weights of type ftype: one kernel where the
+// row fits its registers, else the three separate ones.  xn (fp32) is written only when want_xn.
+static int launch_prefill_norm(hipStream_t st, lv_session *s, const float *w, uint32_t n, uint32_t D, uint32_t ftype, float *const parts[kGemmMaxMats],
+                               uint32_t pending, bool want_xn)
+{
+    const uint32_t n_pad = (n + kGemmTile - 1) / kGemmTile * kGemmTile;
+    if (D <= 8192 && D % 4 == 0 && (ftype == LV_Q4_0 || ftype == LV_Q8_0)) {
+        PrefillNormArgs a{};
+        a.x = s->pf_x; a.nparts = pending; a.w = w; a.xn = want_xn ? s->pf_xn : nullptr; a.xh = s->pf_xh; a.xl = s->pf_xl; a.dim = D; a.n = n;
+        for (uint32_t i = 0; i < pending; i++) a.parts[i] = parts[i];
+        if (ftype == LV_Q4_0) prefill_norm_kernel<4><<<dim3(n_pad), dim3(256), 0, st>>>(a);
+        else prefill_norm_kernel<8><<<dim3(n_pad), dim3(256), 0, st>>>(a);
+        HIP_TRY(hipGetLastError());
+        return LV_OK;
+    }
+    if (pending) LV_TRY(launch_gemm_reduce(st, s->pf_x, D, parts, pending, D, n, true));
+    normalize_kernel<<<dim3(n), dim3(256), 0, st>>>(s->pf_xn, s->pf_x, w, D);
+    HIP_TRY(hipGetLastError());
+    return launch_split(st, s->pf_xh, s->pf_xl, s->pf_xn, n, D, ftype);
+}
+
 // Rows idx0 .. idx0+n-1 of the step at once (llava_layer.cpp:39-75 with batch > 1).  Row z sees cache rows
 // 0..pos+z: all K/V rows of the chunk are appended before any row attends, rows above its own are masked.
 static int record_prefill(lv_session *s, uint32_t idx0, uint32_t n, bool with_head)
@@ -1493,12 +1526,16 @@ static int record_prefill(lv_session *s, uint32_t idx0, uint32_t n, bool with_he
     HIP_TRY(hipGetLastError());
 
     const dim3 kv_grid((D + 255) / 256, n);
+    // q, k and v buffers of a layer are free once attention has run: they take the K slices of the output projection
+    // and of the down projection; `pending` of them wait to be added to the residual stream by the next norm
+    float *const parts[kGemmMaxMats] = {s->pf_q, s->pf_k, s->pf_v};
+    uint32_t pending = 0;
     for (uint32_t li = 0; li < hp.layers; li++) {
         const LayerWeights &lw = m->layers[li];
-        normalize_kernel<<<dim3(n), dim3(256), 0, st>>>(s->pf_xn, s->pf_x, lw.attn_norm, D);
-        HIP_TRY(hipGetLastError());
-        LV_TRY(launch_split(st, s->pf_xh, s->pf_xl, s->pf_xn, n, D, lw.wq.ftype));
-        if (gemm_same(lw.wq, lw.wk) && gemm_same(lw.wq, lw.wv)) {
+        const bool qkv_same = gemm_same(lw.wq, lw.wk) && gemm_same(lw.wq, lw.wv), gate_same = gemm_same(lw.w3, lw.w1);
+        LV_TRY(launch_prefill_norm(st, s, lw.attn_norm, n, D, lw.wq.ftype, parts, pending, !qkv_same));
+        pending = 0;
+        if (qkv_same) {
             float *const outs[3] = {s->pf_q, s->pf_k, s->pf_v};
             const lv_matrix *const ws[3] = {&lw.wq, &lw.wk, &lw.wv};
             LV_TRY(launch_gemm_multi(st, outs, D, ws, 3, n, s->pf_xh, s->pf_xl, false));
@@ -1513,15 +1550,11 @@ static int record_prefill(lv_session *s, uint32_t idx0, uint32_t n, bool with_he
         HIP_TRY(hipGetLastError());
         LV_TRY(launch_attention_batch(st, s->pf_vo, kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->pf_q, s->trig_abs, pos_ptr, idx0, n, s->backlog,
                                       hp.heads, hp.rot));
-        // q, k and v have been consumed: their buffers take the K slices of the output projection, and of the down
-        // projection further on
-        float *const parts[kGemmMaxMats] = {s->pf_q, s->pf_k, s->pf_v};
         LV_TRY(launch_split(st, s->pf_xh, s->pf_xl, s->pf_vo, n, D, lw.wo.ftype));
-        LV_TRY(launch_gemm_sliced(st, s->pf_x, D, lw.wo, n, s->pf_xh, s->pf_xl, true, parts));
-        normalize_kernel<<<dim3(n), dim3(256), 0, st>>>(s->pf_xn, s->pf_x, lw.ffn_norm, D);
-        HIP_TRY(hipGetLastError());
-        LV_TRY(launch_split(st, s->pf_xh, s->pf_xl, s->pf_xn, n, D, lw.w3.ftype));
-        if (gemm_same(lw.w3, lw.w1)) {
+        LV_TRY(launch_gemm_sliced(st, s->pf_x, D, lw.wo, n, s->pf_xh, s->pf_xl, true, parts, &pending));
+        LV_TRY(launch_prefill_norm(st, s, lw.ffn_norm, n, D, lw.w3.ftype, parts, pending, !gate_same));
+        pending = 0;
+        if (gate_same) {
             float *const outs[2] = {s->pf_g1, s->pf_g2};
             const lv_matrix *const ws[2] = {&lw.w3, &lw.w1};
             LV_TRY(launch_gemm_multi(st, outs, F, ws, 2, n, s->pf_xh, s->pf_xl, false));
@@ -1534,8 +1567,9 @@ static int record_prefill(lv_session *s, uint32_t idx0, uint32_t n, bool with_he
         silu_mul_kernel<<<dim3((unsigned)((count + 255) / 256)), dim3(256), 0, st>>>(s->pf_g1, s->pf_g1, s->pf_g2, count);
         HIP_TRY(hipGetLastError());
         LV_TRY(launch_split(st, s->pf_xh, s->pf_xl, s->pf_g1, n, F, lw.w2.ftype));
-        LV_TRY(launch_gemm_sliced(st, s->pf_x, D, lw.w2, n, s->pf_xh, s->pf_xl, true, parts));
+        LV_TRY(launch_gemm_sliced(st, s->pf_x, D, lw.w2, n, s->pf_xh, s->pf_xl, true, parts, &pending));
     }
+    if (pending) LV_TRY(launch_gemm_reduce(st, s->pf_x, D, parts, pending, D, n, true));
     if (with_head) {
         // only the last row's logits are ever read (llava_session.cpp:131-139)
         normalize_kernel<<<dim3(1), dim3(256), 0, st>>>(s->xn, s->pf_x + (size_t)(n - 1) * D, m->norm, D);

@@ -154,6 +154,79 @@ __device__ __forceinline__ void gemm_codes_half(uint16_t *w, const CW &c)
     for (int g = 0; g < 2; g++) *reinterpret_cast<uint4 *>(w + 8 * g) = make_uint4(ph[4 * g], ph[4 * g + 1], ph[4 * g + 2], ph[4 * g + 3]);
 }
 
+// The steps between two GEMMs of a prompt batch as one pass over a token row: x += the K slices of the product
+// before (same order as gemm_reduce_kernel: slices first, then x), xn = normalize(x) * w (normalize_kernel's
+// arithmetic), and xn split in the two fp16 halves the next GEMM reads (split_half_kernel's layout for weight type QT).
+// One 256-thread workgroup per row of the padded batch; rows n.. are written as zeros.  dim <= 8192, a multiple of 4.
+struct PrefillNormArgs {
+    float *x;                              // [n][dim] residual stream, updated when nparts > 0
+    const float *parts[kGemmMaxMats];      // [n][dim] each
+    uint32_t nparts;
+    const float *w;                        // norm weights
+    float *xn;                             // [n][dim] or null: the normalised row as fp32 (for a GEMV-type consumer)
+    uint16_t *xh, *xl;                     // [n_pad][dim]
+    uint32_t dim, n;
+};
+template <int QT>
+__global__ __launch_bounds__(256) void prefill_norm_kernel(PrefillNormArgs a)
+{
+    __shared__ float lds[4];
+    constexpr int PER = 8;
+    const uint32_t row = blockIdx.x, dim = a.dim, n4 = dim / 4;
+    const bool live = row < a.n;
+    const size_t ro = (size_t)(live ? row : 0) * dim;
+    float4 v[PER], wv[PER];
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+        const uint32_t i = threadIdx.x + j * 256;
+        const bool ok = live && i < n4;
+        const uint32_t ic = ok ? i : 0;
+        wv[j] = reinterpret_cast<const float4 *>(a.w)[i < n4 ? i : 0];
+        float4 x4 = reinterpret_cast<const float4 *>(a.x + ro)[ic];
+        if (a.nparts) {
+            float4 s4 = reinterpret_cast<const float4 *>(a.parts[0] + ro)[ic];
+            for (uint32_t q = 1; q < a.nparts; q++) {
+                const float4 p4 = reinterpret_cast<const float4 *>(a.parts[q] + ro)[ic];
+                s4.x += p4.x; s4.y += p4.y; s4.z += p4.z; s4.w += p4.w;
+            }
+            x4.x = s4.x + x4.x; x4.y = s4.y + x4.y; x4.z = s4.z + x4.z; x4.w = s4.w + x4.w;
+            if (ok) reinterpret_cast<float4 *>(a.x + ro)[ic] = x4;
+        }
+        v[j] = ok ? x4 : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < PER; j++) s += (v[j].x + v[j].y) + (v[j].z + v[j].w);
+    const float mean = block_sum_256(s, lds) / (float)dim;
+    float q = 0.f;
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+        if (threadIdx.x + j * 256 < n4) {
+            const float c0 = v[j].x - mean, c1 = v[j].y - mean, c2 = v[j].z - mean, c3 = v[j].w - mean;
+            q = fmaf(c0, c0, q); q = fmaf(c1, c1, q); q = fmaf(c2, c2, q); q = fmaf(c3, c3, q);
+        }
+    }
+    const float inv = rsqrtf(block_sum_256(q, lds) / (float)dim);
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+        const uint32_t i = threadIdx.x + j * 256;
+        if (i >= n4) continue;
+        float f[4] = {(v[j].x * wv[j].x) * inv, (v[j].y * wv[j].y) * inv, (v[j].z * wv[j].z) * inv, (v[j].w * wv[j].w) * inv};
+        if (!live) f[0] = f[1] = f[2] = f[3] = 0.f;        // a padding row (its inv is not finite)
+        if (live && a.xn) reinterpret_cast<float4 *>(a.xn + ro)[i] = make_float4(f[0], f[1], f[2], f[3]);
+        const uint32_t e = i * 4, blk0 = e & ~31u, e0 = e & 31u;
+        uint16_t *hr = a.xh + (size_t)row * dim + blk0, *lr = a.xl + (size_t)row * dim + blk0;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const uint16_t h = float_to_half_bits(f[k]);
+            const uint16_t l = float_to_half_bits(f[k] - half_bits_to_float(h));
+            const int pos = gemm_k_position<QT>((int)e0 + k);
+            hr[pos] = h;
+            lr[pos] = l;
+        }
+    }
+}
+
 // RM = weight rows per workgroup (128 or 64); tokens per workgroup: 128.  The four waves split the tile 2 x 2
 // (RM = 128: 64 tokens x 64 rows each) or 4 x 1 (RM = 64: 32 tokens x 64 rows each).  The narrow form doubles the
 // number of workgroups for matrices that would otherwise not fill 256 CUs.

@@ -100,6 +100,24 @@ def test_prompt_as_one_batch_matches_oracle(lva, orc, ctx, tiny_models, name, n_
     a.close(); b.close(); model.close(); osess.close(); om.close()
 
 
+def test_prompt_batch_of_a_model_wider_than_the_fused_norm_pass(lva, orc, ctx, tmp_path):
+    """rows of 8256 floats: the pass that sums the K slices, normalises and splits in one kernel holds at most 8192 per
+    row in registers, so this model takes the three separate kernels, with three K slices pending between the layers"""
+    path = str(tmp_path / "wide.ggml")
+    lva.write_model(path, wtype=lva.LV_Q4_0, seed=21, vocab=320, layers=2, dim=8256, heads=129, ff=96)
+    om = orc.Model(path)
+    osess = orc.Session(om, 64)
+    model = lva.Model(ctx, path)
+    s = lva.Session(model, 64)
+    prompt = lva.synth_tokens(24, 3, 320, seed=22)
+    want = osess.eval(prompt)
+    s.begin(prompt, 0)
+    got = s.logits()
+    assert np.all(np.abs(got - want) <= 1e-2 + 1e-3 * np.abs(want)), float(np.max(np.abs(got - want)))
+    assert s.argmax() == orc.greedy(want)
+    s.close(); model.close(); osess.close(); om.close()
+
+
 def test_second_batch_appends_behind_the_first(lva, orc, ctx, tiny_models):
     """two batched steps in a row (prompt, then a long addition): rows of the second see the cache of the first"""
     path = tiny_models["tiny_q4"]
