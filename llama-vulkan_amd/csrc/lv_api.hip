@@ -1563,10 +1563,12 @@ static int record_prefill(lv_session *s, uint32_t idx0, uint32_t n, bool with_he
             if (lw.w1.ftype == lw.w3.ftype) LV_TRY(launch_gemm_presplit(st, s->pf_g2, F, lw.w1, n, s->pf_xh, s->pf_xl, false));
             else LV_TRY(launch_gemm(st, s->pf_g2, F, lw.w1, s->pf_xn, n, s->pf_xh, s->pf_xl, false));
         }
-        const size_t count = (size_t)n * F;
-        silu_mul_kernel<<<dim3((unsigned)((count + 255) / 256)), dim3(256), 0, st>>>(s->pf_g1, s->pf_g1, s->pf_g2, count);
-        HIP_TRY(hipGetLastError());
-        LV_TRY(launch_split(st, s->pf_xh, s->pf_xl, s->pf_g1, n, F, lw.w2.ftype));
+        {   // SwiGLU straight into the fp16 halves the down projection reads
+            const dim3 grid((F / 4 + 255) / 256, (n + kGemmTile - 1) / kGemmTile * kGemmTile);
+            if (lw.w2.ftype == LV_Q4_0) silu_split_kernel<4><<<grid, dim3(256), 0, st>>>(s->pf_xh, s->pf_xl, s->pf_g1, s->pf_g2, n, F);
+            else silu_split_kernel<8><<<grid, dim3(256), 0, st>>>(s->pf_xh, s->pf_xl, s->pf_g1, s->pf_g2, n, F);
+            HIP_TRY(hipGetLastError());
+        }
         LV_TRY(launch_gemm_sliced(st, s->pf_x, D, lw.w2, n, s->pf_xh, s->pf_xl, true, parts, &pending));
     }
     if (pending) LV_TRY(launch_gemm_reduce(st, s->pf_x, D, parts, pending, D, n, true));

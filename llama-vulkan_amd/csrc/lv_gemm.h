@@ -52,16 +52,6 @@ __global__ void split_half_kernel(uint16_t *__restrict__ xh, uint16_t *__restric
     }
 }
 
-// ff[n][F] = a * b / (exp(-b) + 1)   (matmul_silu_ff.comp:96 with a = W3 x, b = W1 x)
-__global__ void silu_mul_kernel(float *__restrict__ out, const float *__restrict__ a, const float *__restrict__ b, size_t count)
-{
-    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < count) {
-        const float r1 = a[i], r2 = b[i];
-        out[i] = r1 * r2 / (__expf(-r2) + 1.f);
-    }
-}
-
 constexpr int kGemmMaxMats = 3;
 struct GemmArgs {
     // up to three matrices of one shape and type applied to the same activations in one launch (blockIdx.z picks the
@@ -152,6 +142,34 @@ __device__ __forceinline__ void gemm_codes_half(uint16_t *w, const CW &c)
     }
 #pragma unroll
     for (int g = 0; g < 2; g++) *reinterpret_cast<uint4 *>(w + 8 * g) = make_uint4(ph[4 * g], ph[4 * g + 1], ph[4 * g + 2], ph[4 * g + 3]);
+}
+
+// ff[n][F] = a * b / (exp(-b) + 1) (matmul_silu_ff.comp:96 with a = W3 x, b = W1 x), written as the two fp16 halves
+// the down projection's GEMM reads (split_half_kernel's layout for weight type QT; rows n.. zero)
+template <int QT>
+__global__ void silu_split_kernel(uint16_t *__restrict__ xh, uint16_t *__restrict__ xl, const float *__restrict__ a, const float *__restrict__ b,
+                                  uint32_t n, uint32_t K)
+{
+    const uint32_t row = blockIdx.y;
+    const uint32_t i = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    if (i >= K) return;
+    float f[4] = {0.f, 0.f, 0.f, 0.f};
+    if (row < n) {
+        const float4 r1 = *reinterpret_cast<const float4 *>(a + (size_t)row * K + i), r2 = *reinterpret_cast<const float4 *>(b + (size_t)row * K + i);
+        f[0] = r1.x * r2.x / (__expf(-r2.x) + 1.f);
+        f[1] = r1.y * r2.y / (__expf(-r2.y) + 1.f);
+        f[2] = r1.z * r2.z / (__expf(-r2.z) + 1.f);
+        f[3] = r1.w * r2.w / (__expf(-r2.w) + 1.f);
+    }
+    const uint32_t blk0 = i & ~31u, e0 = i & 31u;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const uint16_t h = float_to_half_bits(f[j]);
+        const uint16_t l = float_to_half_bits(f[j] - half_bits_to_float(h));
+        const int pos = gemm_k_position<QT>((int)e0 + j);
+        xh[(size_t)row * K + blk0 + pos] = h;
+        xl[(size_t)row * K + blk0 + pos] = l;
+    }
 }
 
 // The steps between two GEMMs of a prompt batch as one pass over a token row: x += the K slices of the product
