@@ -721,13 +721,13 @@ static int dispatch_gemm(hipStream_t st, const GemmArgs &a, const lv_matrix &w, 
     constexpr uint32_t cus = 256;
     const uint32_t t128 = (w.view.rows + 127) / 128 * token_tiles * nz, t256 = (w.view.rows + 255) / 256 * token_tiles * nz;
     const bool narrow = t128 < 128;
-    // (q8_0 only: the q4_0 instantiation of the 256-row form spills registers and is 4 % slower than the base form)
-    const bool wide = !narrow && w.ftype == LV_Q8_0 && (double)((t256 + cus - 1) / cus) * 1.84 < (double)((t128 + cus - 1) / cus);
+    const bool wide = !narrow && (double)((t256 + cus - 1) / cus) * 1.84 < (double)((t128 + cus - 1) / cus);
     const uint32_t rm = narrow ? 64 : wide ? 256 : 128;
     const dim3 grid((w.view.rows + rm - 1) / rm, token_tiles, nz);
     const bool sf32 = w.view.scales_f32 != nullptr;
     if (w.ftype == LV_Q4_0) {
         if (narrow) { if (sf32) gemm_kernel<4, 64, 4, true><<<grid, dim3(256), 0, st>>>(a); else gemm_kernel<4, 64, 4, false><<<grid, dim3(256), 0, st>>>(a); }
+        else if (wide) { if (sf32) gemm_kernel<4, 256, 8, true, true><<<grid, dim3(512), 0, st>>>(a); else gemm_kernel<4, 256, 8, false, true><<<grid, dim3(512), 0, st>>>(a); }
         else { if (sf32) gemm_kernel<4, 128, 8, true, true><<<grid, dim3(512), 0, st>>>(a); else gemm_kernel<4, 128, 8, false, true><<<grid, dim3(512), 0, st>>>(a); }
     } else if (w.ftype == LV_Q8_0) {
         if (narrow) { if (sf32) gemm_kernel<8, 64, 4, true><<<grid, dim3(256), 0, st>>>(a); else gemm_kernel<8, 64, 4, false><<<grid, dim3(256), 0, st>>>(a); }

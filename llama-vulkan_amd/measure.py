@@ -6,6 +6,7 @@
     python llama-vulkan_amd/measure.py decode-13b    13B q4_0, 32-token prompt + 256 greedy steps
     python llama-vulkan_amd/measure.py prefill-13b   13B q8_0, 512-token prompt evaluated in one lv_step_begin
     python llama-vulkan_amd/measure.py prefill-7b    7B q4_0, the same
+    python llama-vulkan_amd/measure.py prefill-13b-q4  13B q4_0, the same
     python llama-vulkan_amd/measure.py gemm          isolated 512-token GEMMs at the 13B shapes, q8_0 (for kernel traces and counters)
     python llama-vulkan_amd/measure.py copy          1 GiB device-to-device copy: achievable bandwidth, counter calibration
     python llama-vulkan_amd/measure.py all
@@ -184,6 +185,8 @@ def main():
         decode_case(ctx, "decode-13b", "13b", lva.LV_Q4_0, 2, 512, 32, 256)
     if which in ("prefill-13b", "all"):
         prefill_case(ctx, "prefill-13b", "13b", lva.LV_Q8_0)
+    if which in ("prefill-13b-q4", "all"):
+        prefill_case(ctx, "prefill-13b-q4", "13b", lva.LV_Q4_0)
     if which in ("prefill-7b", "all"):
         prefill_case(ctx, "prefill-7b", "7b", lva.LV_Q4_0)
 
