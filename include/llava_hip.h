@@ -191,6 +191,16 @@ int lv_kernel_kv_append(lv_ctx *ctx, void *cache, const float *in, uint32_t pos,
 int lv_kernel_attention(lv_ctx *ctx, float *out, const void *kcache, const void *vcache, const float *q,
                         uint32_t pos, uint32_t backlog, uint32_t heads, uint32_t rot, uint32_t batch);
 
+/* lv_kernel_attention for callers that cannot allocate device memory (code under HIP graph capture, serving loops and
+ * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments, same result; the rotation
+ * table, the partial sums and the split counters live in a fixed 2 MiB work area that every device holds from library
+ * load to process end, so the call allocates nothing and frees nothing.  Limits (LV_ERR_RANGE beyond them):
+ * backlog * rot / 2 <= 131072, batch * heads * ceil(backlog / 64) * (rot + 1) <= 262144, batch * heads <= 256.
+ * All calls on one device share the work area: calls that overlap on one device (different contexts, different threads)
+ * race; calls on one context are ordered by its stream. */
+int lv_kernel_attention_static(lv_ctx *ctx, float *out, const void *kcache, const void *vcache, const float *q,
+                               uint32_t pos, uint32_t backlog, uint32_t heads, uint32_t rot, uint32_t batch);
+
 #ifdef __cplusplus
 }
 #endif

@@ -117,6 +117,7 @@ _HIP_SIGS = {
     "lv_kernel_normalize": [_VP, _VP, _VP, _VP, _U32, _U32],
     "lv_kernel_kv_append": [_VP, _VP, _VP, _U32, _U32, _U32, _U32],
     "lv_kernel_attention": [_VP, _VP, _VP, _VP, _VP, _U32, _U32, _U32, _U32, _U32],
+    "lv_kernel_attention_static": [_VP, _VP, _VP, _VP, _VP, _U32, _U32, _U32, _U32, _U32],
 }
 
 

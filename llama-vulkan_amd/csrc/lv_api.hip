@@ -69,6 +69,7 @@ struct lv_ctx {
     uint32_t *attn_counters = nullptr;
     size_t attn_part_floats = 0, attn_counter_words = 0;
     hipEvent_t ev_start = nullptr, ev_stop = nullptr;
+    struct AttnScratch *scratch = nullptr;   // this device's copy of the file-scope scratch array (lv_kernel_attention_static)
     // Persistent decode kernels of different sessions (one per thread, llava_context.h:47-49 has the same pools and
     // mutexes for the same reason) must not overlap on the device: each occupies every CU and its workgroups wait
     // for each other.  A launch on another session's stream first waits for the event the last launch recorded.
@@ -177,6 +178,22 @@ static uint16_t *kv_ptr(const lv_session *s, uint32_t layer, int which)
 }
 
 // -----------------------------------------------------------------------------------------------------------
+// Device memory that exists without any allocation call: the work area of lv_kernel_attention_static, for callers that
+// may not allocate.  Every device the library runs on holds its own copy from the moment the code object is loaded until
+// the process ends.  Host code never uses the array's name as an address: lv_ctx_create asks the runtime for this
+// device's copy once (hipGetSymbolAddress) and keeps the pointer in the context.
+// -----------------------------------------------------------------------------------------------------------
+constexpr uint32_t kStaticTrigPairs = 131072;   // rotation table: backlog * rot / 2 (cos, sin) pairs (2048 rows of a 128-wide head)
+constexpr uint32_t kStaticPartFloats = 262144;  // partial sums: batch * heads * ceil(backlog / 64) * (rot + 1)
+constexpr uint32_t kStaticCounters = 256;       // batch * heads
+struct AttnScratch {
+    float2 trig[kStaticTrigPairs];
+    float part[kStaticPartFloats];
+    uint32_t counters[kStaticCounters];
+};
+static __device__ __align__(256) unsigned char scratch[sizeof(AttnScratch)];   // 2 MiB + 1 KiB
+
+// -----------------------------------------------------------------------------------------------------------
 // context
 // -----------------------------------------------------------------------------------------------------------
 extern "C" int lv_ctx_create(int device, lv_ctx **out)
@@ -192,7 +209,10 @@ extern "C" int lv_ctx_create(int device, lv_ctx **out)
     c->device = device;
     hipError_t e = hipGetDeviceProperties(&c->props, device);
     if (e == hipSuccess) e = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking);
+    // the address of the scratch array on THIS device (the current one); each device has its own copy at its own address
+    if (e == hipSuccess) e = hipGetSymbolAddress(reinterpret_cast<void **>(&c->scratch), HIP_SYMBOL(scratch));
     if (e != hipSuccess) {
+        if (c->stream) (void)hipStreamDestroy(c->stream);
         delete c;
         return fail(LV_ERR_HIP, "lv_ctx_create: %s", hipGetErrorString(e));
     }
@@ -910,6 +930,50 @@ extern "C" int lv_kernel_attention(lv_ctx *c, float *out, const void *kcache, co
     }
     return launch_attention(c->stream, out, static_cast<const uint16_t *>(kcache), static_cast<const uint16_t *>(vcache), q,
                             c->trig, c->attn_part, c->attn_counters, nullptr, pos, backlog, heads, rot, batch);
+}
+
+// cos/sin table of build_trig computed on the device (same fp32 angle rounding: theta_i from the host's powf, the
+// product in fp32, the functions in double)
+struct TrigFreq { float f[64]; };
+__global__ void trig_fill_kernel(float2 *__restrict__ t, TrigFreq fr, uint32_t rows, uint32_t half)
+{
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= rows * half) return;
+    const uint32_t d = i / half, j = i % half;
+    const float ang = (float)d * fr.f[j];
+    t[i] = make_float2((float)cos((double)ang), (float)sin((double)ang));
+}
+
+// lv_kernel_attention without a single allocation: rotation table, partial sums and split counters live in this
+// device's copy of the file-scope scratch array.  Calls on one device share that array, so two of them must not overlap
+// (calls on one context are ordered by its stream).  The array keeps the last call's contents: the counters are cleared
+// and the table rewritten by small kernels in front of the attention kernel; the partial sums are written before read.
+extern "C" int lv_kernel_attention_static(lv_ctx *c, float *out, const void *kcache, const void *vcache, const float *q, uint32_t pos,
+                                          uint32_t backlog, uint32_t heads, uint32_t rot, uint32_t batch)
+{
+    if (!c || !out || !kcache || !vcache || !q) return fail(LV_ERR_ARG, "lv_kernel_attention_static: null argument");
+    if (heads == 0 || batch == 0 || backlog == 0) return fail(LV_ERR_ARG, "lv_kernel_attention_static: empty shape");
+    if ((uint64_t)pos + batch > backlog) return fail(LV_ERR_RANGE, "lv_kernel_attention_static: rows %u+%u of %u", pos, batch, backlog);
+    if (rot != 32 && rot != 64 && rot != 128) return fail(LV_ERR_ARG, "lv_kernel_attention_static: head size %u", rot);
+    if (!c->scratch) return fail(LV_ERR_STATE, "lv_kernel_attention_static: the context has no scratch address");
+    const uint64_t splits = ((uint64_t)backlog + kAttnChunk - 1) / kAttnChunk;
+    const uint64_t need_trig = (uint64_t)backlog * (rot / 2), need_part = (uint64_t)batch * heads * splits * (rot + 1),
+                   need_cnt = (uint64_t)batch * heads;
+    if (need_trig > kStaticTrigPairs || need_part > kStaticPartFloats || need_cnt > kStaticCounters)
+        return fail(LV_ERR_RANGE,
+                    "lv_kernel_attention_static: backlog %u x heads %u x head size %u x batch %u exceeds the static work area "
+                    "(backlog * rot / 2 <= %u, batch * heads * ceil(backlog / 64) * (rot + 1) <= %u, batch * heads <= %u)",
+                    backlog, heads, rot, batch, kStaticTrigPairs, kStaticPartFloats, kStaticCounters);
+    HIP_TRY(hipSetDevice(c->device));
+    AttnScratch *sc = c->scratch;
+    TrigFreq fr{};
+    const uint32_t half = rot / 2;
+    for (uint32_t i = 0; i < half; i++) fr.f[i] = powf(10000.0f, -(float)i / (float)half);
+    trig_fill_kernel<<<dim3((unsigned)((need_trig + 255) / 256)), dim3(256), 0, c->stream>>>(sc->trig, fr, backlog, half);
+    HIP_TRY(hipGetLastError());
+    LV_TRY(zero_async(sc->counters, sizeof sc->counters, c->stream));
+    return launch_attention(c->stream, out, static_cast<const uint16_t *>(kcache), static_cast<const uint16_t *>(vcache), q, sc->trig,
+                            sc->part, sc->counters, nullptr, pos, backlog, heads, rot, batch);
 }
 
 // -----------------------------------------------------------------------------------------------------------
