@@ -58,9 +58,6 @@ __device__ __forceinline__ void st_dev(float *p, float v)
 // (__syncthreads would wait for vmcnt(0) and drain the queue at every phase step).
 __device__ __forceinline__ void lds_barrier()
 {
-#ifdef LV_MEGA_FREERUN   // experiment: no synchronisation at all, to time the bare weight stream + tile arithmetic
-    return;
-#endif
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
@@ -176,14 +173,24 @@ __device__ __forceinline__ void poll_values(float (&v)[N], const float *p, int s
     if (pending) *status = 1u;
 }
 
+// The phase's input vector sits in LDS block by block (32 floats = 128 bytes), and lane l of a wave reads block
+// 64 * slab + l: in plain order the 64 lanes of a 128-bit read would all fall on the same four banks (measured: 0.8 us
+// per phase between the vector's arrival and the first tile).  Inside each block the eight 16-byte groups are therefore
+// rotated by the block index, so that eight consecutive lanes cover all 32 banks.
+__device__ __forceinline__ int xs_index(int idx)
+{
+    return (idx & ~31) | ((((idx >> 2) + (idx >> 5)) & 7) << 2) | (idx & 3);
+}
+
 // the 32 activations of this lane's block column, from LDS
 __device__ __forceinline__ void load_slab(float (&xr)[32], float &xsum, const float *xs, int block, bool have)
 {
-    const float4 *src = reinterpret_cast<const float4 *>(xs + (have ? block : 0) * 32);
+    const int blk = have ? block : 0;
+    const float *src = xs + blk * 32;
     float s = 0.f;
 #pragma unroll
     for (int j = 0; j < 8; j++) {
-        float4 v = src[j];
+        float4 v = *reinterpret_cast<const float4 *>(src + 4 * ((j + blk) & 7));
         if (!have) v = make_float4(0.f, 0.f, 0.f, 0.f);
         xr[4 * j] = v.x; xr[4 * j + 1] = v.y; xr[4 * j + 2] = v.z; xr[4 * j + 3] = v.w;
         s += (v.x + v.y) + (v.z + v.w);
@@ -309,30 +316,18 @@ struct MegaLds {
     float xs[XS];                    // the phase's input vector (during attention: exp(score) of the chunk)
     float red[RED_ROWS * RED_COLS];  // per-row partial sums, one column per slab
     float xown[S::ROWS_C];           // this workgroup's rows of the residual stream
-    float scratch[2 * S::NW];        // two halves: mean, then variance
+    float scratch[2 * S::NW];        // two halves: the waves' sums of x, then of x^2 (later: best logit and its index)
     float attn_red[S::NW * (S::R + 1)];
+    float qkv[3 * S::R];             // query of the workgroup's head, K and V row of the newest position
 };
 
-// Sum over the workgroup through NW floats of LDS.  One barrier: the caller guarantees that nobody still reads
-// `scratch` from an earlier use (consecutive sums use different halves of the scratch area, and every phase has
-// barriers of its own before the next pair of sums).
-template <int NW>
-__device__ __forceinline__ float block_sum(float v, float *scratch /* NW floats */)
-{
-    v = wave_sum(v);
-    if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = v;
-    lds_barrier();
-    float t = 0.f;
-#pragma unroll
-    for (int i = 0; i < NW; i++) t += scratch[i];
-    return t;
-}
-
-// Brings the N-float vector at `src` (being produced by other workgroups) into LDS, optionally normalised
-// (normalize.comp:34-64: mean, then mean-centred variance, no epsilon) with weights w.  One round trip to
-// memory when the data is there: the norm weights are requested before the wait, not after it.
+// Brings the N-float vector at `src` (being produced by other workgroups) into LDS.  With NORM the vector is to be
+// normalised (normalize.comp:34-64: x * w * rsqrt(mean((x - mean)^2)), no epsilon): LDS gets x * w, and the scale
+// rsqrt(variance), the same for every element, is returned for the caller to apply to its row sums.  The waves so
+// start on their tiles one barrier after the vector has arrived instead of three; the variance is taken as
+// mean(x^2) - mean(x)^2 from one pass over the registers.  The norm weights are requested before the wait, not after.
 template <int N, int NW, bool NORM, int SLEEP = 0>
-__device__ __forceinline__ void acquire_vector(float *xs, const float *src, const float *w, float *scratch, uint32_t *status, uint32_t spin_limit)
+__device__ __forceinline__ float acquire_vector(float *xs, const float *src, const float *w, float *scratch, uint32_t *status, uint32_t spin_limit)
 {
     constexpr int T = NW * 64, PER = cdiv(N, T);
     float v[PER];
@@ -345,27 +340,32 @@ __device__ __forceinline__ void acquire_vector(float *xs, const float *src, cons
         for (int j = 0; j < PER; j++) wn[j] = want[j] ? w[threadIdx.x + j * T] : 0.f;
     }
     poll_values<PER, SLEEP>(v, src + threadIdx.x, T, want, status, spin_limit);
+    float inv = 1.f;
     if constexpr (NORM) {
-        float s = 0.f;
-#pragma unroll
-        for (int j = 0; j < PER; j++) s += want[j] ? v[j] : 0.f;
-        const float mean = block_sum<NW>(s, scratch) / (float)N;
-        float q = 0.f;
+        float s1 = 0.f, s2 = 0.f;
 #pragma unroll
         for (int j = 0; j < PER; j++) {
-            const float c = want[j] ? v[j] - mean : 0.f;
-            q = fmaf(c, c, q);
+            const float x = want[j] ? v[j] : 0.f;
+            s1 += x;
+            s2 = fmaf(x, x, s2);
+            if (want[j]) xs[xs_index(threadIdx.x + j * T)] = x * wn[j];
         }
-        const float inv = rsqrtf(block_sum<NW>(q, scratch + NW) / (float)N);
+        s1 = wave_sum(s1);
+        s2 = wave_sum(s2);
+        if ((threadIdx.x & 63) == 0) { scratch[threadIdx.x >> 6] = s1; scratch[NW + (threadIdx.x >> 6)] = s2; }
+        lds_barrier();
+        float t1 = 0.f, t2 = 0.f;
 #pragma unroll
-        for (int j = 0; j < PER; j++)
-            if (want[j]) xs[threadIdx.x + j * T] = (v[j] * wn[j]) * inv;
+        for (int i = 0; i < NW; i++) { t1 += scratch[i]; t2 += scratch[NW + i]; }
+        const float mean = t1 / (float)N;
+        inv = rsqrtf(t2 / (float)N - mean * mean);
     } else {
 #pragma unroll
         for (int j = 0; j < PER; j++)
-            if (want[j]) xs[threadIdx.x + j * T] = v[j];
+            if (want[j]) xs[xs_index(threadIdx.x + j * T)] = v[j];
+        lds_barrier();
     }
-    lds_barrier();
+    return inv;
 }
 
 template <class S>
@@ -390,14 +390,12 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
     for (int k = 0; k < S::DEPTH; k++) mw.fetch(q[k], k, 0);
 
     // ---- re-arm the other buffer set for the next token ---------------------------------------------------------
-#ifndef LV_MEGA_NOWAIT   // (experiment builds leave stale, "ready" data in place to time the kernel without hand-over waits)
     {
         const size_t n4 = ((size_t)a.layers * S::XCHG_LAYER + S::XCHG_TAIL) / 4;
         uint4 *dst = reinterpret_cast<uint4 *>(a.xchg_rearm);
         for (size_t i = (size_t)b * T + threadIdx.x; i < n4; i += (size_t)kMegaWGs * T)
             dst[i] = make_uint4(kNotReady, kNotReady, kNotReady, kNotReady);
     }
-#endif
 
     const uint32_t pos = a.pos;
     const float *x_src = a.tok_f32 + (size_t)a.token * D;  // layer 0 reads the embedding row directly (constant data)
@@ -413,13 +411,13 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
 
         // ================= A: norm + QKV ====================================================================
         MEGA_STAMP(0);
-        acquire_vector<D, NW, true, kPollDelay>(xs, x_src, norm_w, scratch, status, spin_limit);
+        const float inv_a = acquire_vector<D, NW, true, kPollDelay>(xs, x_src, norm_w, scratch, status, spin_limit);
         MEGA_STAMP(1);
         load_slab(xr, xsum, xs, mw.sD * 64 + lane, mw.laneD);
         gemv_phase<S, S::SEQ_A, S::TA, S::NSD>(q, mw, layer, xr, xsum, mw.sD, mw.rD, mw.actD, S::ROWS_A, red);
         lds_barrier();
         if (threadIdx.x < S::ROWS_A) {
-            const float v = red_row<S::NSD>(red, threadIdx.x);
+            const float v = red_row<S::NSD>(red, threadIdx.x) * inv_a;
             const int g = b * S::ROWS_A + threadIdx.x, which = g / D, col = g % D;
             if (which == 0) {
                 st_dev(xc + S::OFF_QKV + col, v);
@@ -468,14 +466,32 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
                 };
 #pragma unroll
                 for (int r = 0; r < PRE; r++) request_round(r, p_begin + r * RPR);
-                // one wait for the query and, in the lanes that own the newest position, its K and V row
-                const bool newest = (pos >= p_begin && pos < p_end) && ((pos - p_begin) % RPR) == (uint32_t)rsel;
+                // The query of this head and, where the chunk holds the newest position, that position's K and V row (all
+                // three still on their way from phase A): waves 0, 1 and 2 fetch one of them each, two floats a lane, and
+                // pass them on through LDS (every 16-lane group polling the same 512 bytes for itself cost 32 times the
+                // requests).  The polls travel behind the cache rows requested above: that is the time the producers'
+                // stores need to become visible, so no sleep in front of them.
+                const bool holds_new = pos >= p_begin && pos < p_end;          // uniform over the workgroup
+                if (w < 3 && (w == 0 || holds_new)) {
+                    float pv[2];
+                    const bool want2[2] = {true, true};
+                    poll_values<2, 0>(pv, xc + S::OFF_QKV + w * D + h * R + lane * 2, 1, want2, status, spin_limit);
+                    l.qkv[w * R + lane * 2] = pv[0];
+                    l.qkv[w * R + lane * 2 + 1] = pv[1];
+                }
+                lds_barrier();
+                const bool newest = holds_new && ((pos - p_begin) % RPR) == (uint32_t)rsel;
                 float qkv[24];
                 {
-                    bool want24[24];
+                    const float4 *qs = reinterpret_cast<const float4 *>(l.qkv + sub * 8);
+                    const float4 q0 = qs[0], q1 = qs[1];
+                    qkv[0] = q0.x; qkv[1] = q0.y; qkv[2] = q0.z; qkv[3] = q0.w; qkv[4] = q1.x; qkv[5] = q1.y; qkv[6] = q1.z; qkv[7] = q1.w;
 #pragma unroll
-                    for (int i = 0; i < 24; i++) want24[i] = i < 8 || newest;
-                    poll_values<24, kPollDelay>(qkv, xc + S::OFF_QKV + h * R + sub * 8, 1, want24, status, spin_limit, D / 8);
+                    for (int i = 8; i < 24; i++) qkv[i] = 0.f;
+                    if (newest) {
+#pragma unroll
+                        for (int i = 0; i < 8; i++) { qkv[8 + i] = l.qkv[R + sub * 8 + i]; qkv[16 + i] = l.qkv[2 * R + sub * 8 + i]; }
+                    }
                 }
                 MEGA_STAMP(3);
                 const float scale = rsqrtf((float)R);
@@ -591,14 +607,14 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
 
         // ================= D: norm + SwiGLU ========================================================================
         MEGA_STAMP(7);
-        acquire_vector<D, NW, true, kPollDelay>(xs, xc + S::OFF_X1, norm_w + D, scratch, status, spin_limit);
+        const float inv_d = acquire_vector<D, NW, true, kPollDelay>(xs, xc + S::OFF_X1, norm_w + D, scratch, status, spin_limit);
         MEGA_STAMP(8);
         load_slab(xr, xsum, xs, mw.sD * 64 + lane, mw.laneD);
         gemv_phase<S, S::SEQ_D, S::TD, S::NSD>(q, mw, layer, xr, xsum, mw.sD, mw.rD, mw.actD, S::ROWS_D, red);
         lds_barrier();
         if (st < S::ROWS_D / 2) {
             // rows alternate W3 row k, W1 row k (matmul_silu_ff.comp:96: result1 * result2 / (exp(-result2) + 1))
-            const float r1 = red_row<S::NSD>(red, 2 * st), r2 = red_row<S::NSD>(red, 2 * st + 1);
+            const float r1 = red_row<S::NSD>(red, 2 * st) * inv_d, r2 = red_row<S::NSD>(red, 2 * st + 1) * inv_d;
             st_dev(xc + S::OFF_FF + b * (S::ROWS_D / 2) + st, r1 * r2 / (__expf(-r2) + 1.f));
         }
 
@@ -623,7 +639,7 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
 
     // ================= head: norm + output matrix ====================================================================
     {
-        acquire_vector<D, NW, true, kPollDelay>(xs, x_src, a.norms + (size_t)a.layers * 2 * D, scratch, status, spin_limit);
+        const float inv_h = acquire_vector<D, NW, true, kPollDelay>(xs, x_src, a.norms + (size_t)a.layers * 2 * D, scratch, status, spin_limit);
         load_slab(xr, xsum, xs, mw.sD * 64 + lane, mw.laneD);
         const int rows = (int)mw.vocab_rows, per_set = (rows + S::NRD - 1) / S::NRD;
         // the head's slots are numbered from 0; tiles beyond per_set read the dummy tile
@@ -652,7 +668,7 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
         for (int j = st; j < rows; j += T) {
             const uint32_t n = (uint32_t)b * rows + j;
             if (n < a.vocab) {
-                const float v = red_row<S::NSD>(red, j);
+                const float v = red_row<S::NSD>(red, j) * inv_h;
                 a.logits[n] = v;
                 if (better(v, n, bv, bi)) { bv = v; bi = n; }
             }
