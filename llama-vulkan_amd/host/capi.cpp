@@ -2,6 +2,7 @@
 // Not a second interface: every function forwards to one public method of ggml_file / llava_context /
 // llava_session and adds nothing.
 #include <cstring>
+#include <exception>
 #include <string>
 #include <thread>
 #include <vector>
@@ -23,7 +24,15 @@ unsigned copy_out(const std::string &s, char *out, unsigned cap)
 extern "C" {
 
 // ---- ggml_file ------------------------------------------------------------------------------------------
-void *llh_file_open(const char *path) { return new ggml_file(path); }
+// null only when the object itself cannot be allocated; a bad file gives an object that is not open
+void *llh_file_open(const char *path)
+{
+    try {
+        return new ggml_file(path);
+    } catch (const std::exception &) {
+        return nullptr;
+    }
+}
 void llh_file_close(void *f) { delete static_cast<ggml_file *>(f); }
 int llh_file_is_open(void *f) { return static_cast<ggml_file *>(f)->is_open(); }
 unsigned llh_file_error(void *f, char *out, unsigned cap) { return copy_out(static_cast<ggml_file *>(f)->error(), out, cap); }
@@ -75,10 +84,25 @@ unsigned llh_file_detokenize(void *f, const unsigned *ids, unsigned n, char *out
 // ---- llava_context ----------------------------------------------------------------------------------------
 void *llh_context_new() { return new llava_context; }
 void llh_context_free(void *c) { delete static_cast<llava_context *>(c); }
-int llh_context_load(void *c, const char *path, int device) { return static_cast<llava_context *>(c)->load_model(path, device) ? 0 : -1; }
+// no C++ exception leaves this file: a load that throws (allocation failure) is a failed load
+int llh_context_load(void *c, const char *path, int device)
+{
+    try {
+        return static_cast<llava_context *>(c)->load_model(path, device) ? 0 : -1;
+    } catch (const std::exception &) {
+        return -1;
+    }
+}
 unsigned llh_context_error(void *c, char *out, unsigned cap) { return copy_out(static_cast<llava_context *>(c)->last_error(), out, cap); }
 int llh_context_run(void *c, int argc, char **argv) { return static_cast<llava_context *>(c)->run(argc, argv); }
-int llh_context_open_file(void *c, const char *path) { return static_cast<llava_context *>(c)->open_model_file(path) ? 0 : -1; }
+int llh_context_open_file(void *c, const char *path)
+{
+    try {
+        return static_cast<llava_context *>(c)->open_model_file(path) ? 0 : -1;
+    } catch (const std::exception &) {
+        return -1;
+    }
+}
 
 // ---- lsrv::llava_server: open() + serve_forever() on a thread of its own ----------------------------------
 struct llh_server {
@@ -130,6 +154,8 @@ unsigned llh_session_save_frame(void *s, const char *p) { return static_cast<uns
 unsigned llh_session_snapshot(void *s, const char *p) { return static_cast<unsigned>(static_cast<llava_session *>(s)->snapshot(p)); }
 unsigned llh_session_restore(void *s, const char *p) { return static_cast<unsigned>(static_cast<llava_session *>(s)->restore(p)); }
 void llh_session_seed(void *s, unsigned seed) { static_cast<llava_session *>(s)->set_sampler_seed(seed); }
+// the lv_session the object drives, for calls of the device library that the class does not wrap
+void *llh_session_device(void *s) { return static_cast<llava_session *>(s)->get_device_session(); }
 unsigned llh_session_backlog(void *s) { return static_cast<llava_session *>(s)->get_backlog_size(); }
 unsigned llh_session_tokens_in_gpu(void *s) { return static_cast<llava_session *>(s)->get_tokens_in_gpu(); }
 unsigned llh_session_logits(void *s, float *out, unsigned cap)

@@ -7,6 +7,7 @@
 #include <algorithm>
 #include <cassert>
 #include <cerrno>
+#include <exception>
 #include <cstring>
 #include <fcntl.h>
 #include <iostream>
@@ -120,7 +121,15 @@ ggml_file::ggml_file(const char *filepath)
         return;
     }
     mapping = static_cast<u8 *>(m);
-    if (!parse() && problem.empty()) fail(std::string("Malformed model file ") + filepath);
+    bool parsed = false;
+    try {
+        parsed = parse();
+    } catch (const std::exception &e) {  // allocation failure on a hostile size field: the object ends closed, like any bad file
+        problem.clear();
+        fail(std::string("Malformed model file ") + filepath + ": " + e.what());
+        return;
+    }
+    if (!parsed && problem.empty()) fail(std::string("Malformed model file ") + filepath);
 }
 
 ggml_file::~ggml_file()
@@ -139,7 +148,9 @@ bool ggml_file::parse()
     if (!header.vocab_size || !header.n_heads || !header.n_layers || header.rot * header.n_heads != header.dim)
         return fail("Inconsistent model header"), false;
 
-    // vocabulary: i32 length, bytes, f32 score
+    // vocabulary: i32 length, bytes, f32 score.  A record is at least 8 bytes, so a count the rest of the file cannot
+    // hold is refused before anything is sized by it.
+    if (header.vocab_size > (mapping_size - cur.at()) / 8) return fail("Vocabulary size " + std::to_string(header.vocab_size) + " exceeds the file"), false;
     tokens.reserve(header.vocab_size);
     for (u32 id = 0; id < header.vocab_size; ++id) {
         u32 len;

@@ -140,10 +140,7 @@ bool llava_session::set_backlog_size(u32 new_size)
     if (new_size > kMaxBacklog) return false;
     if (new_size == backlog_size) return true;
     if (new_size < kMinBacklog || new_size < current_tokens_in_gpu) return false;
-    if (step_in_flight) {
-        (void)lv_step_wait(device_session);
-        step_in_flight = false;
-    }
+    settle_step();
     if (lv_session_reserve(device_session, new_size) != LV_OK) {
         std::cerr << "set_backlog_size: " << lv_last_error() << std::endl;
         return false;
@@ -166,6 +163,9 @@ bool llava_session::set_text(const std::string &new_text)
     if (wanted > kMaxBacklog || !set_backlog_size(wanted)) return false;
     u32 keep = 0;
     while (keep < fresh.size() && keep < token_buffer.size() && keep < current_tokens_in_gpu && token_buffer[keep] == fresh[keep]) ++keep;
+    // the last token of the new text is always evaluated again: the logits on the device then belong to this text, also
+    // when it is a prefix of what was evaluated before (the reference re-evaluates in that case too)
+    if (!fresh.empty() && keep == fresh.size()) --keep;
     token_buffer = std::move(fresh);
     current_tokens_in_gpu = keep;
     return true;
@@ -205,6 +205,7 @@ void llava_session::rewind(u32 n)
 bool llava_session::start_next_token_prediction()
 {
     if (!good()) return false;
+    settle_step();  // a caller that starts twice without finishing: the reference would hit its fence too
     const u32 to_process = static_cast<u32>(token_buffer.size()) - current_tokens_in_gpu;
     if (to_process == 0) {
         std::cerr << "GPU is already in sync" << std::endl;
@@ -213,10 +214,6 @@ bool llava_session::start_next_token_prediction()
     if (token_buffer.size() > backlog_size) {
         std::cerr << "Token buffer overflow" << std::endl;
         return false;
-    }
-    if (step_in_flight) {  // a caller that starts twice without finishing: the reference would hit its fence too
-        (void)lv_step_wait(device_session);
-        step_in_flight = false;
     }
     if (batch_size != to_process) {
         batch_size = to_process;
@@ -227,8 +224,28 @@ bool llava_session::start_next_token_prediction()
         return false;
     }
     step_in_flight = true;
+    step_first_row = current_tokens_in_gpu;
     current_tokens_in_gpu += to_process;
     return true;
+}
+
+// The rows a step writes count as evaluated from the moment it is submitted.  When the step turns out to have failed
+// (the device reports an error at the wait), they hold nothing usable: count them as pending again, so that the next
+// start evaluates the same tokens into the same rows.
+void llava_session::step_failed()
+{
+    current_tokens_in_gpu = std::min(current_tokens_in_gpu, step_first_row);
+}
+
+// waits for a step that was started and never finished; false when that step failed
+bool llava_session::settle_step()
+{
+    if (!step_in_flight) return true;
+    step_in_flight = false;
+    if (lv_step_wait(device_session) == LV_OK) return true;
+    std::cerr << "step failed: " << lv_last_error() << std::endl;
+    step_failed();
+    return false;
 }
 
 // llava_session.cpp:231-234; the reference always samples stochastically here
@@ -251,9 +268,11 @@ u32 llava_session::get_last_predicted_token(bool deterministic)
     const u32 n_vocab = model->get_header().vocab_size;
     last_logits.resize(n_vocab);
     const int rc = lv_logits_read(device_session, last_logits.data());  // waits for the step
+    const bool was_in_flight = step_in_flight;
     step_in_flight = false;
     if (rc != LV_OK) {
         std::cerr << "finish_next_token_prediction: " << lv_last_error() << std::endl;
+        if (was_in_flight) step_failed();
         return ~0u;
     }
     std::vector<float> p(last_logits);
@@ -348,10 +367,7 @@ ReturnCode llava_session::set_options(u32 new_options)
 {
     if (options == new_options) return ReturnCode::ok;
     if (!good()) return ReturnCode::nok;
-    if (step_in_flight) {
-        (void)lv_step_wait(device_session);
-        step_in_flight = false;
-    }
+    settle_step();
     if (lv_trace_enable(device_session, new_options != 0) != LV_OK) return ReturnCode::nok;
     options = new_options;
     return ReturnCode::ok;
@@ -378,10 +394,7 @@ ReturnCode llava_session::save_frame(const std::string &path)
 ReturnCode llava_session::snapshot(const std::string &path)
 {
     if (!good()) return ReturnCode::nok;
-    if (step_in_flight) {
-        (void)lv_step_wait(device_session);
-        step_in_flight = false;
-    }
+    settle_step();
     const u32 n = current_tokens_in_gpu, dim = model->get_header().dim;
     const std::size_t per_layer = static_cast<std::size_t>(2) * n * dim * 2;
     const std::size_t total = layer_data.size() * per_layer + 4 * static_cast<std::size_t>(n) + 4;
@@ -462,10 +475,7 @@ ReturnCode llava_session::restore(const std::string &path)
         }
     u32 needed = kMinBacklog;
     while (needed < n) needed <<= 1;
-    if (step_in_flight) {
-        (void)lv_step_wait(device_session);
-        step_in_flight = false;
-    }
+    settle_step();
     rewind(0);
     if (!set_backlog_size(needed)) {
         std::cerr << "Cannot set backlog size" << std::endl;

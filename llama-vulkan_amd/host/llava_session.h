@@ -70,6 +70,8 @@ private:
     [[nodiscard]] u32 get_last_predicted_token(bool deterministic);
     [[nodiscard]] bool set_backlog_size(u32 new_size);
     void recreate_spevars();
+    void step_failed();
+    bool settle_step();
 
     // sampler state and constants (llava_session.h:68-77)
     std::mt19937 rng;
@@ -86,5 +88,6 @@ private:
     u32 batch_size = 0;
     u32 options = 0;
     bool step_in_flight = false;
+    u32 step_first_row = 0;  // first cache row of the step that was started last
     specialization_variables_t specialization_variables{};
 };

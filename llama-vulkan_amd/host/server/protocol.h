@@ -62,8 +62,9 @@ struct tlv_header {
 };
 static_assert(sizeof(tlv_header) == 12, "three packed words");
 
-constexpr u32 kMaxPacketLength = 0x10000;   // a longer packet marks the client as broken (server/client.cpp:129-133)
+constexpr u32 kMaxPacketLength = 0x10000;   // a longer packet ends the connection (the reference marks the client failed: server/client.cpp:129-133)
 constexpr u32 kMaxInputBuffer = 0x20000;    // unread input kept per client
+constexpr u32 kMaxOutputBuffer = 16u << 20; // replies a client may leave unread before it is dropped
 
 inline void put_u32(std::vector<u8> &out, u32 v)
 {

@@ -28,7 +28,7 @@ struct llava_server::client {
     std::vector<u8> input;
     std::vector<u8> output;
     size_t sent = 0;            // prefix of `output` already written to the socket
-    bool broken = false;        // protocol violation: nothing more is parsed
+    bool overflowed = false;    // more output queued than a client may leave unread: dropped at the next write pass
     ~client() { if (fd >= 0) ::close(fd); }
 };
 
@@ -125,6 +125,12 @@ void llava_server::notify_session_death(u32 session_id)
 
 void llava_server::send_to(client &c, OutCommands kind, u32 reply_to, const std::vector<u8> &payload)
 {
+    if (c.overflowed) return;
+    if (c.output.size() - c.sent + sizeof(tlv_header) + payload.size() > kMaxOutputBuffer) {
+        std::cerr << "[!] client " << c.id << " does not read its replies, dropping it" << std::endl;
+        c.overflowed = true;
+        return;
+    }
     put_u32(c.output, kind);
     put_u32(c.output, reply_to);
     put_u32(c.output, static_cast<u32>(payload.size()));
@@ -242,13 +248,14 @@ bool llava_server::service_client(client &c, short revents)
             }
         }
         size_t at = 0;
-        while (!c.broken && c.input.size() - at >= sizeof(tlv_header)) {
+        while (c.input.size() - at >= sizeof(tlv_header)) {
             const u8 *p = c.input.data() + at;
             const tlv_header h = {get_u32(p), get_u32(p + 4), get_u32(p + 8)};
             if (h.length > kMaxPacketLength) {
-                std::cerr << "[!] client " << c.id << ": packet of " << h.length << " bytes, ignoring the connection from here on" << std::endl;
-                c.broken = true;
-                break;
+                // the reference stops parsing such a client and keeps its socket (server/client.cpp:129-133); unread input
+                // would then keep the poll loop spinning, so the connection is closed instead
+                std::cerr << "[!] client " << c.id << ": packet of " << h.length << " bytes, closing the connection" << std::endl;
+                return false;
             }
             if (c.input.size() - at < sizeof(tlv_header) + h.length) break;
             handle_packet(c, h, p + sizeof(tlv_header));
@@ -375,6 +382,10 @@ bool llava_server::serve_forever()
         to_drop.clear();
         for (auto &entry : clients) {
             client &c = *entry.second;
+            if (c.overflowed) {
+                to_drop.push_back(c.id);
+                continue;
+            }
             while (c.sent < c.output.size()) {
                 const ssize_t n = send(c.fd, c.output.data() + c.sent, c.output.size() - c.sent, MSG_NOSIGNAL);
                 if (n > 0) {

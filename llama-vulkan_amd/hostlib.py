@@ -39,7 +39,7 @@ def lib():
             "llh_session_start": (C.c_int, [vp]), "llh_session_finish": (u, [vp, C.c_int]), "llh_session_predict": (u, [vp, C.c_int]),
             "llh_session_rewind": (None, [vp, u]), "llh_session_set_options": (u, [vp, u]), "llh_session_is_tracing": (C.c_int, [vp]),
             "llh_session_save_frame": (u, [vp, cp]), "llh_session_snapshot": (u, [vp, cp]), "llh_session_restore": (u, [vp, cp]),
-            "llh_session_seed": (None, [vp, u]), "llh_session_backlog": (u, [vp]), "llh_session_tokens_in_gpu": (u, [vp]),
+            "llh_session_seed": (None, [vp, u]), "llh_session_backlog": (u, [vp]), "llh_session_device": (vp, [vp]), "llh_session_tokens_in_gpu": (u, [vp]),
             "llh_session_logits": (u, [vp, C.c_void_p, u]), "llh_session_spevars": (None, [vp, C.POINTER(u)]), "llh_session_layer_count": (u, [vp]),
         }
         for name, (res, args) in sig.items():
@@ -195,6 +195,10 @@ class LlavaSession:
 
     def rewind(self, n):
         lib().llh_session_rewind(self.h, n)
+
+    def device_session(self):
+        """the lv_session handle (an integer address) behind this object"""
+        return lib().llh_session_device(self.h)
 
     def set_options(self, o):
         return lib().llh_session_set_options(self.h, o)

@@ -94,6 +94,71 @@ def test_set_text_reuses_the_common_prefix_and_rewind_drops_the_tail(hl, orc, lo
     s.close()
 
 
+def test_text_that_is_a_prefix_of_the_evaluated_context_is_evaluated_again(hl, orc, loaded):
+    """set_text with the same prompt, and with a shorter prompt that is a prefix of it: all rows could be reused, but the
+    logits on the device belong to the longer context, so the last token is evaluated again (the reference re-evaluates
+    here: llava_session.cpp:257-277 finds no reusable prefix) and predict answers for the new text"""
+    c, f, path = loaded
+    s = hl.LlavaSession(c)
+    long_text, short_text = PROMPT + b" jumps over", PROMPT
+    a, b = f.tokenize(long_text, True), f.tokenize(short_text, True)
+    assert a[:len(b)] == b and len(b) < len(a)
+    assert s.set_text(long_text)
+    first = s.predict(True)
+    assert s.tokens_in_gpu() == len(a)
+    assert s.set_text(long_text)                # the same text once more
+    assert s.tokens_in_gpu() == len(a) - 1
+    assert s.predict(True) == first
+    assert s.set_text(short_text)               # a strict prefix of what the cache holds
+    assert s.tokens_in_gpu() == len(b) - 1
+    want, rows = oracle_greedy(orc, path, b, 1)
+    assert s.predict(True) == want[0]
+    assert np.max(np.abs(s.logits() - rows[0])) <= 1e-2 + 1e-3 * np.max(np.abs(rows[0]))
+    assert s.add_text(b"")                      # appends nothing: still answers, for the same text
+    assert s.predict(True) == want[0]
+    s.close()
+
+
+def test_a_failed_step_is_evaluated_again_by_the_next_start(hl, lva, orc, tmp_path):
+    """failure path at the level of llava_session: the persistent kernel's poll bound set to 1 makes its workgroups stop
+    waiting for each other at once (every kernel still runs to its end), finish reports the failure as ~0, and the rows of
+    that step count as pending again: the next predict evaluates the same token into the same row and gives the oracle's
+    token.  Without that the session would refuse ('GPU is already in sync') and go on over rows that hold nothing."""
+    p = str(tmp_path / "wide.ggml")
+    lva.write_model(p, wtype=lva.LV_Q4_0, seed=9, vocab=2048, layers=2, dim=4096, heads=32, ff=11008)
+    c = hl.LlavaContext()
+    assert c.load_model(p), c.error()
+    s = hl.LlavaSession(c)
+    import ctypes
+    dev, path_now = s.device_session(), ctypes.c_int()
+    assert lva.hip().lv_session_path(dev, ctypes.byref(path_now)) == 0 and path_now.value == lva.PATH_PERSISTENT
+    prompt = [int(t) for t in lva.synth_tokens(4, 3, 2048, seed=3)]
+    want, rows = oracle_greedy(orc, p, prompt, 2)
+    for t in prompt:
+        assert s.push_token(t)
+    assert s.predict(True) == want[0]
+    assert s.push_token(want[0])
+    assert lva.hip().lv_session_set_wait_limit(dev, 1) == 0
+    assert s.start()
+    assert s.tokens_in_gpu() == 5
+    assert s.finish(True) == 0xFFFFFFFF
+    assert s.tokens_in_gpu() == 4               # the failed row is pending again
+    assert lva.hip().lv_session_set_wait_limit(dev, 0) == 0
+    assert s.predict(True) == want[1]
+    assert np.max(np.abs(s.logits() - rows[1])) <= 1e-2 + 1e-3 * np.max(np.abs(rows[1]))
+    # a failed step that is never finished (started, then another start) is settled and repeated the same way
+    assert s.push_token(want[1])
+    assert lva.hip().lv_session_set_wait_limit(dev, 1) == 0
+    assert s.start()
+    assert lva.hip().lv_session_set_wait_limit(dev, 0) == 0
+    assert s.start() and s.tokens_in_gpu() == 6
+    third = s.finish(True)
+    more, _ = oracle_greedy(orc, p, prompt, 3)
+    assert third == more[2]
+    s.close()
+    c.close()
+
+
 def test_add_text_appends_through_the_detokenised_text(hl, loaded):
     c, f, _ = loaded
     s = hl.LlavaSession(c)

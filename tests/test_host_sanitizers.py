@@ -40,6 +40,7 @@ def test_parser_and_tokenizer_under_sanitizers(driver, tmp_path):
     where = gb.build(good, vocab, gb.minimal_tensors(vocab=len(vocab)))
     data = np.fromfile(good, dtype=np.uint8)
     first_tensor = min(off for off, _ in where.values())
+    first_record = 36 + sum(8 + len(piece) for piece, _ in vocab)   # the first tensor record follows the vocabulary
     paths = [good]
     # truncations: inside the header, inside the vocabulary, inside a tensor record, inside a payload, one byte short
     cuts = [0, 1, 35, 36, 40, 200, first_tensor - 40, first_tensor - 1, first_tensor, first_tensor + 100, len(data) // 2, len(data) - 1]
@@ -64,6 +65,16 @@ def test_parser_and_tokenizer_under_sanitizers(driver, tmp_path):
         p = str(tmp_path / f"mut_{k}.ggml")
         mutated.tofile(p)
         paths.append(p)
+    # size fields far beyond the file: a 100-byte file whose header claims 2^31-1 or 2^32-1 tokens, the full file with the
+    # same claim, a first token and a first tensor name of such a length.  None may be sized by the claim before it is checked.
+    for k, value in enumerate([0x7FFFFFFF, 0xFFFFFFFF, 0x10000000]):
+        word = np.frombuffer(np.uint32(value).tobytes(), dtype=np.uint8)
+        for label, base, at in [("vocab_short", data[:100], 8), ("vocab_full", data, 8), ("toklen", data, 36), ("namelen", data, first_record + 4)]:
+            mutated = base.copy()
+            mutated[at:at + 4] = word
+            p = str(tmp_path / f"huge_{label}_{k}.ggml")
+            mutated.tofile(p)
+            paths.append(p)
     r = run(driver, paths)
     assert r.returncode == 0, (r.stdout[-500:], r.stderr[-3000:])
     assert "opened" in r.stdout

@@ -96,15 +96,49 @@ def test_framing_split_and_merged_packets(served):
     c.close()
 
 
-def test_oversized_packet_silences_that_client_only(served):
+def test_oversized_packet_ends_that_connection_only(served):
+    """a length field above 0x10000 is a protocol violation (server/client.cpp:129-133 stops parsing that client); here the
+    connection is closed, so that its unread input cannot keep the poll loop busy, and other clients are served as before"""
     server, _ = served
-    bad, good = sc.Client(server.port, timeout=1.0), sc.Client(server.port)
+    bad, good = sc.Client(server.port, timeout=5.0), sc.Client(server.port)
     bad.send_raw(struct.pack("<3I", sc.ADD_TEXT, 1, 0x10001))
-    bad.send_raw(struct.pack("<3I", sc.LIST_SESSIONS, 2, 0))
-    with pytest.raises(socket.timeout):
+    with pytest.raises((ConnectionError, OSError)):
+        bad.send_raw(struct.pack("<3I", sc.LIST_SESSIONS, 2, 0) + b"x" * 0x30000)   # more than the input buffer holds
         bad.read_packet()
     assert good.sessions() == []
     bad.close(); good.close()
+
+
+def test_client_that_never_reads_is_dropped_when_its_replies_pile_up(served):
+    """each token map request queues a reply; a client that keeps asking and never reads is dropped once 16 MiB wait for it,
+    and the server keeps answering others"""
+    server, vocab = served
+    greedy, good = sc.Client(server.port, timeout=5.0), sc.Client(server.port)
+    kind, payload = good.call(sc.GET_TOKEN_MAP)
+    per_reply = 12 + len(payload)
+    wanted = (16 << 20) // per_reply + 64
+    request = struct.pack("<3I", sc.GET_TOKEN_MAP, 7, 0)
+    greedy.sock.settimeout(20.0)
+    dropped = False
+    try:
+        for start in range(0, wanted * 4, 256):               # far more requests than the cap allows replies for
+            greedy.send_raw(request * 256)
+    except (ConnectionError, OSError):
+        dropped = True
+    if not dropped:                                           # everything was accepted into socket buffers: the close shows on read
+        time.sleep(1.5)                                       # the replies pile up while nobody reads
+        total = 0
+        try:
+            while True:
+                chunk = greedy.sock.recv(1 << 20)
+                if not chunk:
+                    break
+                total += len(chunk)
+        except (ConnectionError, OSError):
+            pass
+        assert total < wanted * 4 * per_reply                 # not every request was answered: the connection ended first
+    assert good.sessions() == []
+    greedy.close(); good.close()
 
 
 def test_stop_with_live_sessions_and_clients(hl, tmp_path):
