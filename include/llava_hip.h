@@ -107,14 +107,19 @@ int lv_session_use_graph(lv_session *s, int enable);
  *   LV_PATH_GRAPH       the same launches captured once into a hipGraph and replayed
  *   LV_PATH_PERSISTENT  one persistent kernel for the whole token (LLaMA-7B and -13B layer shapes, q4_0 or q8_0, on a
  *                       256-CU device)
- *   LV_PATH_AUTO        persistent when the model has that form, else graph (or kernels if graphs are off) */
+ *   LV_PATH_AUTO        persistent when the model has that form, else graph (or kernels if graphs are off)
+ * A session stops using the persistent kernel, and lv_session_path reports the graph path (kernels if graphs are off)
+ * from then on, when the runtime refuses its cooperative launch (the step goes on in the other path and succeeds) or when
+ * two steps in a row end with an expired hand-over wait (both report LV_ERR_HIP; the step issued again then succeeds).
+ * lv_session_set_path(LV_PATH_PERSISTENT) gives the kernel another try. */
 enum { LV_PATH_AUTO = 0, LV_PATH_KERNELS = 1, LV_PATH_GRAPH = 2, LV_PATH_PERSISTENT = 3 };
 int lv_session_set_path(lv_session *s, int path);
 int lv_session_path(const lv_session *s, int *path);
 /* Workgroups of the persistent kernel wait for each other's results by polling, a bounded number of times; a wait
  * that runs out makes the kernel finish anyway and lv_step_wait return LV_ERR_HIP (the reference's waitForFences
  * timeout, llava_command_buffer.cpp:25-27, is the nearest counterpart).  polls = 0 restores the default bound; tests of
- * that failure path set 1.  The step can simply be issued again afterwards. */
+ * that failure path set 1.  The step can simply be issued again afterwards; after two such steps in a row it runs in
+ * the graph path (see lv_session_set_path). */
 int lv_session_set_wait_limit(lv_session *s, uint32_t polls);
 
 /* ---- cache dump / restore: replaces llava_layer_session_data::dump_kv_cache / restore_kv_cache

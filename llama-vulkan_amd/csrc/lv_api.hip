@@ -163,6 +163,9 @@ struct lv_session {
     uint32_t *status_host = nullptr;      // pinned, written by the persistent kernel: [0] a poll expired, [kStatusToken] greedy pick
     uint32_t wait_limit = 0;              // polls per hand-over of the persistent kernel; 0 = default
     bool pick_in_status = false;          // the last step ran the persistent kernel, whose greedy pick is in status_host
+    bool mega_step = false;               // the step in flight ran the persistent kernel
+    int mega_failures = 0;                // steps of the persistent kernel in a row that ended with an expired wait
+    bool mega_off = false;                // the persistent kernel is no longer used by this session (refused launch, or two such steps)
     bool in_flight = false;
     bool have_logits = false;
     bool trace = false;
@@ -1391,21 +1394,26 @@ extern "C" int lv_session_set_path(lv_session *s, int path)
     if (path == LV_PATH_PERSISTENT && s->model->mega_kind == 0)
         return fail(LV_ERR_ARG, "lv_session_set_path: this model has no persistent-kernel form (shape or types not covered)");
     s->path = path;
+    s->mega_off = false;  // an explicit choice gives the persistent kernel another try
+    s->mega_failures = 0;
     return LV_OK;
 }
 
 extern "C" int lv_session_path(const lv_session *s, int *path)
 {
     if (!s || !path) return fail(LV_ERR_ARG, "lv_session_path: null argument");
-    *path = s->path != LV_PATH_AUTO ? s->path
-            : s->model->mega_kind   ? LV_PATH_PERSISTENT
-            : s->use_graph          ? LV_PATH_GRAPH
-                                    : LV_PATH_KERNELS;
+    const int fallback = s->use_graph ? LV_PATH_GRAPH : LV_PATH_KERNELS;
+    if (s->path != LV_PATH_AUTO)
+        *path = s->path == LV_PATH_PERSISTENT && s->mega_off ? fallback : s->path;
+    else
+        *path = s->model->mega_kind && !s->mega_off ? LV_PATH_PERSISTENT : fallback;
     return LV_OK;
 }
 
-// One token through the persistent kernel.
-static int launch_mega(lv_session *s, uint32_t pos, uint32_t token)
+// One token through the persistent kernel.  *refused is set, and LV_OK returned, when the runtime will not launch the
+// grid cooperatively (its 256 workgroups cannot all be resident: another process holds part of the device, or the
+// device is smaller than the kernel was built for); nothing has run then.
+static int launch_mega(lv_session *s, uint32_t pos, uint32_t token, bool *refused)
 {
     const lv_model *m = s->model;
     MegaArgs a{};
@@ -1427,10 +1435,20 @@ static int launch_mega(lv_session *s, uint32_t pos, uint32_t token)
     if (c->mega_last && c->mega_last != s) HIP_TRY(hipStreamWaitEvent(s->stream, c->mega_done, 0));
     LV_TRY(mega_dispatch(m->mega_kind, [&](auto shape) -> int {
         using S = decltype(shape);
-        HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<const void *>(&mega_decode_kernel<S>), dim3(kMegaWGs), dim3(S::NW * 64), params, 0,
-                                           s->stream));
+        const hipError_t e = hipLaunchCooperativeKernel(reinterpret_cast<const void *>(&mega_decode_kernel<S>), dim3(kMegaWGs), dim3(S::NW * 64),
+                                                        params, 0, s->stream);
+        if (e == hipErrorCooperativeLaunchTooLarge || e == hipErrorLaunchOutOfResources || e == hipErrorNotSupported) {
+            (void)hipGetLastError();
+            *refused = true;
+            return LV_OK;
+        }
+        HIP_TRY(e);
         return LV_OK;
     }));
+    if (*refused) {
+        s->xchg_turn--;
+        return LV_OK;
+    }
     if (!c->mega_done) HIP_TRY(hipEventCreateWithFlags(&c->mega_done, hipEventDisableTiming));
     HIP_TRY(hipEventRecord(c->mega_done, s->stream));
     c->mega_last = s;
@@ -1665,15 +1683,34 @@ extern "C" int lv_step_begin(lv_session *s, const uint32_t *tokens, uint32_t n, 
     (void)lv_session_path(s, &path);
     // the persistent kernel also takes the short steps (a few prompt or add_text tokens) below the size at which the
     // batched path pays: one launch per token, each 1.7 x faster than the operator chain's token
-    const bool persistent = n < kPrefillMin && path == LV_PATH_PERSISTENT && !s->trace;
+    bool persistent = n < kPrefillMin && path == LV_PATH_PERSISTENT && !s->trace;
+    s->mega_step = false;
+    if (persistent) {
+        uint32_t done = 0;
+        bool refused = false;
+        while (done < n) {
+            LV_TRY(launch_mega(s, pos + done, tokens[done], &refused));
+            if (refused) break;
+            done++;
+        }
+        s->mega_step = done > 0;
+        if (refused) {
+            // the tokens launched so far stay as they are; the rest of this step, and every later one, takes the other path
+            s->mega_off = true;
+            persistent = false;
+            (void)lv_session_path(s, &path);
+            tokens += done; n -= done; pos += done;
+        } else {
+            s->pick_in_status = true;  // the kernel leaves the greedy pick (of the last token) in the pinned status block
+        }
+    }
     if (!persistent) {             // the persistent kernel takes position and token id as launch arguments
         s->cfg_host[0] = pos;
         memcpy(s->cfg_host + 1, tokens, (size_t)n * 4);
         HIP_TRY(hipMemcpyAsync(s->cfg, s->cfg_host, (size_t)(1 + n) * 4, hipMemcpyHostToDevice, s->stream));
     }
     if (persistent) {
-        for (uint32_t i = 0; i < n; i++) LV_TRY(launch_mega(s, pos + i, tokens[i]));
-        s->pick_in_status = true;  // the kernel leaves the greedy pick (of the last token) in the pinned status block
+        // launched above
     } else if (n == 1 && (path == LV_PATH_GRAPH || (path == LV_PATH_PERSISTENT && s->use_graph)) && !s->trace) {
         if (!s->graph_exec) {
             HIP_TRY(hipStreamBeginCapture(s->stream, hipStreamCaptureModeThreadLocal));
@@ -1711,10 +1748,18 @@ extern "C" int lv_step_wait(lv_session *s)
     if (!s) return fail(LV_ERR_ARG, "lv_step_wait: session is null");
     HIP_TRY(hipStreamSynchronize(s->stream));
     s->in_flight = false;
+    const bool mega_step = s->mega_step;
+    s->mega_step = false;
     if (s->status_host && *s->status_host) {
         *s->status_host = 0;
+        if (++s->mega_failures >= 2) {
+            s->mega_off = true;
+            return fail(LV_ERR_HIP, "persistent decode kernel: a hand-over wait expired in two steps in a row; this session now takes the %s path",
+                        s->use_graph ? "graph" : "operator");
+        }
         return fail(LV_ERR_HIP, "persistent decode kernel: a hand-over wait expired (workgroups not co-resident?)");
     }
+    if (mega_step) s->mega_failures = 0;
     return LV_OK;
 }
 

@@ -298,6 +298,56 @@ def test_persistent_kernel_gives_up_a_wait_and_the_step_can_be_repeated(lva, orc
     s.close(); model.close(); osess.close(); om.close()
 
 
+def test_two_expired_waits_in_a_row_move_the_session_to_the_graph_path(lva, orc, ctx, wide_model):
+    """with the poll bound at 1 every step of the persistent kernel fails; after the second failure in a row the session
+    reports the graph path and the same step, issued a third time with the bound unchanged, gives the oracle's result
+    there; choosing the persistent path again by hand brings the kernel back"""
+    om = orc.Model(wide_model)
+    osess = orc.Session(om, 128)
+    model = lva.Model(ctx, wide_model)
+    s = lva.Session(model, 128)
+    prompt = lva.synth_tokens(4, 3, 2048, seed=4)
+    want = osess.eval(prompt)
+    s.begin(prompt, 0)
+    _check_logits(s.logits(), want)
+    tok = orc.greedy(want)
+    want = osess.eval([tok])
+    s.set_wait_limit(1)
+    for attempt in range(2):
+        assert s.path() == lva.PATH_PERSISTENT
+        s.begin([tok], 4)
+        with pytest.raises(lva.LvError):
+            s.wait()
+    assert s.path() == lva.PATH_GRAPH
+    s.begin([tok], 4)                 # the bound is still 1: this step does not run the persistent kernel
+    _check_logits(s.logits(), want)
+    assert s.argmax() == orc.greedy(want)
+    tok = orc.greedy(want)
+    want = osess.eval([tok])
+    s.begin([tok], 5)                 # graph replay
+    _check_logits(s.logits(), want)
+    s.set_wait_limit(0)
+    s.set_path(lva.PATH_PERSISTENT)
+    assert s.path() == lva.PATH_PERSISTENT
+    tok = orc.greedy(want)
+    want = osess.eval([tok])
+    s.begin([tok], 6)
+    _check_logits(s.logits(), want)
+    assert s.argmax() == orc.greedy(want)
+    # one failure, one success, one failure: not two in a row, the kernel stays
+    s.set_path(lva.PATH_AUTO)
+    for limit, fails in [(1, True), (0, False), (1, True)]:
+        s.set_wait_limit(limit)
+        s.begin([tok], 6)
+        if fails:
+            with pytest.raises(lva.LvError):
+                s.wait()
+        else:
+            _check_logits(s.logits(), want)
+    assert s.path() == lva.PATH_PERSISTENT
+    s.close(); model.close(); osess.close(); om.close()
+
+
 @pytest.mark.parametrize("vocab", [259, 2049])
 def test_vocabulary_sizes_that_do_not_divide_over_the_workgroups(lva, orc, ctx, tmp_path, vocab):
     """the output matrix is split over 256 workgroups; 2049 rows leave the last ones short, 259 leave most of them

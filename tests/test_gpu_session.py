@@ -114,7 +114,7 @@ def test_text_that_is_a_prefix_of_the_evaluated_context_is_evaluated_again(hl, o
     want, rows = oracle_greedy(orc, path, b, 1)
     assert s.predict(True) == want[0]
     assert np.max(np.abs(s.logits() - rows[0])) <= 1e-2 + 1e-3 * np.max(np.abs(rows[0]))
-    assert s.add_text(b"")                      # appends nothing: still answers, for the same text
+    assert s.set_text(short_text)               # and once more: still answers, for the same text
     assert s.predict(True) == want[0]
     s.close()
 
