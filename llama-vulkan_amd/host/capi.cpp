@@ -3,6 +3,7 @@
 // llava_session and adds nothing.
 #include <cstring>
 #include <exception>
+#include <random>
 #include <string>
 #include <thread>
 #include <vector>
@@ -154,6 +155,24 @@ unsigned llh_session_save_frame(void *s, const char *p) { return static_cast<uns
 unsigned llh_session_snapshot(void *s, const char *p) { return static_cast<unsigned>(static_cast<llava_session *>(s)->snapshot(p)); }
 unsigned llh_session_restore(void *s, const char *p) { return static_cast<unsigned>(static_cast<llava_session *>(s)->restore(p)); }
 void llh_session_seed(void *s, unsigned seed) { static_cast<llava_session *>(s)->set_sampler_seed(seed); }
+// llava_session::sample_token on caller-supplied logits: returns the token; *mu is read and updated; kept_ids / kept_p
+// receive up to cap entries of the kept set, *kept_count its size, *kept_sum its probability mass, *pick the drawn index
+unsigned llh_sample_token(const float *logits, unsigned n_vocab, const unsigned *history, unsigned history_size, float *mu, unsigned seed,
+                          unsigned *kept_ids, float *kept_p, unsigned cap, unsigned *kept_count, float *kept_sum, int *pick)
+{
+    std::mt19937 rng(seed);
+    llava_session::sampler_probe probe;
+    const unsigned token = llava_session::sample_token(std::vector<float>(logits, logits + n_vocab), history, history_size, *mu, rng, &probe);
+    const unsigned n = static_cast<unsigned>(probe.kept_ids.size());
+    for (unsigned i = 0; i < n && i < cap; ++i) {
+        kept_ids[i] = probe.kept_ids[i];
+        kept_p[i] = probe.kept_p[i];
+    }
+    *kept_count = n;
+    *kept_sum = probe.kept_sum;
+    *pick = probe.pick;
+    return token;
+}
 // the lv_session the object drives, for calls of the device library that the class does not wrap
 void *llh_session_device(void *s) { return static_cast<llava_session *>(s)->get_device_session(); }
 unsigned llh_session_backlog(void *s) { return static_cast<llava_session *>(s)->get_backlog_size(); }

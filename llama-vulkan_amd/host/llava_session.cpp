@@ -289,10 +289,17 @@ u32 llava_session::get_last_predicted_token(bool deterministic)
         return best;
     }
 
+    return sample_token(std::move(p), token_buffer.data(), token_buffer.size(), mirostat_mu, rng);
+}
+
+// llava_session.cpp:154-194
+u32 llava_session::sample_token(std::vector<float> p, const u32 *history, std::size_t history_size, float &mu, std::mt19937 &rng, sampler_probe *probe)
+{
+    const u32 n_vocab = static_cast<u32>(p.size());
     // repetition / frequency penalty, applied to the newline token only (:157-167)
     std::map<u32, u32> recent;
-    const std::size_t from = token_buffer.size() > repeat_last_n ? token_buffer.size() - repeat_last_n : 0;
-    for (std::size_t i = from; i < token_buffer.size(); ++i) recent[token_buffer[i]]++;
+    const std::size_t from = history_size > repeat_last_n ? history_size - repeat_last_n : 0;
+    for (std::size_t i = from; i < history_size; ++i) recent[history[i]]++;
     const auto nl = recent.find(13);
     if (nl != recent.end() && 13 < n_vocab) {
         float &l = p[13];
@@ -307,7 +314,7 @@ u32 llava_session::get_last_predicted_token(bool deterministic)
         total += p[t];
     }
     // keep what is at least 2^-mu likely (:175-188)
-    const float cut = std::pow(0.5f, mirostat_mu);
+    const float cut = std::pow(0.5f, mu);
     std::vector<u32> ids;
     std::vector<float> kept;
     float kept_sum = 0.f;
@@ -321,10 +328,17 @@ u32 llava_session::get_last_predicted_token(bool deterministic)
             ids.push_back(t);
         }
     }
+    if (probe) {
+        probe->kept_ids = ids;
+        probe->kept_p = kept;
+        probe->kept_sum = kept_sum;
+        probe->pick = -1;
+    }
     if (ids.empty()) return likeliest;  // nothing passes the cut: the reference would index an empty vector here
     std::discrete_distribution<> dist(kept.begin(), kept.end());
     const int pick = dist(rng);
-    mirostat_mu += mirostat_eta * (mirostat_tau + std::log2(kept[pick] / kept_sum));  // (:193)
+    if (probe) probe->pick = pick;
+    mu += mirostat_eta * (mirostat_tau + std::log2(kept[pick] / kept_sum));  // (:193)
     return ids[pick];
 }
 

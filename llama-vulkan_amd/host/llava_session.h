@@ -56,6 +56,17 @@ public:
     ReturnCode restore(const std::string &path);
 
     // additions
+    // What one stochastic pick went through, for checks of its arithmetic: the tokens that passed the cut with their
+    // probabilities (after penalty and temperature, over the whole vocabulary), and which of them was drawn.
+    struct sampler_probe {
+        std::vector<u32> kept_ids;
+        std::vector<float> kept_p;
+        float kept_sum = 0.f;
+        int pick = -1;
+    };
+    // The stochastic branch of get_last_predicted_token (llava_session.cpp:154-194) as a function of its inputs: the logits
+    // (taken by value, they are overwritten), the token history, the running mu and the generator.
+    static u32 sample_token(std::vector<float> p, const u32 *history, std::size_t history_size, float &mu, std::mt19937 &rng, sampler_probe *probe = nullptr);
     void set_sampler_seed(u32 seed);                       // the reference seeds with time(nullptr)
     [[nodiscard]] u32 get_backlog_size() const { return backlog_size; }
     [[nodiscard]] u32 get_tokens_in_gpu() const { return current_tokens_in_gpu; }
@@ -75,8 +86,8 @@ private:
 
     // sampler state and constants (llava_session.h:68-77)
     std::mt19937 rng;
-    const u32 repeat_last_n = 64;
-    const float repeat_penalty = 1.1f, alpha_frequency = 0.1f, alpha_presence = 0.0f, temp = 0.8f, mirostat_tau = 5.0f, mirostat_eta = 0.1f;
+    static constexpr u32 repeat_last_n = 64;
+    static constexpr float repeat_penalty = 1.1f, alpha_frequency = 0.1f, alpha_presence = 0.0f, temp = 0.8f, mirostat_tau = 5.0f, mirostat_eta = 0.1f;
     float mirostat_mu;
 
     lv_session *device_session = nullptr;

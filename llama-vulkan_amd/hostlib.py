@@ -39,7 +39,9 @@ def lib():
             "llh_session_start": (C.c_int, [vp]), "llh_session_finish": (u, [vp, C.c_int]), "llh_session_predict": (u, [vp, C.c_int]),
             "llh_session_rewind": (None, [vp, u]), "llh_session_set_options": (u, [vp, u]), "llh_session_is_tracing": (C.c_int, [vp]),
             "llh_session_save_frame": (u, [vp, cp]), "llh_session_snapshot": (u, [vp, cp]), "llh_session_restore": (u, [vp, cp]),
-            "llh_session_seed": (None, [vp, u]), "llh_session_backlog": (u, [vp]), "llh_session_device": (vp, [vp]), "llh_session_tokens_in_gpu": (u, [vp]),
+            "llh_session_seed": (None, [vp, u]), "llh_session_backlog": (u, [vp]), "llh_session_device": (vp, [vp]),
+            "llh_sample_token": (u, [C.POINTER(C.c_float), u, C.POINTER(u), u, C.POINTER(C.c_float), u, C.POINTER(u), C.POINTER(C.c_float), u,
+                                     C.POINTER(u), C.POINTER(C.c_float), C.POINTER(C.c_int)]), "llh_session_tokens_in_gpu": (u, [vp]),
             "llh_session_logits": (u, [vp, C.c_void_p, u]), "llh_session_spevars": (None, [vp, C.POINTER(u)]), "llh_session_layer_count": (u, [vp]),
         }
         for name, (res, args) in sig.items():
@@ -111,6 +113,19 @@ class GgmlFile:
         buf = C.create_string_buffer(cap)
         n = lib().llh_file_detokenize(self.h, arr, len(ids), buf, cap)
         return buf.raw[:n]
+
+
+def sample_token(logits, history, mu, seed):
+    """llava_session::sample_token (the stochastic pick of llava_session.cpp:154-194) on given logits and token history.
+    Returns (token, new mu, kept ids, kept probabilities, their sum, index drawn among the kept)."""
+    n = len(logits)
+    lg = (C.c_float * n)(*[float(v) for v in logits])
+    hist = (C.c_uint * max(len(history), 1))(*[int(t) for t in history])
+    mu_io, ids, ps = C.c_float(mu), (C.c_uint * n)(), (C.c_float * n)()
+    count, total, pick = C.c_uint(), C.c_float(), C.c_int()
+    tok = lib().llh_sample_token(lg, n, hist, len(history), C.byref(mu_io), seed, ids, ps, n, C.byref(count), C.byref(total), C.byref(pick))
+    k = count.value
+    return tok, mu_io.value, [int(ids[i]) for i in range(k)], [float(ps[i]) for i in range(k)], total.value, pick.value
 
 
 class LlavaContext:
