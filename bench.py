@@ -69,12 +69,58 @@ def prefill_report(n, ms):
             "executed_tflops": round(2 * tf, 1), "mfma_peak_tflops": 2500.0, "frac_of_mfma_peak": round(2 * tf / 2500.0, 4)}
 
 
+def lavapipe_status():
+    """The baseline this metric would ideally sit beside is the reference's own Vulkan build run on the host cores by Mesa
+    lavapipe.  That needs a Vulkan loader, the lavapipe ICD, a GLSL compiler for the 30 shaders and the reference's
+    sources, and a patched device selection (the reference accepts discrete and integrated GPUs only,
+    llava_context.cpp:36-60).  Reports what is missing on this machine."""
+    import ctypes.util
+    import glob
+    import shutil
+    missing = []
+    if not ctypes.util.find_library("vulkan"):
+        missing.append("no libvulkan")
+    if not glob.glob("/usr/share/vulkan/icd.d/*lvp*") and not glob.glob("/etc/vulkan/icd.d/*lvp*"):
+        missing.append("no lavapipe ICD")
+    if not (shutil.which("glslc") or shutil.which("glslangValidator")):
+        missing.append("no GLSL compiler")
+    missing.append("the reference's sources and build are not on this machine")
+    return "unavailable: " + ", ".join(missing)
+
+
+def other_cases(lva, ctx):
+    """The other configurations under the same clock, after the headline's timed region: isolated GEMVs at the 7B decode
+    shapes in both weight types, 7B q8_0 at positions 1920..2047, 13B q4_0 with a 32-token prompt and 256 steps (on the
+    persistent kernel and on the hipGraph of the operator chain), the 7B q4_0 headline workload on the hipGraph path, and
+    the 13B q8_0 512-token prompt.  Each entry carries tok_s or ms or us, and frac of the roofline that bounds it (HBM for
+    decode and GEMV, matrix cores for the prompt)."""
+    measure = importlib.import_module("llama-vulkan_amd.measure")
+    q = measure.quiet
+    cases = []
+    for g in measure.gemv_cases(ctx, report=q):
+        cases.append({"name": f"gemv {g['wtype']} {g['rows']}x{g['cols']} {g['mode']}", "us": g["us"], "GBps": g["GBps"], "frac": g["frac_of_peak"],
+                      "bound": "hbm"})
+    for name, args, kw in (
+            ("7B q8_0 decode, positions 1920..2047", ("decode-q8", "7b", lva.LV_Q8_0, 1, 2048, 1916, 128), {}),
+            ("13B q4_0 decode, 32-token prompt + 256 steps, persistent kernel", ("decode-13b", "13b", lva.LV_Q4_0, 2, 512, 32, 256), {}),
+            ("13B q4_0 decode, 32-token prompt + 256 steps, hipGraph", ("decode-13b-graph", "13b", lva.LV_Q4_0, 2, 512, 32, 256), {"force_path": lva.PATH_GRAPH}),
+            ("7B q4_0 decode, positions 444..511, hipGraph", ("decode-7b-graph", "7b", lva.LV_Q4_0, 0, 512, 440, 68), {"force_path": lva.PATH_GRAPH})):
+        d = measure.decode_case(ctx, *args, report=q, **kw)
+        cases.append({"name": name, "path": d["path"], "tok_s": d["tok_s"], "ms": d["ms_per_token"], "GBps": d["GBps"], "frac": d["frac_of_peak"],
+                      "bound": "hbm"})
+    p = measure.prefill_case(ctx, "prefill-13b", "13b", lva.LV_Q8_0, report=q)
+    cases.append({"name": "13B q8_0 prompt of 512 tokens as one step", "tok_s": p["tok_s"], "ms": p["ms"], "executed_TFLOPs": p["executed_TFLOPs"],
+                  "frac": p["frac_of_mfma_peak"], "bound": "mfma"})
+    return cases
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--cpu-steps", type=int, default=3, help="decode steps the CPU checker is timed on (0 = skip)")
+    ap.add_argument("--no-cases", action="store_true", help="skip the other configurations (the \"cases\" key)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs the decode path on ONE GPU (batch-1 decode has nothing to shard in this "
@@ -162,7 +208,8 @@ def main():
             raise SystemExit(f"bench.py: logits differ from the CPU checker by {worst}")
         cpu = {"value": round(n_cpu / cpu_dt, 3), "unit": "tok/s", "cores": oracle.num_threads(), "kind": "port",
                "sample": f"{n_cpu} greedy decode steps of the same model at positions {start}..{pos - 1} "
-                         f"(cache restored from the GPU run; tokens identical, max |dlogit| {worst:.1e})"}
+                         f"(cache restored from the GPU run; tokens identical, max |dlogit| {worst:.1e})",
+               "lavapipe": lavapipe_status()}
         osess.close()
         om.close()
 
@@ -188,9 +235,11 @@ def main():
         "cpu_baseline": cpu,
         "prefill": prefill_report(first, prefill_ms),
     }
-    print(json.dumps(out), flush=True)
     sess.close()
     model.close()
+    if not args.no_cases:
+        out["cases"] = other_cases(lva, ctx)
+    print(json.dumps(out), flush=True)
     ctx.close()
 
 

@@ -3,7 +3,9 @@
 
     python llama-vulkan_amd/measure.py gemv          isolated dequant-fused GEMVs at the 7B shapes, q4_0 and q8_0
     python llama-vulkan_amd/measure.py decode-q8     7B q8_0, cache positions 1920..2047 (128 greedy steps)
-    python llama-vulkan_amd/measure.py decode-13b    13B q4_0, 32-token prompt + 256 greedy steps
+    python llama-vulkan_amd/measure.py decode-13b    13B q4_0, 32-token prompt + 256 greedy steps (persistent kernel)
+    python llama-vulkan_amd/measure.py decode-13b-graph   the same on the hipGraph of the operator chain
+    python llama-vulkan_amd/measure.py decode-7b-graph    7B q4_0, positions 444..511 on the hipGraph of the operator chain
     python llama-vulkan_amd/measure.py prefill-13b   13B q8_0, 512-token prompt evaluated in one lv_step_begin
     python llama-vulkan_amd/measure.py prefill-7b    7B q4_0, the same
     python llama-vulkan_amd/measure.py prefill-13b-q4  13B q4_0, the same
@@ -13,7 +15,8 @@
 
 Every figure is algorithmic bytes (weights as stored in the GGML file, 18 B / 34 B per 32 weights, plus vectors and the
 fp16 cache rows a step reads) divided by the time measured with HIP events on the stream that runs the kernels.
-Models are seeded synthetic GGJT files written to /dev/shm (or /tmp) on first use."""
+Models are seeded synthetic GGJT files written to /dev/shm (or /tmp) on first use.  Every case function returns its
+figures as a dict (bench.py collects them under "cases"); run as a script, each is printed as one JSON line."""
 import importlib
 import json
 import os
@@ -29,14 +32,16 @@ SHAPES = {"7b": dict(vocab=32000, dim=4096, heads=32, layers=32, ff=11008), "13b
 
 def emit(**kw):
     print(json.dumps(kw), flush=True)
+    return kw
 
 
 def block_bytes(ftype):
     return 18 if ftype == lva.LV_Q4_0 else 34
 
 
-def gemv_cases(ctx):
+def gemv_cases(ctx, report=emit):
     """reference: matmul.glsl / matmul_q8.glsl / matmul_silu_ff.comp at the three layer shapes and the output matrix"""
+    out_cases = []
     for ftype, tname in ((lva.LV_Q4_0, "q4_0"), (lva.LV_Q8_0, "q8_0")):
         for rows, cols, mode in ((4096, 4096, "store"), (11008, 4096, "silu"), (4096, 11008, "add"), (32000, 4096, "store")):
             nbytes = rows * cols // 32 * block_bytes(ftype) * (2 if mode == "silu" else 1) + 4 * cols + 4 * rows * (2 if mode == "add" else 1)
@@ -62,12 +67,17 @@ def gemv_cases(ctx):
                 for i in range(nmat):
                     run(i)
             us = ctx.timer_stop() * 1e3 / (iters * nmat)
-            emit(case="gemv", wtype=tname, rows=rows, cols=cols, mode=mode, us=round(us, 2), algorithmic_bytes=nbytes,
-                 GBps=round(nbytes / us / 1e3, 1), frac_of_peak=round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4))
+            out_cases.append(report(case="gemv", wtype=tname, rows=rows, cols=cols, mode=mode, us=round(us, 2), algorithmic_bytes=nbytes,
+                                    GBps=round(nbytes / us / 1e3, 1), frac_of_peak=round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)))
             for m in mats:
                 ctx.matrix_free(m)
             ctx.free(x)
             ctx.free(out)
+    return out_cases
+
+
+def quiet(**kw):
+    return kw
 
 
 def copy_case(ctx):
@@ -87,6 +97,8 @@ def copy_case(ctx):
 def model_file(preset, wtype, seed):
     base = "/dev/shm" if os.access("/dev/shm", os.W_OK) else "/tmp"
     path = os.path.join(base, f"llava_measure_{preset}_{'q4_0' if wtype == lva.LV_Q4_0 else 'q8_0'}_seed{seed}.ggml")
+    if (preset, wtype, seed) == ("7b", lva.LV_Q4_0, 0):
+        path = os.path.join(base, "llava_bench_7b_q4_0_seed0.ggml")      # the file bench.py and the full-size tests use
     if not os.path.exists(path):
         lva.write_model(path + ".tmp", wtype=wtype, seed=seed, **SHAPES[preset])
         os.replace(path + ".tmp", path)
@@ -99,11 +111,13 @@ def step_bytes(shape, wtype, pos):
     return L * per_layer + V * D // 32 * block_bytes(wtype) + (2 * L + 1) * D * 4 + L * 2 * D * 2 * (pos + 2) + V * 4 + D * 4
 
 
-def decode_case(ctx, name, preset, wtype, seed, backlog, first, steps):
+def decode_case(ctx, name, preset, wtype, seed, backlog, first, steps, force_path=None, report=emit):
     shape = SHAPES[preset]
     path = model_file(preset, wtype, seed)
     model = lva.Model(ctx, path)
     s = lva.Session(model, backlog)
+    if force_path is not None:
+        s.set_path(force_path)
     kind = {lva.PATH_KERNELS: "kernels", lva.PATH_GRAPH: "graph", lva.PATH_PERSISTENT: "persistent"}[s.path()]
     prompt = lva.synth_tokens(first, 3, shape["vocab"], seed=seed)
     t0 = time.perf_counter()
@@ -123,14 +137,18 @@ def decode_case(ctx, name, preset, wtype, seed, backlog, first, steps):
         total += step_bytes(shape, wtype, pos)
         pos += 1
     dt = time.perf_counter() - t0
-    emit(case=name, model=preset, wtype="q4_0" if wtype == lva.LV_Q4_0 else "q8_0", path=kind, positions=[first + 4, pos - 1], steps=steps,
-         tok_s=round(steps / dt, 1), ms_per_token=round(dt / steps * 1e3, 4), GBps=round(total / dt / 1e9, 1),
-         frac_of_peak=round(total / dt / 1e9 / HBM_PEAK_GBS, 4), prompt_tokens=first, prompt_s=round(prefill_s, 3))
+    r = report(case=name, model=preset, wtype="q4_0" if wtype == lva.LV_Q4_0 else "q8_0", path=kind, positions=[first + 4, pos - 1], steps=steps,
+               tok_s=round(steps / dt, 1), ms_per_token=round(dt / steps * 1e3, 4), GBps=round(total / dt / 1e9, 1),
+               frac_of_peak=round(total / dt / 1e9 / HBM_PEAK_GBS, 4), prompt_tokens=first, prompt_s=round(prefill_s, 3))
     s.close()
     model.close()
+    return r
 
 
-def prefill_case(ctx, case, name, wtype):
+MFMA_PEAK_TFLOPS = 2500.0
+
+
+def prefill_case(ctx, case, name, wtype, report=emit):
     shape = SHAPES[name]
     path = model_file(name, wtype, 3)
     model = lva.Model(ctx, path)
@@ -143,10 +161,13 @@ def prefill_case(ctx, case, name, wtype):
     ms = s.timer_stop()
     D, F, V, L = shape["dim"], shape["ff"], shape["vocab"], shape["layers"]
     flops = 2.0 * 512 * L * (4 * D * D + 3 * D * F) + 2.0 * V * D      # the output matrix sees the last row only
-    emit(case=case, model=name, wtype="q4_0" if wtype == lva.LV_Q4_0 else "q8_0", tokens=512, ms=round(ms, 2),
-         tok_s=round(512 / ms * 1e3, 1), TFLOPs=round(flops / ms / 1e9, 2))
+    # every product is executed twice (activations are a pair of halves), so the matrix cores run at twice the useful rate
+    r = report(case=case, model=name, wtype="q4_0" if wtype == lva.LV_Q4_0 else "q8_0", tokens=512, ms=round(ms, 2),
+               tok_s=round(512 / ms * 1e3, 1), TFLOPs=round(flops / ms / 1e9, 2), executed_TFLOPs=round(2 * flops / ms / 1e9, 2),
+               frac_of_mfma_peak=round(2 * flops / ms / 1e9 / MFMA_PEAK_TFLOPS, 4))
     s.close()
     model.close()
+    return r
 
 
 def gemm_cases(ctx):
@@ -183,6 +204,10 @@ def main():
         decode_case(ctx, "decode-q8", "7b", lva.LV_Q8_0, 1, 2048, 1916, 128)
     if which in ("decode-13b", "all"):
         decode_case(ctx, "decode-13b", "13b", lva.LV_Q4_0, 2, 512, 32, 256)
+    if which in ("decode-13b-graph", "all"):
+        decode_case(ctx, "decode-13b-graph", "13b", lva.LV_Q4_0, 2, 512, 32, 256, force_path=lva.PATH_GRAPH)
+    if which in ("decode-7b-graph", "all"):
+        decode_case(ctx, "decode-7b-graph", "7b", lva.LV_Q4_0, 0, 512, 440, 68, force_path=lva.PATH_GRAPH)
     if which in ("prefill-13b", "all"):
         prefill_case(ctx, "prefill-13b", "13b", lva.LV_Q8_0)
     if which in ("prefill-13b-q4", "all"):
