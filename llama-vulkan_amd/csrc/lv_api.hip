@@ -84,6 +84,7 @@ struct lv_matrix {
     MatView view{};
     uint32_t ftype = 0;
     uint64_t bytes = 0;
+    const uint16_t *h16 = nullptr;   // prompt copy (lv_gemm.h): codes as fp16 integers and fp32 scales in tile order; null until a batch needs it
 };
 
 struct LayerWeights {
@@ -107,6 +108,10 @@ struct lv_model {
     uint8_t *mega_stream = nullptr;
     float *mega_norms = nullptr;    // [layers][2][D] + final norm [D]
     float *tok_f32_own = nullptr;   // fp32 copy of a quantised embedding table (the persistent kernel reads rows as fp32)
+    // prompt copy of the layer matrices (lv_gemm.h), made when the first batch is evaluated; sessions of several threads share it
+    std::mutex prompt_mutex;
+    int prompt_state = 0;           // 0 not made yet, 1 ready, -1 could not be made (batches then go token by token)
+    uint16_t *prompt_arena = nullptr;
 };
 
 // Shape classes the persistent kernel is compiled for: LLaMA-7B and LLaMA-13B layer shapes, q4_0 and q8_0.
@@ -711,53 +716,42 @@ extern "C" int lv_kernel_gemv_silu(lv_ctx *c, float *out, const lv_matrix *w3, c
 static int launch_gemm_presplit(hipStream_t st, float *out, uint32_t ldo, const lv_matrix &w, uint32_t n, const uint16_t *xh, const uint16_t *xl,
                                 bool accumulate);
 
-// fp32 activations -> fp16 halves in the element order the GEMM for weight type `ftype` expects
-static int launch_split(hipStream_t st, uint16_t *xh, uint16_t *xl, const float *x, uint32_t n, uint32_t K, uint32_t ftype)
+// fp32 activations -> the two fp16 halves the GEMM multiplies
+static int launch_split(hipStream_t st, uint16_t *xh, uint16_t *xl, const float *x, uint32_t n, uint32_t K)
 {
-    const uint32_t n_pad = (n + kGemmTile - 1) / kGemmTile * kGemmTile;
-    const dim3 grid((K / 4 + 255) / 256, n_pad);
-    if (ftype == LV_Q4_0) split_half_kernel<4><<<grid, dim3(256), 0, st>>>(xh, xl, x, n, K);
-    else split_half_kernel<8><<<grid, dim3(256), 0, st>>>(xh, xl, x, n, K);
+    const uint32_t n_pad = (n + kGemmTile - 1) / kGemmTile * kGemmTile, Kp = gemm_k_padded(K);
+    split_half_kernel<<<dim3(Kp / 64, n_pad / 32), dim3(256), 0, st>>>(xh, xl, x, n, K, Kp);
     HIP_TRY(hipGetLastError());
     return LV_OK;
 }
 
-static int launch_gemm(hipStream_t st, float *out, uint32_t ldo, const lv_matrix &w, const float *x, uint32_t n, uint16_t *xh, uint16_t *xl,
-                       bool accumulate)
+// the prompt copy of one matrix into dst (gemm_copy_halfs halfs)
+static uint64_t prompt_copy_halfs(const lv_matrix &w) { return gemm_copy_halfs(w.view.rows, w.view.cols); }
+static int launch_expand(hipStream_t st, uint16_t *dst, const lv_matrix &w)
 {
-    const uint32_t K = w.view.cols;
-    if (K % 32) return fail(LV_ERR_ARG, "gemm: %u columns", K);
-    LV_TRY(launch_split(st, xh, xl, x, n, K, w.ftype));
-    return launch_gemm_presplit(st, out, ldo, w, n, xh, xl, accumulate);
+    const uint64_t threads = (uint64_t)gemm_rows_padded(w.view.rows) * (gemm_k_padded(w.view.cols) / 32);
+    const dim3 grid((unsigned)((threads + 255) / 256));
+    if (w.ftype == LV_Q4_0) expand_codes_kernel<4><<<grid, dim3(256), 0, st>>>(dst, w.view);
+    else if (w.ftype == LV_Q8_0) expand_codes_kernel<8><<<grid, dim3(256), 0, st>>>(dst, w.view);
+    else return fail(LV_ERR_ARG, "gemm: matrix type %u", w.ftype);
+    HIP_TRY(hipGetLastError());
+    return LV_OK;
 }
 
-// launches gemm_kernel for args whose ws[0..nz-1] are set: nz matrices, or nz K slices of one
-static int dispatch_gemm(hipStream_t st, const GemmArgs &a, const lv_matrix &w, uint32_t nz)
+// launches gemm_kernel for args whose w16[0..nz-1] and outs[0..nz-1] are set: nz matrices of one shape, or nz K slices of one
+static int dispatch_gemm(hipStream_t st, GemmArgs a, const lv_matrix &w, uint32_t nz)
 {
-    // Three forms.  128 tokens x 128 rows with eight waves and two LDS buffers (one workgroup per CU) is the base.
-    // 128 x 256 (every wave 64 x 64: a quarter fewer operand reads from LDS per MFMA) does the same work about 8 %
-    // faster per CU, so it is taken when its coarser rounds of 256 workgroups do not cost more than that.  Fewer than
-    // 128 workgroups of the base form: 64-row ones of four waves, twice as many.  Measured at 512 tokens, q8_0,
-    // 5120 x 5120 / 13824 x 5120 / 5120 x 13824: base 103 / 216 / 263 us; with one LDS buffer 106 / 224 / 280; the
-    // 64-row form at those sizes 135 / - / 355.
-    const uint32_t token_tiles = (a.n + kGemmTile - 1) / kGemmTile;
-    constexpr uint32_t cus = 256;
-    const uint32_t t128 = (w.view.rows + 127) / 128 * token_tiles * nz, t256 = (w.view.rows + 255) / 256 * token_tiles * nz;
-    const bool narrow = t128 < 128;
-    const bool wide = !narrow && (double)((t256 + cus - 1) / cus) * 1.84 < (double)((t128 + cus - 1) / cus);
-    const uint32_t rm = narrow ? 64 : wide ? 256 : 128;
-    const dim3 grid((w.view.rows + rm - 1) / rm, token_tiles, nz);
-    const bool sf32 = w.view.scales_f32 != nullptr;
-    if (w.ftype == LV_Q4_0) {
-        if (narrow) { if (sf32) gemm_kernel<4, 64, 4, true><<<grid, dim3(256), 0, st>>>(a); else gemm_kernel<4, 64, 4, false><<<grid, dim3(256), 0, st>>>(a); }
-        else if (wide) { if (sf32) gemm_kernel<4, 256, 8, true, true><<<grid, dim3(512), 0, st>>>(a); else gemm_kernel<4, 256, 8, false, true><<<grid, dim3(512), 0, st>>>(a); }
-        else { if (sf32) gemm_kernel<4, 128, 8, true, true><<<grid, dim3(512), 0, st>>>(a); else gemm_kernel<4, 128, 8, false, true><<<grid, dim3(512), 0, st>>>(a); }
-    } else if (w.ftype == LV_Q8_0) {
-        if (narrow) { if (sf32) gemm_kernel<8, 64, 4, true><<<grid, dim3(256), 0, st>>>(a); else gemm_kernel<8, 64, 4, false><<<grid, dim3(256), 0, st>>>(a); }
-        else if (wide) { if (sf32) gemm_kernel<8, 256, 8, true, true><<<grid, dim3(512), 0, st>>>(a); else gemm_kernel<8, 256, 8, false, true><<<grid, dim3(512), 0, st>>>(a); }
-        else { if (sf32) gemm_kernel<8, 128, 8, true, true><<<grid, dim3(512), 0, st>>>(a); else gemm_kernel<8, 128, 8, false, true><<<grid, dim3(512), 0, st>>>(a); }
-    }
-    else return fail(LV_ERR_ARG, "gemm: matrix type %u", w.ftype);
+    a.rows = w.view.rows; a.K = w.view.cols;
+    for (uint32_t i = 0; i < nz; i++)
+        if (!a.w16[i]) return fail(LV_ERR_STATE, "gemm: the matrix has no prompt copy");
+    static std::once_flag lds_once;
+    static hipError_t lds_rc = hipSuccess;
+    std::call_once(lds_once, [] { lds_rc = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLdsBytes); });
+    HIP_TRY(lds_rc);
+    const uint32_t token_tiles = (a.n + kGemmTile - 1) / kGemmTile, row_tiles = (a.rows + kGemmRows - 1) / kGemmRows;
+    a.nz = nz;
+    const dim3 grid((row_tiles * nz + 7) / 8 * 8 * token_tiles);
+    gemm_kernel<<<grid, dim3(512), kGemmLdsBytes, st>>>(a);
     HIP_TRY(hipGetLastError());
     return LV_OK;
 }
@@ -768,12 +762,12 @@ static int launch_gemm_multi(hipStream_t st, float *const outs[], uint32_t ldo, 
                              const uint16_t *xh, const uint16_t *xl, bool accumulate)
 {
     GemmArgs a{};
-    for (int i = 0; i < nmat; i++) { a.outs[i] = outs[i]; a.ws[i] = ws[i]->view; }
+    for (int i = 0; i < nmat; i++) { a.outs[i] = outs[i]; a.w16[i] = ws[i]->h16; }
     a.xh = xh; a.xl = xl; a.n = n; a.ldo = ldo; a.accumulate = accumulate ? 1 : 0;
     return dispatch_gemm(st, a, *ws[0], (uint32_t)nmat);
 }
 
-// Into how many K slices to cut a product whose 128 x 128 output tiles alone number `tiles`: the count (1..3) that
+// Into how many K slices to cut a product whose 128 x 256 output tiles alone number `tiles`: the count (1..3) that
 // leaves the fewest CU-rounds idle, the smaller count unless a larger one fills them clearly better.  A slice keeps
 // at least 16 K steps.
 static uint32_t gemm_k_slices(uint32_t tiles, uint32_t k_steps)
@@ -807,7 +801,7 @@ static uint32_t gemm_slices_for(const lv_matrix &w, uint32_t n, uint32_t ldo)
 {
     const uint32_t rows = w.view.rows, k_steps = (w.view.cols + kGemmK - 1) / kGemmK;
     const uint32_t token_tiles = (n + kGemmTile - 1) / kGemmTile;
-    return (rows % 4 || ldo % 4) ? 1 : gemm_k_slices((rows + 127) / 128 * token_tiles, k_steps);
+    return (rows % 4 || ldo % 4) ? 1 : gemm_k_slices((rows + kGemmRows - 1) / kGemmRows * token_tiles, k_steps);
 }
 
 // one matrix, activations already split, K cut in slices when that fills the CUs better: the slices go to parts[]
@@ -823,12 +817,13 @@ static int launch_gemm_sliced(hipStream_t st, float *out, uint32_t ldo, const lv
     GemmArgs a{};
     a.xh = xh; a.xl = xl; a.n = n;
     if (slices == 1) {
-        a.outs[0] = out; a.ws[0] = w.view; a.ldo = ldo; a.accumulate = accumulate ? 1 : 0;
+        a.outs[0] = out; a.w16[0] = w.h16; a.ldo = ldo; a.accumulate = accumulate ? 1 : 0;
         return dispatch_gemm(st, a, w, 1);
     }
-    a.slice_steps = (k_steps + slices - 1) / slices;
-    const uint32_t used = (k_steps + a.slice_steps - 1) / a.slice_steps;      // every slice launched has a step
-    for (uint32_t i = 0; i < used; i++) { a.outs[i] = parts[i]; a.ws[i] = w.view; }
+    const uint32_t slice_steps = (k_steps + slices - 1) / slices;
+    a.slice_k = slice_steps * kGemmK;
+    const uint32_t used = (k_steps + slice_steps - 1) / slice_steps;      // every slice launched has a step
+    for (uint32_t i = 0; i < used; i++) { a.outs[i] = parts[i]; a.w16[i] = w.h16; }
     a.ldo = rows;
     LV_TRY(dispatch_gemm(st, a, w, used));
     if (pending && accumulate) { *pending = used; return LV_OK; }
@@ -855,21 +850,29 @@ extern "C" int lv_kernel_gemm(lv_ctx *c, float *out, const lv_matrix *w, const f
     if (batch == 0) return LV_OK;
     if (batch > kMaxStepTokens) return fail(LV_ERR_RANGE, "lv_kernel_gemm: batch %u (limit %u)", batch, kMaxStepTokens);
     HIP_TRY(hipSetDevice(c->device));
-    const size_t n_pad = (batch + kGemmTile - 1) / kGemmTile * kGemmTile, halfs = n_pad * w->view.cols;
+    const size_t n_pad = (batch + kGemmTile - 1) / kGemmTile * kGemmTile, halfs = n_pad * gemm_k_padded(w->view.cols);
     if (w->view.cols % 32) return fail(LV_ERR_ARG, "gemm: %u columns", w->view.cols);
-    // workspace: the two fp16 halves of the activations and, where K is cut in slices, their partial results
+    // workspace: the matrix's prompt copy, the two fp16 halves of the activations and, where K is cut in slices, their
+    // partial results
     const uint32_t slices = gemm_slices_for(*w, batch, w->view.rows);
     const size_t part = slices > 1 ? (size_t)batch * w->view.rows : 0;
-    uint16_t *xh = nullptr;
-    hipError_t e = hipMalloc(reinterpret_cast<void **>(&xh), halfs * 4 + part * slices * 4);
+    const size_t w_halfs = w->h16 ? 0 : (size_t)prompt_copy_halfs(*w);
+    uint16_t *ws = nullptr;
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&ws), (w_halfs + halfs * 2) * 2 + part * slices * 4);
     if (e != hipSuccess) return fail(LV_ERR_OOM, "lv_kernel_gemm: workspace");
-    uint16_t *xl = xh + halfs;
+    uint16_t *xh = ws + w_halfs, *xl = xh + halfs;
     float *p0 = reinterpret_cast<float *>(xl + halfs);
     float *const parts[kGemmMaxMats] = {p0, p0 + part, p0 + 2 * part};
-    int rc = launch_split(c->stream, xh, xl, x, batch, w->view.cols, w->ftype);
-    if (rc == LV_OK) rc = launch_gemm_sliced(c->stream, out, w->view.rows, *w, batch, xh, xl, accumulate != 0, slices > 1 ? parts : nullptr);
+    lv_matrix wm = *w;
+    int rc = LV_OK;
+    if (!wm.h16) {
+        rc = launch_expand(c->stream, ws, *w);
+        wm.h16 = ws;
+    }
+    if (rc == LV_OK) rc = launch_split(c->stream, xh, xl, x, batch, w->view.cols);
+    if (rc == LV_OK) rc = launch_gemm_sliced(c->stream, out, w->view.rows, wm, batch, xh, xl, accumulate != 0, slices > 1 ? parts : nullptr);
     (void)hipStreamSynchronize(c->stream);
-    (void)hipFree(xh);
+    (void)hipFree(ws);
     return rc;
 }
 
@@ -1195,6 +1198,7 @@ extern "C" int lv_model_destroy(lv_model *m)
 {
     if (!m) return LV_OK;
     (void)hipSetDevice(m->ctx->device);
+    (void)hipFree(m->prompt_arena);
     (void)hipFree(m->mega_stream);
     (void)hipFree(m->mega_norms);
     (void)hipFree(m->tok_f32_own);
@@ -1542,6 +1546,34 @@ static int record_token(lv_session *s, uint32_t idx, bool with_head)
 }
 
 // ---- batched prompt evaluation -----------------------------------------------------------------------------
+// The prompt copy of every layer matrix, made when a model evaluates its first batch (2 bytes a weight: 13.5 GB for a
+// 7B model; decode never reads it).  False when the device has no room for it: batches then go token by token.
+static bool ensure_prompt_copy(lv_model *m)
+{
+    std::lock_guard<std::mutex> lock(m->prompt_mutex);
+    if (m->prompt_state) return m->prompt_state > 0;
+    uint64_t halfs = 0;
+    for (LayerWeights &lw : m->layers)
+        for (lv_matrix *x : {&lw.wq, &lw.wk, &lw.wv, &lw.wo, &lw.w1, &lw.w2, &lw.w3}) halfs += prompt_copy_halfs(*x);
+    m->prompt_state = -1;
+    if (hipMalloc(reinterpret_cast<void **>(&m->prompt_arena), halfs * 2) != hipSuccess) {
+        (void)hipGetLastError();
+        m->prompt_arena = nullptr;
+        return false;
+    }
+    uint16_t *at = m->prompt_arena;
+    hipStream_t st = m->ctx->stream;
+    for (LayerWeights &lw : m->layers)
+        for (lv_matrix *x : {&lw.wq, &lw.wk, &lw.wv, &lw.wo, &lw.w1, &lw.w2, &lw.w3}) {
+            if (launch_expand(st, at, *x) != LV_OK) return false;
+            x->h16 = at;
+            at += prompt_copy_halfs(*x);
+        }
+    if (hipStreamSynchronize(st) != hipSuccess) return false;
+    m->prompt_state = 1;
+    return true;
+}
+
 constexpr uint32_t kPrefillChunk = 512;    // tokens evaluated together (bounds the workspace)
 constexpr uint32_t kPrefillMin = 16;       // below this the rows go through the one-token kernels
 
@@ -1554,7 +1586,8 @@ static int prefill_reserve(lv_session *s, uint32_t n)
         HIP_TRY(hipStreamSynchronize(s->stream));
         void **bufs[] = {(void **)&s->pf_x, (void **)&s->pf_xn, (void **)&s->pf_q, (void **)&s->pf_k, (void **)&s->pf_v, (void **)&s->pf_vo,
                          (void **)&s->pf_g1, (void **)&s->pf_g2, (void **)&s->pf_xh, (void **)&s->pf_xl};
-        const size_t sizes[] = {D * 4, D * 4, D * 4, D * 4, D * 4, D * 4, F * 4, F * 4, (F > D ? F : D) * 2, (F > D ? F : D) * 2};
+        const size_t halfs = gemm_k_padded((uint32_t)(F > D ? F : D)) * 2;   // an activation half: padded K, 2 bytes each
+        const size_t sizes[] = {D * 4, D * 4, D * 4, D * 4, D * 4, D * 4, F * 4, F * 4, halfs, halfs};
         s->pf_cap = 0;
         for (int i = 0; i < 10; i++) {
             (void)hipFree(*bufs[i]);
@@ -1567,25 +1600,25 @@ static int prefill_reserve(lv_session *s, uint32_t n)
     return LV_OK;
 }
 
-// x += pending K slices, xn = normalize(x) * w, halves of xn for a GEMM on weights of type ftype: one kernel where the
+// x += pending K slices, xn = normalize(x) * w, halves of xn for the next GEMM: one kernel where the
 // row fits its registers, else the three separate ones.  xn (fp32) is written only when want_xn.
-static int launch_prefill_norm(hipStream_t st, lv_session *s, const float *w, uint32_t n, uint32_t D, uint32_t ftype, float *const parts[kGemmMaxMats],
+static int launch_prefill_norm(hipStream_t st, lv_session *s, const float *w, uint32_t n, uint32_t D, float *const parts[kGemmMaxMats],
                                uint32_t pending, bool want_xn)
 {
     const uint32_t n_pad = (n + kGemmTile - 1) / kGemmTile * kGemmTile;
-    if (D <= 8192 && D % 4 == 0 && (ftype == LV_Q4_0 || ftype == LV_Q8_0)) {
+    if (D <= 8192 && D % 8 == 0) {
         PrefillNormArgs a{};
         a.x = s->pf_x; a.nparts = pending; a.w = w; a.xn = want_xn ? s->pf_xn : nullptr; a.xh = s->pf_xh; a.xl = s->pf_xl; a.dim = D; a.n = n;
+        a.Kp = gemm_k_padded(D);
         for (uint32_t i = 0; i < pending; i++) a.parts[i] = parts[i];
-        if (ftype == LV_Q4_0) prefill_norm_kernel<4><<<dim3(n_pad), dim3(256), 0, st>>>(a);
-        else prefill_norm_kernel<8><<<dim3(n_pad), dim3(256), 0, st>>>(a);
+        prefill_norm_kernel<<<dim3(n_pad), dim3(256), 0, st>>>(a);
         HIP_TRY(hipGetLastError());
         return LV_OK;
     }
     if (pending) LV_TRY(launch_gemm_reduce(st, s->pf_x, D, parts, pending, D, n, true));
     normalize_kernel<<<dim3(n), dim3(256), 0, st>>>(s->pf_xn, s->pf_x, w, D);
     HIP_TRY(hipGetLastError());
-    return launch_split(st, s->pf_xh, s->pf_xl, s->pf_xn, n, D, ftype);
+    return launch_split(st, s->pf_xh, s->pf_xl, s->pf_xn, n, D);
 }
 
 // Rows idx0 .. idx0+n-1 of the step at once (llava_layer.cpp:39-75 with batch > 1).  Row z sees cache rows
@@ -1615,7 +1648,7 @@ static int record_prefill(lv_session *s, uint32_t idx0, uint32_t n, bool with_he
     for (uint32_t li = 0; li < hp.layers; li++) {
         const LayerWeights &lw = m->layers[li];
         const bool qkv_same = gemm_same(lw.wq, lw.wk) && gemm_same(lw.wq, lw.wv), gate_same = gemm_same(lw.w3, lw.w1);
-        LV_TRY(launch_prefill_norm(st, s, lw.attn_norm, n, D, lw.wq.ftype, parts, pending, !qkv_same));
+        LV_TRY(launch_prefill_norm(st, s, lw.attn_norm, n, D, parts, pending, !qkv_same));
         pending = 0;
         if (qkv_same) {
             float *const outs[3] = {s->pf_q, s->pf_k, s->pf_v};
@@ -1623,18 +1656,16 @@ static int record_prefill(lv_session *s, uint32_t idx0, uint32_t n, bool with_he
             LV_TRY(launch_gemm_multi(st, outs, D, ws, 3, n, s->pf_xh, s->pf_xl, false));
         } else {
             LV_TRY(launch_gemm_presplit(st, s->pf_q, D, lw.wq, n, s->pf_xh, s->pf_xl, false));
-            if (lw.wk.ftype == lw.wq.ftype) LV_TRY(launch_gemm_presplit(st, s->pf_k, D, lw.wk, n, s->pf_xh, s->pf_xl, false));
-            else LV_TRY(launch_gemm(st, s->pf_k, D, lw.wk, s->pf_xn, n, s->pf_xh, s->pf_xl, false));
-            if (lw.wv.ftype == lw.wk.ftype) LV_TRY(launch_gemm_presplit(st, s->pf_v, D, lw.wv, n, s->pf_xh, s->pf_xl, false));
-            else LV_TRY(launch_gemm(st, s->pf_v, D, lw.wv, s->pf_xn, n, s->pf_xh, s->pf_xl, false));
+            LV_TRY(launch_gemm_presplit(st, s->pf_k, D, lw.wk, n, s->pf_xh, s->pf_xl, false));
+            LV_TRY(launch_gemm_presplit(st, s->pf_v, D, lw.wv, n, s->pf_xh, s->pf_xl, false));
         }
         kv_append2_kernel<<<dim3(kv_grid.x, kv_grid.y, 2), dim3(256), 0, st>>>(kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->pf_k, s->pf_v, pos_ptr, idx0, D, s->backlog);
         HIP_TRY(hipGetLastError());
         LV_TRY(launch_attention_batch(st, s->pf_vo, kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->pf_q, s->trig_abs, pos_ptr, idx0, n, s->backlog,
                                       hp.heads, hp.rot));
-        LV_TRY(launch_split(st, s->pf_xh, s->pf_xl, s->pf_vo, n, D, lw.wo.ftype));
+        LV_TRY(launch_split(st, s->pf_xh, s->pf_xl, s->pf_vo, n, D));
         LV_TRY(launch_gemm_sliced(st, s->pf_x, D, lw.wo, n, s->pf_xh, s->pf_xl, true, parts, &pending));
-        LV_TRY(launch_prefill_norm(st, s, lw.ffn_norm, n, D, lw.w3.ftype, parts, pending, !gate_same));
+        LV_TRY(launch_prefill_norm(st, s, lw.ffn_norm, n, D, parts, pending, !gate_same));
         pending = 0;
         if (gate_same) {
             float *const outs[2] = {s->pf_g1, s->pf_g2};
@@ -1642,13 +1673,12 @@ static int record_prefill(lv_session *s, uint32_t idx0, uint32_t n, bool with_he
             LV_TRY(launch_gemm_multi(st, outs, F, ws, 2, n, s->pf_xh, s->pf_xl, false));
         } else {
             LV_TRY(launch_gemm_presplit(st, s->pf_g1, F, lw.w3, n, s->pf_xh, s->pf_xl, false));
-            if (lw.w1.ftype == lw.w3.ftype) LV_TRY(launch_gemm_presplit(st, s->pf_g2, F, lw.w1, n, s->pf_xh, s->pf_xl, false));
-            else LV_TRY(launch_gemm(st, s->pf_g2, F, lw.w1, s->pf_xn, n, s->pf_xh, s->pf_xl, false));
+            LV_TRY(launch_gemm_presplit(st, s->pf_g2, F, lw.w1, n, s->pf_xh, s->pf_xl, false));
         }
         {   // SwiGLU straight into the fp16 halves the down projection reads
-            const dim3 grid((F / 4 + 255) / 256, (n + kGemmTile - 1) / kGemmTile * kGemmTile);
-            if (lw.w2.ftype == LV_Q4_0) silu_split_kernel<4><<<grid, dim3(256), 0, st>>>(s->pf_xh, s->pf_xl, s->pf_g1, s->pf_g2, n, F);
-            else silu_split_kernel<8><<<grid, dim3(256), 0, st>>>(s->pf_xh, s->pf_xl, s->pf_g1, s->pf_g2, n, F);
+            const uint32_t Fp = gemm_k_padded(F);
+            const dim3 grid(Fp / 64, (n + kGemmTile - 1) / kGemmTile * kGemmTile / 32);
+            silu_split_kernel<<<grid, dim3(256), 0, st>>>(s->pf_xh, s->pf_xl, s->pf_g1, s->pf_g2, n, F, Fp);
             HIP_TRY(hipGetLastError());
         }
         LV_TRY(launch_gemm_sliced(st, s->pf_x, D, lw.w2, n, s->pf_xh, s->pf_xl, true, parts, &pending));
@@ -1729,7 +1759,7 @@ extern "C" int lv_step_begin(lv_session *s, const uint32_t *tokens, uint32_t n, 
     } else {
         // rows are evaluated one after the other: row z sees cache rows 0..pos+z, which is what the batched
         // shaders compute (every row's K/V is appended before any row attends, and rows above are masked)
-        if (n >= kPrefillMin && !s->trace) {
+        if (n >= kPrefillMin && !s->trace && ensure_prompt_copy(s->model)) {
             for (uint32_t i = 0; i < n; i += kPrefillChunk) {
                 const uint32_t m = n - i < kPrefillChunk ? n - i : kPrefillChunk;
                 LV_TRY(record_prefill(s, i, m, i + m == n));

@@ -10,9 +10,21 @@
 // lane: in the MFMA result a lane holds one weight row) and added to the fp32 result.  The batched path therefore
 // agrees with the one-token fp32 path to fp32 rounding, not to fp16 rounding.
 //
-// Tiling: workgroup = 8 (or 4) waves, output tile 128 tokens x 128 (or 64) weight rows, K step 64 (two quant blocks).
-// Two threads unpack one (row, block) pair per step; every wave owns a 32-token x 64-row sub-tile of
-// v_mfma_f32_32x32x16_f16 tiles.  The global loads of step s+2 are issued before the MFMAs of step s.
+// Operands in memory.  The kernel's inner loop does nothing but MFMAs and the scale multiply-adds: the codes are not
+// unpacked there.  A model keeps a second copy of its layer matrices for this path only (the "prompt copy", made when the
+// first batch is evaluated): every code as the fp16 integer it stands for, and the block scales as fp32, both in the
+// order in which a workgroup's tile lies in LDS.  The producers of the activations (the split, norm and SwiGLU kernels
+// below) write the two halves in tile order as well.  With that a K step of a tile is one contiguous run of memory,
+// which global_load_lds_dwordx4 copies to LDS without passing through registers, four steps ahead of the MFMAs.
+//   weights      [row tile of 256][K/8 chunks][256 rows][8 halfs]
+//   scales       [row tile of 256][K/32 blocks][256 rows] fp32
+//   activations  [token tile of 128][K/8 chunks][128 tokens][8 halfs], high halves and low halves apart
+// K is padded to a multiple of 64 with zero codes and zero activations, rows to 256 with zero scales.
+// In LDS a chunk row of 16 bytes is what one lane feeds an MFMA (v_mfma_f32_32x32x16_f16: lane l holds row l%32,
+// k (l/32)*8..+7), and 32 consecutive lanes read 512 consecutive bytes: no bank conflicts, no padding.
+//
+// Tiling: workgroup = 8 waves, output tile 128 tokens x 256 weight rows, K step 32 (one quant block), every wave a
+// 64 x 64 sub-tile (2 x 2 MFMA tiles).  Four LDS stages of 33 KB.
 #pragma once
 
 #include "lv_kernels.h"
@@ -21,51 +33,116 @@ namespace lv {
 
 typedef _Float16 lv_h8 __attribute__((ext_vector_type(8)));
 typedef float lv_f16v __attribute__((ext_vector_type(16)));
+typedef __attribute__((address_space(3))) void lv_lds_void;
+typedef const __attribute__((address_space(1))) void lv_glb_void;
 
-constexpr int kGemmTile = 128;  // tokens per workgroup (batches are padded to multiples of it)
-constexpr int kGemmK = 64;      // K per step
-constexpr int kGemmLd = kGemmK + 8;  // LDS row stride in halfs (the pad spreads 16-byte reads over the banks)
+constexpr int kGemmTile = 128;   // tokens per workgroup (batches are padded to multiples of it)
+constexpr int kGemmRows = 256;   // weight rows per workgroup (the prompt copy pads matrices to multiples of it)
+constexpr int kGemmK = 64;       // K is padded to multiples of it; the unit in which K is cut in slices
+constexpr int kGemmStep = 32;    // K per pipeline stage: one quant block
+constexpr int kGemmStages = 4;
+constexpr int kGemmWBytes = kGemmStep / 8 * kGemmRows * 16;                    // 16 KB of weights per stage
+constexpr int kGemmXBytes = kGemmStep / 8 * kGemmTile * 16;                    // 8 KB per activation half
+constexpr int kGemmScBytes = kGemmRows * 4;
+constexpr int kGemmStageBytes = kGemmWBytes + 2 * kGemmXBytes + kGemmScBytes;  // 33 KB
+constexpr int kGemmLdsBytes = kGemmStages * kGemmStageBytes;                   // 132 KB: one workgroup per CU
 
-// x[n][K] fp32 -> xh, xl [n_pad][K] fp16 (rows n..n_pad-1 zero).  Inside every 32-element block the halves are stored
-// in the order the GEMM for weight type QT keeps its weight halves in (gemm_k_position).
-template <int QT>
-__global__ void split_half_kernel(uint16_t *__restrict__ xh, uint16_t *__restrict__ xl, const float *__restrict__ x, uint32_t n, uint32_t K)
+__host__ __device__ constexpr uint32_t gemm_k_padded(uint32_t K) { return (K + kGemmK - 1) / kGemmK * kGemmK; }
+__host__ __device__ constexpr uint32_t gemm_rows_padded(uint32_t rows) { return (rows + kGemmRows - 1) / kGemmRows * kGemmRows; }
+// halfs (2-byte units) of a matrix's prompt copy: the codes, then the scale plane
+__host__ __device__ constexpr uint64_t gemm_copy_code_halfs(uint32_t rows, uint32_t K) { return (uint64_t)gemm_rows_padded(rows) * gemm_k_padded(K); }
+__host__ __device__ constexpr uint64_t gemm_copy_halfs(uint32_t rows, uint32_t K)
 {
-    const uint32_t row = blockIdx.y;
-    const uint32_t i = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
-    if (i >= K) return;
-    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (row < n) v = *reinterpret_cast<const float4 *>(x + (size_t)row * K + i);
-    const float f[4] = {v.x, v.y, v.z, v.w};
-    const uint32_t blk0 = i & ~31u, e0 = i & 31u;
+    return gemm_copy_code_halfs(rows, K) + (uint64_t)gemm_rows_padded(rows) * (gemm_k_padded(K) / 32) * 2;
+}
+// offset in halfs of the 8 halfs (token, k..k+7), k a multiple of 8, in a tile-ordered activation plane of padded width Kp
+__device__ __forceinline__ size_t gemm_x_offset(uint32_t token, uint32_t k, uint32_t Kp)
+{
+    return (((size_t)(token / kGemmTile) * (Kp / 8) + k / 8) * kGemmTile + token % kGemmTile) * 8;
+}
+
+__device__ __forceinline__ void gemm_split8(uint4 &h, uint4 &l, const float (&f)[8])
+{
+    uint32_t hw[4], lw[4];
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-        const uint16_t h = float_to_half_bits(f[j]);
-        const uint16_t l = float_to_half_bits(f[j] - half_bits_to_float(h));
-        int pos = (int)e0 + j;
-        if constexpr (QT == 4) {
-            const int hi = pos >= 16 ? 1 : 0, ee = pos & 15, ii = ee >> 2, b = ee & 3;
-            pos = 8 * ii + 2 * ((b & 1) * 2 + hi) + (b >> 1);
-        }
-        xh[(size_t)row * K + blk0 + pos] = h;
-        xl[(size_t)row * K + blk0 + pos] = l;
+        const uint16_t h0 = float_to_half_bits(f[2 * j]), h1 = float_to_half_bits(f[2 * j + 1]);
+        const uint16_t l0 = float_to_half_bits(f[2 * j] - half_bits_to_float(h0)), l1 = float_to_half_bits(f[2 * j + 1] - half_bits_to_float(h1));
+        hw[j] = (uint32_t)h0 | ((uint32_t)h1 << 16);
+        lw[j] = (uint32_t)l0 | ((uint32_t)l1 << 16);
     }
+    h = make_uint4(hw[0], hw[1], hw[2], hw[3]);
+    l = make_uint4(lw[0], lw[1], lw[2], lw[3]);
+}
+
+// Thread -> (token, chunk of 8 k) for the elementwise producers: a wave covers 8 tokens x 8 chunks, so that it reads
+// 256 consecutive bytes of each token's fp32 row and writes, per chunk, the 128 consecutive bytes of its 8 tokens.
+// grid (Kp / 64, n_pad / 32), 256 threads.
+__device__ __forceinline__ void gemm_producer_coords(uint32_t &token, uint32_t &k)
+{
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    token = blockIdx.y * 32 + wave * 8 + (lane >> 3);
+    k = blockIdx.x * 64 + (lane & 7) * 8;
+}
+
+// x[n][K] fp32 -> xh, xl (tile order, n_pad tokens x Kp; everything outside n x K is written as zero)
+__global__ __launch_bounds__(256) void split_half_kernel(uint16_t *__restrict__ xh, uint16_t *__restrict__ xl, const float *__restrict__ x, uint32_t n,
+                                                          uint32_t K, uint32_t Kp)
+{
+    uint32_t token, k;
+    gemm_producer_coords(token, k);
+    if (k >= Kp) return;
+    float f[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (token < n && k < K) {       // K is a multiple of 32: a chunk of 8 lies inside or outside
+        const float4 a = *reinterpret_cast<const float4 *>(x + (size_t)token * K + k), b = *reinterpret_cast<const float4 *>(x + (size_t)token * K + k + 4);
+        f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+    }
+    uint4 h, l;
+    gemm_split8(h, l, f);
+    const size_t o = gemm_x_offset(token, k, Kp);
+    *reinterpret_cast<uint4 *>(xh + o) = h;
+    *reinterpret_cast<uint4 *>(xl + o) = l;
+}
+
+// ff[n][F] = a * b / (exp(-b) + 1) (matmul_silu_ff.comp:96 with a = W3 x, b = W1 x), written as the two fp16 halves
+// the down projection's GEMM reads (same layout and grid as split_half_kernel)
+__global__ __launch_bounds__(256) void silu_split_kernel(uint16_t *__restrict__ xh, uint16_t *__restrict__ xl, const float *__restrict__ a,
+                                                          const float *__restrict__ b, uint32_t n, uint32_t K, uint32_t Kp)
+{
+    uint32_t token, k;
+    gemm_producer_coords(token, k);
+    if (k >= Kp) return;
+    float f[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (token < n && k < K) {
+        const float *pa = a + (size_t)token * K + k, *pb = b + (size_t)token * K + k;
+        const float4 a0 = *reinterpret_cast<const float4 *>(pa), a1 = *reinterpret_cast<const float4 *>(pa + 4);
+        const float4 b0 = *reinterpret_cast<const float4 *>(pb), b1 = *reinterpret_cast<const float4 *>(pb + 4);
+        const float av[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w}, bv[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+#pragma unroll
+        for (int j = 0; j < 8; j++) f[j] = av[j] * bv[j] / (__expf(-bv[j]) + 1.f);
+    }
+    uint4 h, l;
+    gemm_split8(h, l, f);
+    const size_t o = gemm_x_offset(token, k, Kp);
+    *reinterpret_cast<uint4 *>(xh + o) = h;
+    *reinterpret_cast<uint4 *>(xl + o) = l;
 }
 
 constexpr int kGemmMaxMats = 3;
 struct GemmArgs {
-    // up to three matrices of one shape and type applied to the same activations in one launch (blockIdx.z picks the
-    // matrix): q, k and v of a layer together fill the CUs that each alone leaves idle
-    float *outs[kGemmMaxMats];  // [n][ldo] each
-    const uint16_t *xh, *xl;  // [n_pad][K] fp16 halves of the activations, n_pad a multiple of 128
-    MatView ws[kGemmMaxMats];   // rows x K each
-    uint32_t n;             // tokens
-    uint32_t ldo;           // floats between output rows
-    int accumulate;         // out += instead of out =
-    // 0: blockIdx.z picks the matrix.  Otherwise the launch splits K: ws[] all name one matrix, slice z multiplies the
-    // K steps z*slice_steps .. (z+1)*slice_steps-1 into outs[z], and gemm_reduce_kernel adds the slices up (a matrix
-    // with few rows and a long K, like the down projection, fills the CUs that way)
-    uint32_t slice_steps;
+    // up to three matrices of one shape applied to the same activations in one launch: q, k and v of a layer together fill the CUs that each alone leaves idle
+    float *outs[kGemmMaxMats];          // [n][ldo] each
+    const uint16_t *xh, *xl;            // activation halves, tile order, n_pad x Kp
+    const uint16_t *w16[kGemmMaxMats];  // prompt copies (codes, then scales)
+    uint32_t rows, K;                   // of every matrix
+    uint32_t n;                         // tokens
+    uint32_t ldo;                       // floats between output rows
+    int accumulate;                     // out += instead of out =
+    // 0: nz matrices.  Otherwise the launch splits K: w16[] all name one matrix, slice y multiplies the
+    // K range y*slice_k .. (y+1)*slice_k-1 (slice_k a multiple of 64) into outs[y], and gemm_reduce_kernel adds the slices
+    // up (a matrix with few rows and a long K, like the down projection, fills the CUs that way)
+    uint32_t slice_k;
+    uint32_t nz;                        // matrices or slices in this launch
 };
 
 // out[n][ldo] (+)= p[0] + p[1] (+ p[2]), the K slices of one product, each [n][rows]; always summed in this order
@@ -93,382 +170,284 @@ __global__ void gemm_reduce_kernel(GemmReduceArgs a)
     *dst = s;
 }
 
-typedef _Float16 lv_h2 __attribute__((ext_vector_type(2)));
-
-// Position inside a 32-element block at which the weight halves of element e are stored in LDS, and therefore at
-// which the activation halves must be stored too (split_half_kernel).  q8_0: natural order.  q4_0: the order in
-// which whole dwords of codes unpack into pairs of fp16 — dword i, shift 4j holds elements (4i, 4i+2), (16+4i, 18+4i),
-// (4i+1, 4i+3), (17+4i, 19+4i) for j = 0..3 (byte b of a block carries element b in its low and b+16 in its high nibble).
+// The prompt copy of one matrix: codes as fp16 integers (q4_0: q - 8, q8_0: q) and scales as fp32, in the tile order
+// described at the top of this file.  One thread per (row of the padded matrix, block of the padded K); consecutive
+// threads take consecutive rows, so that every 16-byte chunk row they write is next to its neighbour's.
 template <int QT>
-__host__ __device__ constexpr int gemm_k_position(int e)
+__global__ __launch_bounds__(256) void expand_codes_kernel(uint16_t *__restrict__ dst, MatView m)
 {
-    if (QT != 4) return e;
-    const int hi = e >= 16 ? 1 : 0, ee = e & 15, i = ee >> 2, b = ee & 3;
-    const int j = (b & 1) * 2 + hi;
-    return 8 * i + 2 * j + (b >> 1);
-}
-
-// 16 codes of half a block (q8_0: 16 bytes; q4_0: 8 bytes, the two dwords whose nibbles unpack to positions
-// 16*half .. 16*half+15 of gemm_k_position order) -> 16 halfs at w, as the integers they are (q4_0: q - 8, q8_0: q):
-// 1024 + u has the fp16 bit pattern 0x6400 | u, and subtracting 1024 + offset is exact.  A block outside the matrix
-// is given the scale 0 by the caller, which removes it from the sum whatever codes were unpacked for it.
-template <int QT, typename CW>
-__device__ __forceinline__ void gemm_codes_half(uint16_t *w, const CW &c)
-{
-    uint32_t ph[8];
-    auto emit = [&](int slot, uint32_t packed_codes, _Float16 bias) {
-        // packed_codes: two halfs 0x6400 | u
-        union { uint32_t u; lv_h2 h; } cc, v;
-        cc.u = packed_codes;
-        const lv_h2 bb = {bias, bias};
-        v.h = cc.h - bb;                             // exact: small integers
-        ph[slot] = v.u;
-    };
-    if constexpr (QT == 4) {
-        const uint32_t q[2] = {c.x, c.y};
+    const uint32_t Kp = gemm_k_padded(m.cols), rows_pad = gemm_rows_padded(m.rows), nbp = Kp / 32, nb = m.cols / 32;
+    const uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t r = (uint32_t)(t % kGemmRows);
+    const uint64_t rest = t / kGemmRows;
+    const uint32_t blk = (uint32_t)(rest % nbp), rt = (uint32_t)(rest / nbp);
+    const uint32_t row = rt * kGemmRows + r;
+    if (row >= rows_pad) return;
+    const bool real = row < m.rows && blk < nb;
+    _Float16 v[32];
+    float d = 0.f;
+    if (real) {
+        const uint64_t sb = (uint64_t)row * nb + blk;
+        d = mat_scale(m, sb);
+        if constexpr (QT == 4) {
+            const uint4 c = m.codes[sb];        // byte b: element b in the low nibble, element b + 16 in the high one
+            const uint32_t q[4] = {c.x, c.y, c.z, c.w};
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+            for (int b = 0; b < 16; b++) {
+                const uint32_t byte = (q[b >> 2] >> (8 * (b & 3))) & 0xffu;
+                v[b] = (_Float16)((int)(byte & 15u) - 8);
+                v[b + 16] = (_Float16)((int)(byte >> 4) - 8);
+            }
+        } else {
+            const uint4 c0 = m.codes[sb * 2], c1 = m.codes[sb * 2 + 1];
+            const uint32_t q[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
 #pragma unroll
-            for (int j = 0; j < 4; j++) emit(4 * i + j, ((q[i] >> (4 * j)) & 0x000f000fu) | 0x64006400u, (_Float16)1032.f);
-    } else {
-        const uint32_t q[4] = {c.x, c.y, c.z, c.w};      // CW = uint4
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const uint32_t u = q[i] ^ 0x80808080u;   // int8 -> biased unsigned
-            // one byte permute per pair: bytes (u.b0, 0x64, u.b1, 0x64) and (u.b2, 0x64, u.b3, 0x64)
-            emit(2 * i, __builtin_amdgcn_perm(u, 0x64646464u, 0x00050004u), (_Float16)1152.f);
-            emit(2 * i + 1, __builtin_amdgcn_perm(u, 0x64646464u, 0x00070006u), (_Float16)1152.f);
+            for (int b = 0; b < 32; b++) v[b] = (_Float16)(int)(int8_t)((q[b >> 2] >> (8 * (b & 3))) & 0xffu);
         }
-    }
+    } else {
 #pragma unroll
-    for (int g = 0; g < 2; g++) *reinterpret_cast<uint4 *>(w + 8 * g) = make_uint4(ph[4 * g], ph[4 * g + 1], ph[4 * g + 2], ph[4 * g + 3]);
-}
-
-// ff[n][F] = a * b / (exp(-b) + 1) (matmul_silu_ff.comp:96 with a = W3 x, b = W1 x), written as the two fp16 halves
-// the down projection's GEMM reads (split_half_kernel's layout for weight type QT; rows n.. zero)
-template <int QT>
-__global__ void silu_split_kernel(uint16_t *__restrict__ xh, uint16_t *__restrict__ xl, const float *__restrict__ a, const float *__restrict__ b,
-                                  uint32_t n, uint32_t K)
-{
-    const uint32_t row = blockIdx.y;
-    const uint32_t i = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
-    if (i >= K) return;
-    float f[4] = {0.f, 0.f, 0.f, 0.f};
-    if (row < n) {
-        const float4 r1 = *reinterpret_cast<const float4 *>(a + (size_t)row * K + i), r2 = *reinterpret_cast<const float4 *>(b + (size_t)row * K + i);
-        f[0] = r1.x * r2.x / (__expf(-r2.x) + 1.f);
-        f[1] = r1.y * r2.y / (__expf(-r2.y) + 1.f);
-        f[2] = r1.z * r2.z / (__expf(-r2.z) + 1.f);
-        f[3] = r1.w * r2.w / (__expf(-r2.w) + 1.f);
+        for (int b = 0; b < 32; b++) v[b] = (_Float16)0.f;
     }
-    const uint32_t blk0 = i & ~31u, e0 = i & 31u;
+    const uint64_t nchunk = Kp / 8;
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-        const uint16_t h = float_to_half_bits(f[j]);
-        const uint16_t l = float_to_half_bits(f[j] - half_bits_to_float(h));
-        const int pos = gemm_k_position<QT>((int)e0 + j);
-        xh[(size_t)row * K + blk0 + pos] = h;
-        xl[(size_t)row * K + blk0 + pos] = l;
+    for (int c = 0; c < 4; c++) {
+        union { _Float16 h[8]; uint4 u; } pk;
+#pragma unroll
+        for (int e = 0; e < 8; e++) pk.h[e] = v[8 * c + e];
+        *reinterpret_cast<uint4 *>(dst + (((uint64_t)rt * nchunk + (uint64_t)blk * 4 + c) * kGemmRows + r) * 8) = pk.u;
     }
+    float *sc = reinterpret_cast<float *>(dst + gemm_copy_code_halfs(m.rows, m.cols));
+    sc[((uint64_t)rt * nbp + blk) * kGemmRows + r] = d;
 }
 
 // The steps between two GEMMs of a prompt batch as one pass over a token row: x += the K slices of the product
 // before (same order as gemm_reduce_kernel: slices first, then x), xn = normalize(x) * w (normalize_kernel's
-// arithmetic), and xn split in the two fp16 halves the next GEMM reads (split_half_kernel's layout for weight type QT).
-// One 256-thread workgroup per row of the padded batch; rows n.. are written as zeros.  dim <= 8192, a multiple of 4.
+// arithmetic), and xn split in the two fp16 halves the next GEMM reads (tile order, padded to Kp with zeros).
+// One 256-thread workgroup per row of the padded batch; rows n.. are written as zeros.  dim <= 8192, a multiple of 8.
+// Workgroups are dealt to the 8 XCDs in turn; the row a workgroup takes is chosen so that the 8 tokens whose chunks
+// share a 128-byte line are written through one XCD's L2.
 struct PrefillNormArgs {
     float *x;                              // [n][dim] residual stream, updated when nparts > 0
     const float *parts[kGemmMaxMats];      // [n][dim] each
     uint32_t nparts;
     const float *w;                        // norm weights
     float *xn;                             // [n][dim] or null: the normalised row as fp32 (for a GEMV-type consumer)
-    uint16_t *xh, *xl;                     // [n_pad][dim]
-    uint32_t dim, n;
+    uint16_t *xh, *xl;                     // tile order, n_pad x Kp
+    uint32_t dim, n, Kp;
 };
-template <int QT>
 __global__ __launch_bounds__(256) void prefill_norm_kernel(PrefillNormArgs a)
 {
     __shared__ float lds[4];
-    constexpr int PER = 8;
-    const uint32_t row = blockIdx.x, dim = a.dim, n4 = dim / 4;
+    constexpr int PER = 4;                 // chunks of 8 per thread
+    const uint32_t b = blockIdx.x, row = (b >> 6) * 64 + (b & 7) * 8 + ((b >> 3) & 7);     // n_pad is a multiple of 128
+    const uint32_t dim = a.dim, n8 = dim / 8;
     const bool live = row < a.n;
     const size_t ro = (size_t)(live ? row : 0) * dim;
-    float4 v[PER], wv[PER];
+    float v[PER][8], wv[PER][8];
 #pragma unroll
     for (int j = 0; j < PER; j++) {
         const uint32_t i = threadIdx.x + j * 256;
-        const bool ok = live && i < n4;
+        const bool ok = live && i < n8;
         const uint32_t ic = ok ? i : 0;
-        wv[j] = reinterpret_cast<const float4 *>(a.w)[i < n4 ? i : 0];
-        float4 x4 = reinterpret_cast<const float4 *>(a.x + ro)[ic];
-        if (a.nparts) {
-            float4 s4 = reinterpret_cast<const float4 *>(a.parts[0] + ro)[ic];
-            for (uint32_t q = 1; q < a.nparts; q++) {
-                const float4 p4 = reinterpret_cast<const float4 *>(a.parts[q] + ro)[ic];
-                s4.x += p4.x; s4.y += p4.y; s4.z += p4.z; s4.w += p4.w;
+#pragma unroll
+        for (int hf = 0; hf < 2; hf++) {
+            const float4 w4 = reinterpret_cast<const float4 *>(a.w)[(i < n8 ? i : 0) * 2 + hf];
+            wv[j][4 * hf] = w4.x; wv[j][4 * hf + 1] = w4.y; wv[j][4 * hf + 2] = w4.z; wv[j][4 * hf + 3] = w4.w;
+            float4 x4 = reinterpret_cast<const float4 *>(a.x + ro)[ic * 2 + hf];
+            if (a.nparts) {
+                float4 s4 = reinterpret_cast<const float4 *>(a.parts[0] + ro)[ic * 2 + hf];
+                for (uint32_t q = 1; q < a.nparts; q++) {
+                    const float4 p4 = reinterpret_cast<const float4 *>(a.parts[q] + ro)[ic * 2 + hf];
+                    s4.x += p4.x; s4.y += p4.y; s4.z += p4.z; s4.w += p4.w;
+                }
+                x4.x = s4.x + x4.x; x4.y = s4.y + x4.y; x4.z = s4.z + x4.z; x4.w = s4.w + x4.w;
+                if (ok) reinterpret_cast<float4 *>(a.x + ro)[ic * 2 + hf] = x4;
             }
-            x4.x = s4.x + x4.x; x4.y = s4.y + x4.y; x4.z = s4.z + x4.z; x4.w = s4.w + x4.w;
-            if (ok) reinterpret_cast<float4 *>(a.x + ro)[ic] = x4;
+            if (!ok) x4 = make_float4(0.f, 0.f, 0.f, 0.f);
+            v[j][4 * hf] = x4.x; v[j][4 * hf + 1] = x4.y; v[j][4 * hf + 2] = x4.z; v[j][4 * hf + 3] = x4.w;
         }
-        v[j] = ok ? x4 : make_float4(0.f, 0.f, 0.f, 0.f);
     }
     float s = 0.f;
 #pragma unroll
-    for (int j = 0; j < PER; j++) s += (v[j].x + v[j].y) + (v[j].z + v[j].w);
+    for (int j = 0; j < PER; j++) s += ((v[j][0] + v[j][1]) + (v[j][2] + v[j][3])) + ((v[j][4] + v[j][5]) + (v[j][6] + v[j][7]));
     const float mean = block_sum_256(s, lds) / (float)dim;
     float q = 0.f;
 #pragma unroll
     for (int j = 0; j < PER; j++) {
-        if (threadIdx.x + j * 256 < n4) {
-            const float c0 = v[j].x - mean, c1 = v[j].y - mean, c2 = v[j].z - mean, c3 = v[j].w - mean;
-            q = fmaf(c0, c0, q); q = fmaf(c1, c1, q); q = fmaf(c2, c2, q); q = fmaf(c3, c3, q);
+        if (threadIdx.x + j * 256 < n8) {
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const float c = v[j][e] - mean;
+                q = fmaf(c, c, q);
+            }
         }
     }
     const float inv = rsqrtf(block_sum_256(q, lds) / (float)dim);
+    const uint32_t chunks = a.Kp / 8;
 #pragma unroll
     for (int j = 0; j < PER; j++) {
         const uint32_t i = threadIdx.x + j * 256;
-        if (i >= n4) continue;
-        float f[4] = {(v[j].x * wv[j].x) * inv, (v[j].y * wv[j].y) * inv, (v[j].z * wv[j].z) * inv, (v[j].w * wv[j].w) * inv};
-        if (!live) f[0] = f[1] = f[2] = f[3] = 0.f;        // a padding row (its inv is not finite)
-        if (live && a.xn) reinterpret_cast<float4 *>(a.xn + ro)[i] = make_float4(f[0], f[1], f[2], f[3]);
-        const uint32_t e = i * 4, blk0 = e & ~31u, e0 = e & 31u;
-        uint16_t *hr = a.xh + (size_t)row * dim + blk0, *lr = a.xl + (size_t)row * dim + blk0;
+        if (i >= chunks) continue;
+        float f[8];
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            const uint16_t h = float_to_half_bits(f[k]);
-            const uint16_t l = float_to_half_bits(f[k] - half_bits_to_float(h));
-            const int pos = gemm_k_position<QT>((int)e0 + k);
-            hr[pos] = h;
-            lr[pos] = l;
+        for (int e = 0; e < 8; e++) f[e] = (live && i < n8) ? (v[j][e] * wv[j][e]) * inv : 0.f;   // padding rows and columns: zero
+        if (live && i < n8 && a.xn) {
+            reinterpret_cast<float4 *>(a.xn + ro)[i * 2] = make_float4(f[0], f[1], f[2], f[3]);
+            reinterpret_cast<float4 *>(a.xn + ro)[i * 2 + 1] = make_float4(f[4], f[5], f[6], f[7]);
         }
+        uint4 h, l;
+        gemm_split8(h, l, f);
+        const size_t o = gemm_x_offset(row, i * 8, a.Kp);
+        *reinterpret_cast<uint4 *>(a.xh + o) = h;
+        *reinterpret_cast<uint4 *>(a.xl + o) = l;
     }
 }
 
-// RM = weight rows per workgroup (128 or 64); tokens per workgroup: 128.  The four waves split the tile 2 x 2
-// (RM = 128: 64 tokens x 64 rows each) or 4 x 1 (RM = 64: 32 tokens x 64 rows each).  The narrow form doubles the
-// number of workgroups for matrices that would otherwise not fill 256 CUs.
-template <int QT, int RM, int NWV = 4, bool SF32 = false /* fp32 scale plane (file version 1) */, bool DB = false /* two LDS buffers */>
-__global__ __launch_bounds__(NWV * 64) void gemm_kernel(GemmArgs a)
+// One workgroup: 128 tokens x 256 weight rows over a range of K.  The grid enumerates (matrix or K slice, row tile, token
+// tile) so that the token tiles of one row tile run on one XCD (workgroups are dealt to the 8 XCDs in turn) and find its
+// weights in that XCD's L2, and so that the XCDs get equal numbers of workgroups.
+//
+// Pipeline.  Stage s (K step s: 16 KB of weights, 2 x 8 KB of activation halves, 1 KB of scales) is copied to LDS buffer
+// s % 4 by five direct loads per thread, issued three and a half steps before its MFMAs.  A wave holds the operands of
+// the step it multiplies in registers (twelve 16-byte reads); in the second half of a step it waits for the next
+// stage's loads, meets the other waves at the step's only barrier, lets the loads of stage s + 4 overwrite the buffer
+// of stage s (which every wave has by then read into registers), and reads the next step's operands between its MFMAs.
+// The scale multiply-adds of a 32 x 32 tile follow its last MFMA five issue slots later, four after each MFMA, so that
+// neither the matrix pipe nor the vector pipe waits for the other.
+__global__ __launch_bounds__(512) void gemm_kernel(GemmArgs a)
 {
-    constexpr int TN = kGemmTile;                 // tokens per workgroup
-    constexpr int WN = RM / 64;                   // waves along the rows
-    constexpr int WM = NWV / WN;                  // waves along the tokens
-    constexpr int NT = NWV * 64;                  // threads
-    constexpr int XP = TN * 8 / NT;               // 16-byte pieces of an activation half-tile per thread
-    constexpr int MT = TN / WM / 32;              // 32-token tiles per wave
-    constexpr int NBUF = DB ? 2 : 1;
-    __shared__ __attribute__((aligned(16))) uint16_t sXh_[NBUF][TN * kGemmLd], sXl_[NBUF][TN * kGemmLd], sW_[NBUF][RM * kGemmLd];
-    __shared__ float sD_[NBUF][2][RM];            // scale of (block of the step, row)
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave / WN, wn = wave % WN;
-    const uint32_t tok0 = blockIdx.y * TN, row0 = blockIdx.x * RM;
-    const MatView w = a.ws[blockIdx.z];
-    float *const out = a.outs[blockIdx.z];
-    const uint32_t K = w.cols, nb = K / 32, all_steps = (K + kGemmK - 1) / kGemmK;
-    // this workgroup's K steps: step0 .. step0 + steps - 1 (the host gives every slice at least one)
-    const uint32_t step0 = a.slice_steps ? blockIdx.z * a.slice_steps : 0;
-    const uint32_t steps = a.slice_steps ? min(a.slice_steps, all_steps - step0) : all_steps;
+    constexpr int TN = kGemmTile, RM = kGemmRows, NST = kGemmStages;
+    constexpr int LPS = 5;   // direct loads per thread per stage
+    extern __shared__ __attribute__((aligned(16))) uint8_t gemm_lds[];
+    uint8_t *const lds = gemm_lds;
+    const int tid = threadIdx.x, lane = tid & 63, l31 = lane & 31, lhi = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wn = wave & 3, wm = wave >> 2;
+    const uint32_t tok_tiles = (a.n + TN - 1) / TN, row_tiles = (a.rows + RM - 1) / RM;
+    // unit = (matrix or slice, row tile); unit u runs on XCD u % 8, its token tiles in consecutive slots of that XCD
+    const uint32_t L = blockIdx.x, xcd = L & 7, slot = L >> 3;
+    const uint32_t unit = (slot / tok_tiles) * 8 + xcd, tt = slot % tok_tiles;
+    if (unit >= row_tiles * a.nz) return;
+    const uint32_t z = unit / row_tiles, rt = unit % row_tiles;
+    const uint32_t Kp = gemm_k_padded(a.K), nchunk = Kp / 8, nblk = Kp / 32;
+    // this workgroup's K steps: step0 .. step0 + steps - 1, an even number (slices are multiples of 64, and so is Kp)
+    const uint32_t step0 = a.slice_k ? z * (a.slice_k / kGemmStep) : 0;
+    const uint32_t steps = a.slice_k ? min(a.slice_k / kGemmStep, nblk - step0) : nblk;
+    const uint8_t *w16 = reinterpret_cast<const uint8_t *>(a.w16[z]);
+    const uint8_t *gw = w16 + ((size_t)rt * nchunk * RM + tid) * 16;
+    const uint8_t *gs = w16 + gemm_copy_code_halfs(a.rows, a.K) * 2 + ((size_t)rt * nblk * RM + (wave & 3) * 64 + lane) * 4;
+    const uint8_t *gh = reinterpret_cast<const uint8_t *>(a.xh) + ((size_t)tt * nchunk * TN + tid) * 16;
+    const uint8_t *gl = reinterpret_cast<const uint8_t *>(a.xl) + ((size_t)tt * nchunk * TN + tid) * 16;
 
-    // this thread's share of the weights of a step: half h_w of block (2*step + b_w) of row r_w.  Every thread has one,
-    // and every load below is issued by every thread at every step (addresses are clamped, results discarded where
-    // there is nothing to load): the compiler can then count the loads in flight exactly and wait for the oldest set
-    // only, which a load under a condition would force it to give up.
-    static_assert(RM * 4 % NT == 0, "two threads per (row, block)");
-    constexpr int WP = RM * 4 / NT;               // (row, block, half) pieces per thread: rows r_w + (NT/4)*i
-    const int r_w = tid >> 2, b_w = (tid >> 1) & 1, h_w = tid & 1;
-    // this thread's 16-byte pieces of the activation tile of a step: token rows tid/8 + XR*i, halfs (tid%8)*8..+7
-    const int xr = tid >> 3, xc = (tid & 7) * 8;
-    constexpr int XR = NT / 8;                    // token rows covered per piece index
-    const uint32_t steps2 = (steps + 1) & ~1u;    // the loop takes two steps at a time; a step past the end multiplies zeros
-
-    // two register sets: the loads of step s + 2 are in flight while step s is multiplied (one step of MFMAs is
-    // shorter than a trip to memory)
-    using CodeWords = typename std::conditional<QT == 8, uint4, uint2>::type;     // 16 codes
-    // register sets of the two-buffer form: three (loads two and three steps ahead) where they fit; the 256-row q4_0
-    // form would spill with three and runs with two (loads two steps ahead, issued after the unpacking instead of
-    // before it), which costs q8_0 8 % but is 12 % faster than the 128-row form for q4_0
-    constexpr int kSets = (QT == 4 && RM == 256) ? 2 : 3;
-    struct Staged {
-        CodeWords c[WP];
-        uint32_t dbits[WP]; // raw scale word
-        bool wvalid[WP];
-        uint4 gh[XP], gl[XP];
-    } pre[DB ? kSets : 2];
-    auto fetch = [&](Staged &p, uint32_t step) {
-        const bool real = step < steps;
-        const uint32_t sc = step0 + (real ? step : steps - 1);
-        const uint32_t blk = 2 * sc + b_w;
-#pragma unroll
-        for (int i = 0; i < WP; i++) {
-            const uint32_t wrow = row0 + r_w + (NT / 4) * i;
-            p.wvalid[i] = real && wrow < w.rows && blk < nb;
-            const size_t sb = (size_t)(p.wvalid[i] ? wrow : 0) * nb + (p.wvalid[i] ? blk : 0);
-            if constexpr (QT == 8) {
-                p.c[i] = w.codes[sb * 2 + h_w];
-            } else {
-                p.c[i] = reinterpret_cast<const uint2 *>(w.codes)[sb * 2 + h_w];
-            }
-            if constexpr (SF32) p.dbits[i] = __float_as_uint(w.scales_f32[sb]);
-            else p.dbits[i] = w.scales[sb];
-        }
-        const uint32_t k = sc * kGemmK + xc;
-        const bool kok = real && k < K;
-#pragma unroll
-        for (int i = 0; i < XP; i++) {
-            const size_t off = (size_t)(tok0 + xr + XR * i) * K + (kok ? k : 0);
-            p.gh[i] = *reinterpret_cast<const uint4 *>(a.xh + off);
-            p.gl[i] = *reinterpret_cast<const uint4 *>(a.xl + off);
-            if (!kok) p.gh[i] = p.gl[i] = make_uint4(0, 0, 0, 0);
-        }
+    // the five loads of this thread for stage s; past the end a harmless repeat of the last stage into a free buffer, which
+    // keeps the number of loads in flight the same in every step
+    auto issue = [&](uint32_t s) {
+        const size_t sc = step0 + (s < steps ? s : steps - 1);
+        uint8_t *buf = lds + (s % NST) * kGemmStageBytes;
+        const uint8_t *pw = gw + sc * kGemmWBytes;
+        __builtin_amdgcn_global_load_lds((lv_glb_void *)pw, (lv_lds_void *)(buf + wave * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((lv_glb_void *)(pw + 8192), (lv_lds_void *)(buf + 8192 + wave * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((lv_glb_void *)(gh + sc * kGemmXBytes), (lv_lds_void *)(buf + kGemmWBytes + wave * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((lv_glb_void *)(gl + sc * kGemmXBytes), (lv_lds_void *)(buf + kGemmWBytes + kGemmXBytes + wave * 1024), 16, 0, 0);
+        // scales: 1 KB, four waves' worth of 4-byte loads; waves 4..7 repeat them (same bytes to the same place)
+        __builtin_amdgcn_global_load_lds((lv_glb_void *)(gs + sc * kGemmScBytes), (lv_lds_void *)(buf + kGemmWBytes + 2 * kGemmXBytes + (wave & 3) * 256), 4, 0, 0);
     };
 
-    lv_f16v acc[MT][2];
+    lv_f16v acc[2][2];
 #pragma unroll
-    for (int i = 0; i < MT; i++)
+    for (int i = 0; i < 2; i++)
 #pragma unroll
         for (int j = 0; j < 2; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+    const lv_f16v zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
-    fetch(pre[0], 0);
-    // registers -> LDS buffer `buf`
-    auto stage = [&](const Staged &P, int buf) {
-        uint16_t *sXh = sXh_[buf], *sXl = sXl_[buf], *sW = sW_[buf];
+    struct Frag { lv_h8 xh[2][2], xl[2][2], wc[2][2]; float d[2]; };
+    // one sixth of the operand reads of a stage (two 16-byte reads), the scales with the last
+    auto read_part = [&](Frag &f, const uint8_t *buf, int part) {
+        const uint8_t *sW = buf, *sH = buf + kGemmWBytes, *sL = buf + kGemmWBytes + kGemmXBytes;
+        const int kk = part & 1, what = part >> 1;      // what: 0 weights, 1 low halves, 2 high halves
+        const int chunk = 2 * kk + lhi;
 #pragma unroll
-        for (int i = 0; i < WP; i++) {
-            const int r = r_w + (NT / 4) * i;
-            gemm_codes_half<QT>(sW + r * kGemmLd + b_w * 32 + h_w * 16, P.c[i]);
-            if (h_w == 0) sD_[buf][b_w][r] = !P.wvalid[i] ? 0.f : SF32 ? __uint_as_float(P.dbits[i]) : half_bits_to_float((uint16_t)P.dbits[i]);
+        for (int t = 0; t < 2; t++) {
+            if (what == 0) f.wc[kk][t] = *reinterpret_cast<const lv_h8 *>(sW + (chunk * RM + wn * 64 + t * 32 + l31) * 16);
+            if (what == 1) f.xl[kk][t] = *reinterpret_cast<const lv_h8 *>(sL + (chunk * TN + wm * 64 + t * 32 + l31) * 16);
+            if (what == 2) f.xh[kk][t] = *reinterpret_cast<const lv_h8 *>(sH + (chunk * TN + wm * 64 + t * 32 + l31) * 16);
         }
+        if (part == 5) {
+            const float *sD = reinterpret_cast<const float *>(buf + kGemmWBytes + 2 * kGemmXBytes);
 #pragma unroll
-        for (int i = 0; i < XP; i++) {
-            *reinterpret_cast<uint4 *>(sXh + (xr + XR * i) * kGemmLd + xc) = P.gh[i];
-            *reinterpret_cast<uint4 *>(sXl + (xr + XR * i) * kGemmLd + xc) = P.gl[i];
-        }
-    };
-    // the step held by LDS buffer `buf` into the accumulators
-    auto multiply = [&](int buf) {
-        const uint16_t *sXh = sXh_[buf], *sXl = sXl_[buf], *sW = sW_[buf];
-#pragma unroll
-        for (int b = 0; b < kGemmK / 32; b++) {          // the two quant blocks of the step
-            lv_f16v blk[MT][2];
-#pragma unroll
-            for (int i = 0; i < MT; i++)
-#pragma unroll
-                for (int j = 0; j < 2; j++)
-#pragma unroll
-                    for (int r = 0; r < 16; r++) blk[i][j][r] = 0.f;
-#pragma unroll
-            for (int kk = 2 * b; kk < 2 * b + 2; kk++) {
-                const int ko = kk * 16 + (lane >> 5) * 8;
-                lv_h8 xh[MT], xl[MT], wc[2];
-#pragma unroll
-                for (int t = 0; t < MT; t++) {
-                    const int xrow = (wm * MT + t) * 32 + (lane & 31);
-                    xh[t] = *reinterpret_cast<const lv_h8 *>(sXh + xrow * kGemmLd + ko);
-                    xl[t] = *reinterpret_cast<const lv_h8 *>(sXl + xrow * kGemmLd + ko);
-                }
-#pragma unroll
-                for (int t = 0; t < 2; t++) {
-                    const int wr = wn * 64 + t * 32 + (lane & 31);
-                    wc[t] = *reinterpret_cast<const lv_h8 *>(sW + wr * kGemmLd + ko);
-                }
-                // product by product over all tiles: consecutive MFMAs do not wait for each other's accumulator
-#pragma unroll
-                for (int i = 0; i < MT; i++)
-#pragma unroll
-                    for (int j = 0; j < 2; j++) blk[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xl[i], wc[j], blk[i][j], 0, 0, 0);
-#pragma unroll
-                for (int i = 0; i < MT; i++)
-#pragma unroll
-                    for (int j = 0; j < 2; j++) blk[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh[i], wc[j], blk[i][j], 0, 0, 0);
-            }
-            // times the block's scale: a lane's sixteen results of a tile belong to one weight row
-#pragma unroll
-            for (int j = 0; j < 2; j++) {
-                const float d = sD_[buf][b][wn * 64 + j * 32 + (lane & 31)];
-#pragma unroll
-                for (int i = 0; i < MT; i++)
-#pragma unroll
-                    for (int r = 0; r < 16; r++) acc[i][j][r] = fmaf(blk[i][j][r], d, acc[i][j][r]);
-            }
+            for (int j = 0; j < 2; j++) f.d[j] = sD[wn * 64 + j * 32 + l31];
         }
     };
-    if constexpr (!DB) {
-        // one buffer: unpack, barrier, multiply, barrier; two register sets, the loads of step s + 2 in flight
-        fetch(pre[1], 1);
-        auto one_step = [&](Staged &P, uint32_t step) {
-            stage(P, 0);
-            __syncthreads();
-            fetch(P, step + 2);
-            multiply(0);
-            __syncthreads();
-        };
-        for (uint32_t step = 0; step < steps2; step += 2) {
-            one_step(pre[0], step);
-            one_step(pre[1], step + 1);
-        }
-    } else {
-        // two buffers, one barrier per step: step s + 1 is unpacked into one buffer while step s is multiplied out of
-        // the other, so a wave's unpacking sits between its MFMAs; three register sets, the loads of steps s + 2 and
-        // s + 3 in flight
-        if constexpr (kSets == 2) {
-            fetch(pre[1], 1);
-            stage(pre[0], 0);
-            fetch(pre[0], 2);
-            __syncthreads();
-            auto it2 = [&](uint32_t s, Staged &next) {
-                stage(next, (s + 1) & 1);
-                fetch(next, s + 3);
-                multiply(s & 1);
-                __syncthreads();
-            };
-            for (uint32_t s = 0; s < steps; s += 2) {
-                it2(s, pre[1]);
-                if (s + 1 >= steps) break;
-                it2(s + 1, pre[0]);
+    lv_f16v c3 = zero;              // tile 3 of the step before and the last four values of its tile 2: their scaling into
+    float c2[4] = {0.f, 0.f, 0.f, 0.f}, dc[2] = {0.f, 0.f};   // the result is interleaved with this step's first MFMAs
+    auto step = [&](uint32_t s, const Frag &cur, Frag &nxt) {
+        lv_f16v T[4];
+#pragma unroll
+        for (int g = 0; g < 16; g++) {
+            const int t = g >> 2, m = g & 3, i = t >> 1, j = t & 1;
+            if (g == 8) {
+                // stage s + 1 has landed for everyone, and everyone holds stage s in registers: its buffer takes stage s + 4
+                asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NST - 2) * LPS) : "memory");
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+                issue(s + NST);
+                __builtin_amdgcn_sched_barrier(0);
             }
-        } else {
-        fetch(pre[1], 1);
-        fetch(pre[kSets - 1], 2);
-        stage(pre[0], 0);
-        __syncthreads();
-        // mine: the set that held step s (in LDS since the iteration before), reloaded with step s + 3;
-        // next: the set holding step s + 1
-        auto iteration = [&](uint32_t s, Staged &mine, const Staged &next) {
-            fetch(mine, s + 3);
-            stage(next, (s + 1) & 1);
-            multiply(s & 1);
-            __syncthreads();
-        };
-        for (uint32_t s = 0; s < steps; s += 6) {
-            iteration(s, pre[0], pre[1]);
-            if (s + 1 >= steps) break;
-            iteration(s + 1, pre[1], pre[kSets - 1]);
-            if (s + 2 >= steps) break;
-            iteration(s + 2, pre[kSets - 1], pre[0]);
-            if (s + 3 >= steps) break;
-            iteration(s + 3, pre[0], pre[1]);
-            if (s + 4 >= steps) break;
-            iteration(s + 4, pre[1], pre[kSets - 1]);
-            if (s + 5 >= steps) break;
-            iteration(s + 5, pre[kSets - 1], pre[0]);
+            const lv_h8 &xa = m < 2 ? cur.xl[m & 1][i] : cur.xh[m & 1][i];
+            if (m == 0) T[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xa, cur.wc[0][j], zero, 0, 0, 0);
+            else T[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xa, cur.wc[m & 1][j], T[t], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (g == 0) {
+#pragma unroll
+                for (int r = 0; r < 4; r++) acc[1][0][12 + r] = fmaf(c2[r], dc[0], acc[1][0][12 + r]);
+            } else if (g <= 4) {
+#pragma unroll
+                for (int r = 4 * (g - 1); r < 4 * g; r++) acc[1][1][r] = fmaf(c3[r], dc[1], acc[1][1][r]);
+            } else {
+                const int q = g - 5, pt = q >> 2;
+#pragma unroll
+                for (int r = 4 * (q & 3); r < 4 * (q & 3) + 4; r++) acc[pt >> 1][pt & 1][r] = fmaf(T[pt][r], cur.d[pt & 1], acc[pt >> 1][pt & 1][r]);
+            }
+            if (g >= 8 && g < 14) read_part(nxt, lds + ((s + 1) % NST) * kGemmStageBytes, g - 8);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        }
+#pragma unroll
+        for (int r = 0; r < 4; r++) c2[r] = T[2][12 + r];
+        c3 = T[3];
+        dc[0] = cur.d[0]; dc[1] = cur.d[1];
+    };
+    Frag FA, FB;
+#pragma unroll
+    for (int s = 0; s < NST; s++) issue(s);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NST - 1) * LPS) : "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int p = 0; p < 6; p++) read_part(FA, lds, p);
+    for (uint32_t s = 0; s < steps; s += 2) {
+        step(s, FA, FB);
+        step(s + 1, FB, FA);
     }
+#pragma unroll
+    for (int r = 0; r < 4; r++) acc[1][0][12 + r] = fmaf(c2[r], dc[0], acc[1][0][12 + r]);
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[1][1][r] = fmaf(c3[r], dc[1], acc[1][1][r]);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // the repeats past the end have landed before the workgroup gives up its LDS
 
     // D[i][j]: i = token within the 32-tile, j = weight row; lane l holds j = l%32 and, in register r,
     // i = 8*(r/4) + 4*(l/32) + r%4
+    float *const out = a.outs[z];
 #pragma unroll
-    for (int ti = 0; ti < MT; ti++)
+    for (int ti = 0; ti < 2; ti++)
 #pragma unroll
         for (int tj = 0; tj < 2; tj++) {
-            const uint32_t m = row0 + wn * 64 + tj * 32 + (lane & 31);
+            const uint32_t m = rt * RM + wn * 64 + tj * 32 + l31;
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const uint32_t n = tok0 + (wm * MT + ti) * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
-                if (n < a.n && m < w.rows) {
+                const uint32_t n = tt * TN + wm * 64 + ti * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
+                if (n < a.n && m < a.rows) {
                     float *dst = out + (size_t)n * a.ldo + m;
                     *dst = a.accumulate ? *dst + acc[ti][tj][r] : acc[ti][tj][r];
                 }
