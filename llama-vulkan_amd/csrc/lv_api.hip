@@ -767,19 +767,18 @@ static int launch_gemm_multi(hipStream_t st, float *const outs[], uint32_t ldo, 
     return dispatch_gemm(st, a, *ws[0], (uint32_t)nmat);
 }
 
-// Into how many K slices to cut a product whose 128 x 256 output tiles alone number `tiles`: the count (1..3) that
-// leaves the fewest CU-rounds idle, the smaller count unless a larger one fills them clearly better.  A slice keeps
-// at least 16 K steps.
-static uint32_t gemm_k_slices(uint32_t tiles, uint32_t k_steps)
+// Into how many K slices (1..4) to cut a product of `row_tiles` x `token_tiles` output tiles over `k_steps` steps of 64.
+// gemm_kernel deals (slice, row tile) units to the 8 XCDs in turn, each unit's token tiles to CUs of its XCD (32 a
+// round); the cost of a choice is its rounds times the steps of a slice, plus two steps per extra slice for the pass
+// that adds the slices up.  A slice keeps at least 16 steps.
+static uint32_t gemm_k_slices(uint32_t row_tiles, uint32_t token_tiles, uint32_t k_steps)
 {
-    constexpr uint32_t cus = 256;
-    uint32_t best = 1;
-    double best_fill = 0;
+    uint32_t best = 1, best_cost = ~0u;
     for (uint32_t s = 1; s <= (uint32_t)kGemmMaxMats; s++) {
         if (s > 1 && k_steps / s < 16) break;
-        const uint32_t wgs = tiles * s, rounds = (wgs + cus - 1) / cus;
-        const double fill = (double)wgs / ((double)rounds * cus);
-        if (fill > best_fill + 0.05) { best_fill = fill; best = s; }
+        const uint32_t per_xcd = (row_tiles * s + 7) / 8 * token_tiles, rounds = (per_xcd + 31) / 32;
+        const uint32_t cost = rounds * ((k_steps + s - 1) / s) + 2 * (s - 1);
+        if (cost < best_cost) { best_cost = cost; best = s; }
     }
     return best;
 }
@@ -801,7 +800,7 @@ static uint32_t gemm_slices_for(const lv_matrix &w, uint32_t n, uint32_t ldo)
 {
     const uint32_t rows = w.view.rows, k_steps = (w.view.cols + kGemmK - 1) / kGemmK;
     const uint32_t token_tiles = (n + kGemmTile - 1) / kGemmTile;
-    return (rows % 4 || ldo % 4) ? 1 : gemm_k_slices((rows + kGemmRows - 1) / kGemmRows * token_tiles, k_steps);
+    return (rows % 4 || ldo % 4) ? 1 : gemm_k_slices((rows + kGemmRows - 1) / kGemmRows, token_tiles, k_steps);
 }
 
 // one matrix, activations already split, K cut in slices when that fills the CUs better: the slices go to parts[]
@@ -862,7 +861,7 @@ extern "C" int lv_kernel_gemm(lv_ctx *c, float *out, const lv_matrix *w, const f
     if (e != hipSuccess) return fail(LV_ERR_OOM, "lv_kernel_gemm: workspace");
     uint16_t *xh = ws + w_halfs, *xl = xh + halfs;
     float *p0 = reinterpret_cast<float *>(xl + halfs);
-    float *const parts[kGemmMaxMats] = {p0, p0 + part, p0 + 2 * part};
+    float *const parts[kGemmMaxMats] = {p0, p0 + part, p0 + 2 * part, p0 + 3 * part};
     lv_matrix wm = *w;
     int rc = LV_OK;
     if (!wm.h16) {
@@ -1643,7 +1642,7 @@ static int record_prefill(lv_session *s, uint32_t idx0, uint32_t n, bool with_he
     const dim3 kv_grid((D + 255) / 256, n);
     // q, k and v buffers of a layer are free once attention has run: they take the K slices of the output projection
     // and of the down projection; `pending` of them wait to be added to the residual stream by the next norm
-    float *const parts[kGemmMaxMats] = {s->pf_q, s->pf_k, s->pf_v};
+    float *const parts[kGemmMaxMats] = {s->pf_q, s->pf_k, s->pf_v, s->pf_vo};
     uint32_t pending = 0;
     for (uint32_t li = 0; li < hp.layers; li++) {
         const LayerWeights &lw = m->layers[li];

@@ -128,9 +128,9 @@ __global__ __launch_bounds__(256) void silu_split_kernel(uint16_t *__restrict__ 
     *reinterpret_cast<uint4 *>(xl + o) = l;
 }
 
-constexpr int kGemmMaxMats = 3;
+constexpr int kGemmMaxMats = 4;
 struct GemmArgs {
-    // up to three matrices of one shape applied to the same activations in one launch: q, k and v of a layer together fill the CUs that each alone leaves idle
+    // up to four matrices of one shape applied to the same activations in one launch: q, k and v of a layer together fill the CUs that each alone leaves idle
     float *outs[kGemmMaxMats];          // [n][ldo] each
     const uint16_t *xh, *xl;            // activation halves, tile order, n_pad x Kp
     const uint16_t *w16[kGemmMaxMats];  // prompt copies (codes, then scales)
@@ -145,7 +145,7 @@ struct GemmArgs {
     uint32_t nz;                        // matrices or slices in this launch
 };
 
-// out[n][ldo] (+)= p[0] + p[1] (+ p[2]), the K slices of one product, each [n][rows]; always summed in this order
+// out[n][ldo] (+)= p[0] + p[1] (+ p[2] + p[3]), the K slices of one product, each [n][rows]; always summed in this order
 struct GemmReduceArgs {
     float *out;
     const float *parts[kGemmMaxMats];
