@@ -114,6 +114,9 @@ struct MegaArgs {
 // Optional phase timestamps (built only with -DLV_MEGA_TIMING): workgroup 0 records the 100 MHz wall clock at
 // every phase boundary of layers 0..3 into status[16 + ...].
 #ifdef LV_MEGA_TIMING
+#ifndef LV_MEGA_TIMING_WG
+#define LV_MEGA_TIMING_WG 0
+#endif
 #define MEGA_STAMP(idx)                                                                                        \
     do {                                                                                                       \
         if (blockIdx.x == LV_MEGA_TIMING_WG && threadIdx.x == 0 && layer < 4)                                  \

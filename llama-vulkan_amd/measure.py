@@ -2,7 +2,9 @@
 """Measurements of the decode path beyond the headline bench: one JSON line per case.
 
     python llama-vulkan_amd/measure.py gemv          isolated dequant-fused GEMVs at the 7B shapes, q4_0 and q8_0
+    python llama-vulkan_amd/measure.py attention     the one-token attention kernel by itself (7B heads) over 512 and 2048 cache rows
     python llama-vulkan_amd/measure.py decode-q8     7B q8_0, cache positions 1920..2047 (128 greedy steps)
+    python llama-vulkan_amd/measure.py decode-q8-graph    the same on the hipGraph of the operator chain (attention_kernel over 2048 rows)
     python llama-vulkan_amd/measure.py decode-13b    13B q4_0, 32-token prompt + 256 greedy steps (persistent kernel)
     python llama-vulkan_amd/measure.py decode-13b-graph   the same on the hipGraph of the operator chain
     python llama-vulkan_amd/measure.py decode-7b-graph    7B q4_0, positions 444..511 on the hipGraph of the operator chain
@@ -10,6 +12,8 @@
     python llama-vulkan_amd/measure.py prefill-7b    7B q4_0, the same
     python llama-vulkan_amd/measure.py prefill-13b-q4  13B q4_0, the same
     python llama-vulkan_amd/measure.py gemm          isolated 512-token GEMMs at the 13B shapes, q8_0 (for kernel traces and counters)
+    python llama-vulkan_amd/measure.py handover      phases of the persistent kernel inside a layer (7B q4_0, position 511; timing build)
+    python llama-vulkan_amd/measure.py handover-q8   the same for 7B q8_0 at position 2047
     python llama-vulkan_amd/measure.py copy          1 GiB device-to-device copy: achievable bandwidth, counter calibration
     python llama-vulkan_amd/measure.py all
 
@@ -78,6 +82,40 @@ def gemv_cases(ctx, report=emit):
 
 def quiet(**kw):
     return kw
+
+
+def attention_cases(ctx, report=emit):
+    """reference: mhsa.comp + softmax.comp + kqv_matching.comp for one query.  32 heads of 128 at the last row of a 512- and
+    of a 2048-row cache; algorithmic bytes = the fp16 K and V rows 0..pos (4 * (pos + 1) * dim bytes) plus q in and out.
+    Sixteen caches in turn (0.5 / 2 GB), so that the rows come from HBM."""
+    import numpy as np
+    out_cases = []
+    heads, rot = 32, 128
+    dim = heads * rot
+    for backlog in (512, 2048):
+        pos = backlog - 1
+        ncache = 16
+        rng = np.random.default_rng(backlog)
+        host = (rng.standard_normal((backlog, dim)) * 0.5).astype(np.float16)
+        ks = [ctx.to_device(host) for _ in range(ncache)]
+        vs = [ctx.to_device(host) for _ in range(ncache)]
+        q = ctx.to_device(lva.synth_normal(1, dim, seed=3))
+        out = ctx.zeros(dim * 4)
+        for i in range(ncache):
+            lva.check(ctx.lib.lv_kernel_attention(ctx.h, out, ks[i], vs[i], q, pos, backlog, heads, rot, 1))
+        ctx.sync()
+        iters = 20
+        ctx.timer_start()
+        for _ in range(iters):
+            for i in range(ncache):
+                lva.check(ctx.lib.lv_kernel_attention(ctx.h, out, ks[i], vs[i], q, pos, backlog, heads, rot, 1))
+        us = ctx.timer_stop() * 1e3 / (iters * ncache)
+        nbytes = 4 * (pos + 1) * dim + 8 * dim
+        out_cases.append(report(case="attention", heads=heads, head_size=rot, rows=pos + 1, us=round(us, 2), algorithmic_bytes=nbytes,
+                                GBps=round(nbytes / us / 1e3, 1), frac_of_peak=round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)))
+        for b in ks + vs + [q, out]:
+            ctx.free(b)
+    return out_cases
 
 
 def copy_case(ctx):
@@ -170,6 +208,45 @@ def prefill_case(ctx, case, name, wtype, report=emit):
     return r
 
 
+def handover_case(name, wtype, seed, backlog, last):
+    """Loads the timing build of the library (libllava_hip_timing.so, -DLV_MEGA_TIMING: workgroup 0 of the persistent kernel
+    writes the 100 MHz wall clock at every phase boundary of layers 0..3) and prints, for the decode step at position
+    `last`, the time between the boundaries, averaged over 16 launches and the four layers.  acq = waiting for and fetching
+    the vector the workgroups before handed over; the rest is the phase's own work."""
+    import ctypes as C
+    import numpy as np
+    lva._libs["libllava_hip.so"] = C.CDLL(os.path.join(HERE, "libllava_hip_timing.so"), mode=C.RTLD_GLOBAL)
+    ctx = lva.Context(0)
+    shape = SHAPES["7b"]
+    model = lva.Model(ctx, model_file("7b", wtype, seed))
+    s = lva.Session(model, backlog)
+    first = last - 7
+    s.begin(lva.synth_tokens(first, 3, shape["vocab"], seed=seed), 0)
+    tok = s.argmax()
+    for pos in range(first, last):
+        s.begin([tok], pos)
+        tok = s.argmax()
+    ctx.lib.lv_debug_status_words.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32]
+    names = ["A acq (x)", "A norm+QKV", "B acq (q,k,v)", "B attention", "B' combine", "C acq (o)", "C Wo", "D acq (x)", "D norm+gate.up", "E acq (ff)", "E W2"]
+    acc, ms = np.zeros(len(names)), []
+    reps = 16
+    for _ in range(reps):
+        s.timer_start()
+        s.begin([tok], last)
+        ms.append(s.timer_stop())
+        words = np.zeros(256, dtype=np.uint32)
+        lva.check(ctx.lib.lv_debug_status_words(s.h, words.ctypes.data_as(C.c_void_p), 256))
+        for layer in range(4):
+            t = words[16 + layer * 16: 16 + layer * 16 + 12].astype(np.int64)
+            acc += np.diff(t) * 0.01 / (4 * reps)                      # 100 MHz ticks -> us
+    emit(case=name, wtype="q4_0" if wtype == lva.LV_Q4_0 else "q8_0", position=last, kernel_ms=round(float(np.mean(ms)), 4),
+         layer_us=round(float(acc.sum()), 2), phases_us={n: round(float(v), 2) for n, v in zip(names, acc)},
+         handover_us=round(float(acc[[0, 2, 4, 5, 7, 9]].sum()), 2), work_us=round(float(acc[[1, 3, 6, 8, 10]].sum()), 2))
+    s.close()
+    model.close()
+    ctx.close()
+
+
 def gemm_cases(ctx):
     """lv_kernel_gemm allocates its workspace and splits the activations in every call, so the time of a call is not the
     kernel's: this case exists to put gemm_kernel launches of known shape under rocprofv3 (kernel trace, counters)"""
@@ -191,6 +268,10 @@ def gemm_cases(ctx):
 
 def main():
     which = sys.argv[1] if len(sys.argv) > 1 else "all"
+    if which == "handover":
+        return handover_case("handover", lva.LV_Q4_0, 0, 512, 511)
+    if which == "handover-q8":
+        return handover_case("handover-q8", lva.LV_Q8_0, 1, 2048, 2047)
     ctx = lva.Context(0)
     name, cus, hbm = ctx.info()
     emit(case="device", name=name, compute_units=cus, hbm_GiB=hbm >> 30)
@@ -198,10 +279,14 @@ def main():
         copy_case(ctx)
     if which in ("gemv", "all"):
         gemv_cases(ctx)
+    if which in ("attention", "all"):
+        attention_cases(ctx)
     if which == "gemm":
         gemm_cases(ctx)
     if which in ("decode-q8", "all"):
         decode_case(ctx, "decode-q8", "7b", lva.LV_Q8_0, 1, 2048, 1916, 128)
+    if which in ("decode-q8-graph", "all"):
+        decode_case(ctx, "decode-q8-graph", "7b", lva.LV_Q8_0, 1, 2048, 1916, 128, force_path=lva.PATH_GRAPH)
     if which in ("decode-13b", "all"):
         decode_case(ctx, "decode-13b", "13b", lva.LV_Q4_0, 2, 512, 32, 256)
     if which in ("decode-13b-graph", "all"):
