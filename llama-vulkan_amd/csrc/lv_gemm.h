@@ -308,7 +308,7 @@ __global__ __launch_bounds__(256) void prefill_norm_kernel(PrefillNormArgs a)
 // weights in that XCD's L2, and so that the XCDs get equal numbers of workgroups.
 //
 // Pipeline.  Stage s (K step s: 16 KB of weights, 2 x 8 KB of activation halves, 1 KB of scales) is copied to LDS buffer
-// s % 4 by five direct loads per thread, issued three and a half steps before its MFMAs.  A wave holds the operands of
+// s % 4 by five direct loads per thread, issued three to three and a half steps before its MFMAs.  A wave holds the operands of
 // the step it multiplies in registers (twelve 16-byte reads); in the second half of a step it waits for the next
 // stage's loads, meets the other waves at the step's only barrier, lets the loads of stage s + 4 overwrite the buffer
 // of stage s (which every wave has by then read into registers), and reads the next step's operands between its MFMAs.
@@ -339,18 +339,18 @@ __global__ __launch_bounds__(512) void gemm_kernel(GemmArgs a)
     const uint8_t *gh = reinterpret_cast<const uint8_t *>(a.xh) + ((size_t)tt * nchunk * TN + tid) * 16;
     const uint8_t *gl = reinterpret_cast<const uint8_t *>(a.xl) + ((size_t)tt * nchunk * TN + tid) * 16;
 
-    // the five loads of this thread for stage s; past the end a harmless repeat of the last stage into a free buffer, which
-    // keeps the number of loads in flight the same in every step
-    auto issue = [&](uint32_t s) {
+    // load p (0..4) of this thread's five for stage s; past the end a harmless repeat of the last stage into a free buffer,
+    // which keeps the number of loads in flight the same in every step
+    auto issue_one = [&](uint32_t s, int p) {
         const size_t sc = step0 + (s < steps ? s : steps - 1);
         uint8_t *buf = lds + (s % NST) * kGemmStageBytes;
         const uint8_t *pw = gw + sc * kGemmWBytes;
-        __builtin_amdgcn_global_load_lds((lv_glb_void *)pw, (lv_lds_void *)(buf + wave * 1024), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds((lv_glb_void *)(pw + 8192), (lv_lds_void *)(buf + 8192 + wave * 1024), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds((lv_glb_void *)(gh + sc * kGemmXBytes), (lv_lds_void *)(buf + kGemmWBytes + wave * 1024), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds((lv_glb_void *)(gl + sc * kGemmXBytes), (lv_lds_void *)(buf + kGemmWBytes + kGemmXBytes + wave * 1024), 16, 0, 0);
+        if (p == 0) __builtin_amdgcn_global_load_lds((lv_glb_void *)pw, (lv_lds_void *)(buf + wave * 1024), 16, 0, 0);
+        if (p == 1) __builtin_amdgcn_global_load_lds((lv_glb_void *)(pw + 8192), (lv_lds_void *)(buf + 8192 + wave * 1024), 16, 0, 0);
+        if (p == 2) __builtin_amdgcn_global_load_lds((lv_glb_void *)(gh + sc * kGemmXBytes), (lv_lds_void *)(buf + kGemmWBytes + wave * 1024), 16, 0, 0);
+        if (p == 3) __builtin_amdgcn_global_load_lds((lv_glb_void *)(gl + sc * kGemmXBytes), (lv_lds_void *)(buf + kGemmWBytes + kGemmXBytes + wave * 1024), 16, 0, 0);
         // scales: 1 KB, four waves' worth of 4-byte loads; waves 4..7 repeat them (same bytes to the same place)
-        __builtin_amdgcn_global_load_lds((lv_glb_void *)(gs + sc * kGemmScBytes), (lv_lds_void *)(buf + kGemmWBytes + 2 * kGemmXBytes + (wave & 3) * 256), 4, 0, 0);
+        if (p == 4) __builtin_amdgcn_global_load_lds((lv_glb_void *)(gs + sc * kGemmScBytes), (lv_lds_void *)(buf + kGemmWBytes + 2 * kGemmXBytes + (wave & 3) * 256), 4, 0, 0);
     };
 
     lv_f16v acc[2][2];
@@ -388,11 +388,11 @@ __global__ __launch_bounds__(512) void gemm_kernel(GemmArgs a)
         for (int g = 0; g < 16; g++) {
             const int t = g >> 2, m = g & 3, i = t >> 1, j = t & 1;
             if (g == 8) {
-                // stage s + 1 has landed for everyone, and everyone holds stage s in registers: its buffer takes stage s + 4
+                // stage s + 1 has landed for everyone, and everyone holds stage s in registers: from here on its buffer may
+                // take stage s + 4
                 asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NST - 2) * LPS) : "memory");
                 __builtin_amdgcn_s_barrier();
                 asm volatile("" ::: "memory");
-                issue(s + NST);
                 __builtin_amdgcn_sched_barrier(0);
             }
             const lv_h8 &xa = m < 2 ? cur.xl[m & 1][i] : cur.xh[m & 1][i];
@@ -411,6 +411,14 @@ __global__ __launch_bounds__(512) void gemm_kernel(GemmArgs a)
                 for (int r = 4 * (q & 3); r < 4 * (q & 3) + 4; r++) acc[pt >> 1][pt & 1][r] = fmaf(T[pt][r], cur.d[pt & 1], acc[pt >> 1][pt & 1][r]);
             }
             if (g >= 8 && g < 14) read_part(nxt, lds + ((s + 1) % NST) * kGemmStageBytes, g - 8);
+            // the five loads of stage s + 4, one at a time between the MFMAs of this step's second half and the next step's
+            // first: issued together right behind the barrier, the forty of a workgroup back up and hold the waves that
+            // issue them, MFMAs included (1520 instead of 1300 cycles a step)
+            if (g == 9) issue_one(s + NST, 0);
+            if (g == 12) issue_one(s + NST, 1);
+            if (g == 15) issue_one(s + NST, 2);
+            if (g == 2) issue_one(s + NST - 1, 3);
+            if (g == 5) issue_one(s + NST - 1, 4);
             __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
@@ -420,8 +428,10 @@ __global__ __launch_bounds__(512) void gemm_kernel(GemmArgs a)
     };
     Frag FA, FB;
 #pragma unroll
-    for (int s = 0; s < NST; s++) issue(s);
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NST - 1) * LPS) : "memory");
+    for (int s = 0; s < NST; s++)
+#pragma unroll
+        for (int p = 0; p < (s == NST - 1 ? 3 : LPS); p++) issue_one(s, p);      // the last two of stage 3 follow in step 0
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NST - 1) * LPS - 2) : "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 #pragma unroll
