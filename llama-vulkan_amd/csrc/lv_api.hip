@@ -163,6 +163,7 @@ struct lv_session {
     uint32_t pf_cap = 0;
     float *pf_x = nullptr, *pf_xn = nullptr, *pf_q = nullptr, *pf_k = nullptr, *pf_v = nullptr, *pf_vo = nullptr, *pf_g1 = nullptr, *pf_g2 = nullptr;
     uint16_t *pf_xh = nullptr, *pf_xl = nullptr;
+    float *pf_xs = nullptr;   // per token: the power of two the halves written by prefill_norm_kernel are scaled down by
     float *xchg[2] = {nullptr, nullptr};  // hand-over buffer sets of the persistent kernel
     uint32_t xchg_turn = 0;
     uint32_t *status_host = nullptr;      // pinned, written by the persistent kernel: [0] a poll expired, [kStatusToken] greedy pick
@@ -714,13 +715,17 @@ extern "C" int lv_kernel_gemv_silu(lv_ctx *c, float *out, const lv_matrix *w3, c
 
 // out[n][ldo] (+)= x[n][K] * W^T on the matrix cores; xh/xl = workspace for the fp16 halves of x, n_pad rows
 static int launch_gemm_presplit(hipStream_t st, float *out, uint32_t ldo, const lv_matrix &w, uint32_t n, const uint16_t *xh, const uint16_t *xl,
-                                bool accumulate);
+                                bool accumulate, const float *xscale = nullptr);
 
-// fp32 activations -> the two fp16 halves the GEMM multiplies
-static int launch_split(hipStream_t st, uint16_t *xh, uint16_t *xl, const float *x, uint32_t n, uint32_t K)
+// fp32 activations -> the two fp16 halves the GEMM multiplies; with xscale, scaled row by row (inputs of unknown size)
+static int launch_split(hipStream_t st, uint16_t *xh, uint16_t *xl, float *xscale, const float *x, uint32_t n, uint32_t K)
 {
     const uint32_t n_pad = (n + kGemmTile - 1) / kGemmTile * kGemmTile, Kp = gemm_k_padded(K);
-    split_half_kernel<<<dim3(Kp / 64, n_pad / 32), dim3(256), 0, st>>>(xh, xl, x, n, K, Kp);
+    if (K % 8) return fail(LV_ERR_ARG, "gemm: %u columns", K);
+    if (!xscale) split_half_kernel<<<dim3(Kp / 64, n_pad / 32), dim3(256), 0, st>>>(xh, xl, x, n, K, Kp);
+    else if (Kp <= 2048 * 3) split_rows_kernel<3><<<dim3(n_pad), dim3(256), 0, st>>>(xh, xl, xscale, x, n, K, Kp);
+    else if (Kp <= 2048 * 7) split_rows_kernel<7><<<dim3(n_pad), dim3(256), 0, st>>>(xh, xl, xscale, x, n, K, Kp);
+    else split_rows_kernel<0><<<dim3(n_pad), dim3(256), 0, st>>>(xh, xl, xscale, x, n, K, Kp);
     HIP_TRY(hipGetLastError());
     return LV_OK;
 }
@@ -759,9 +764,10 @@ static int dispatch_gemm(hipStream_t st, GemmArgs a, const lv_matrix &w, uint32_
 // the same with the activations already split (one split serves wq, wk, wv or w3, w1); nmat matrices of one shape,
 // type and scale plane as one launch
 static int launch_gemm_multi(hipStream_t st, float *const outs[], uint32_t ldo, const lv_matrix *const ws[], int nmat, uint32_t n,
-                             const uint16_t *xh, const uint16_t *xl, bool accumulate)
+                             const uint16_t *xh, const uint16_t *xl, bool accumulate, const float *xscale = nullptr)
 {
     GemmArgs a{};
+    a.xscale = xscale;
     for (int i = 0; i < nmat; i++) { a.outs[i] = outs[i]; a.w16[i] = ws[i]->h16; }
     a.xh = xh; a.xl = xl; a.n = n; a.ldo = ldo; a.accumulate = accumulate ? 1 : 0;
     return dispatch_gemm(st, a, *ws[0], (uint32_t)nmat);
@@ -808,13 +814,13 @@ static uint32_t gemm_slices_for(const lv_matrix &w, uint32_t n, uint32_t ldo)
 // With `pending` given, the slices are left unsummed and *pending says how many there are (0: out is complete): the
 // caller adds them to out itself (prefill_norm_kernel does, on its way through the row).
 static int launch_gemm_sliced(hipStream_t st, float *out, uint32_t ldo, const lv_matrix &w, uint32_t n, const uint16_t *xh, const uint16_t *xl,
-                              bool accumulate, float *const parts[kGemmMaxMats], uint32_t *pending = nullptr)
+                              const float *xscale, bool accumulate, float *const parts[kGemmMaxMats], uint32_t *pending = nullptr)
 {
     if (pending) *pending = 0;
     const uint32_t rows = w.view.rows, k_steps = (w.view.cols + kGemmK - 1) / kGemmK;
     const uint32_t slices = parts ? gemm_slices_for(w, n, ldo) : 1;
     GemmArgs a{};
-    a.xh = xh; a.xl = xl; a.n = n;
+    a.xh = xh; a.xl = xl; a.n = n; a.xscale = xscale;
     if (slices == 1) {
         a.outs[0] = out; a.w16[0] = w.h16; a.ldo = ldo; a.accumulate = accumulate ? 1 : 0;
         return dispatch_gemm(st, a, w, 1);
@@ -830,11 +836,11 @@ static int launch_gemm_sliced(hipStream_t st, float *out, uint32_t ldo, const lv
 }
 
 static int launch_gemm_presplit(hipStream_t st, float *out, uint32_t ldo, const lv_matrix &w, uint32_t n, const uint16_t *xh, const uint16_t *xl,
-                                bool accumulate)
+                                bool accumulate, const float *xscale)
 {
     float *const outs[1] = {out};
     const lv_matrix *const ws[1] = {&w};
-    return launch_gemm_multi(st, outs, ldo, ws, 1, n, xh, xl, accumulate);
+    return launch_gemm_multi(st, outs, ldo, ws, 1, n, xh, xl, accumulate, xscale);
 }
 
 // can these matrices share a launch?  (one shape, one type, one kind of scale plane)
@@ -857,10 +863,11 @@ extern "C" int lv_kernel_gemm(lv_ctx *c, float *out, const lv_matrix *w, const f
     const size_t part = slices > 1 ? (size_t)batch * w->view.rows : 0;
     const size_t w_halfs = w->h16 ? 0 : (size_t)prompt_copy_halfs(*w);
     uint16_t *ws = nullptr;
-    hipError_t e = hipMalloc(reinterpret_cast<void **>(&ws), (w_halfs + halfs * 2) * 2 + part * slices * 4);
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&ws), (w_halfs + halfs * 2) * 2 + n_pad * 4 + part * slices * 4);
     if (e != hipSuccess) return fail(LV_ERR_OOM, "lv_kernel_gemm: workspace");
     uint16_t *xh = ws + w_halfs, *xl = xh + halfs;
-    float *p0 = reinterpret_cast<float *>(xl + halfs);
+    float *xscale = reinterpret_cast<float *>(xl + halfs);
+    float *p0 = xscale + n_pad;
     float *const parts[kGemmMaxMats] = {p0, p0 + part, p0 + 2 * part, p0 + 3 * part};
     lv_matrix wm = *w;
     int rc = LV_OK;
@@ -868,8 +875,8 @@ extern "C" int lv_kernel_gemm(lv_ctx *c, float *out, const lv_matrix *w, const f
         rc = launch_expand(c->stream, ws, *w);
         wm.h16 = ws;
     }
-    if (rc == LV_OK) rc = launch_split(c->stream, xh, xl, x, batch, w->view.cols);
-    if (rc == LV_OK) rc = launch_gemm_sliced(c->stream, out, w->view.rows, wm, batch, xh, xl, accumulate != 0, slices > 1 ? parts : nullptr);
+    if (rc == LV_OK) rc = launch_split(c->stream, xh, xl, xscale, x, batch, w->view.cols);
+    if (rc == LV_OK) rc = launch_gemm_sliced(c->stream, out, w->view.rows, wm, batch, xh, xl, xscale, accumulate != 0, slices > 1 ? parts : nullptr);
     (void)hipStreamSynchronize(c->stream);
     (void)hipFree(ws);
     return rc;
@@ -1243,7 +1250,7 @@ extern "C" int lv_session_destroy(lv_session *s)
     drop_graph(s);
     void *dev[] = {s->kv, s->trig, s->trig_abs, s->x, s->xn, s->q, s->k, s->v, s->vo, s->ff, s->logits, s->attn_part, s->attn_counters,
                    s->cfg, s->argmax_dev, s->trace_buf, s->trace_attn, s->pf_x, s->pf_xn, s->pf_q, s->pf_k, s->pf_v, s->pf_vo, s->pf_g1, s->pf_g2,
-                   s->pf_xh, s->pf_xl};
+                   s->pf_xh, s->pf_xl, s->pf_xs};
     for (void *p : dev) (void)hipFree(p);
     (void)hipFree(s->xchg[0]);
     (void)hipFree(s->xchg[1]);
@@ -1584,11 +1591,11 @@ static int prefill_reserve(lv_session *s, uint32_t n)
     if (cap > s->pf_cap) {
         HIP_TRY(hipStreamSynchronize(s->stream));
         void **bufs[] = {(void **)&s->pf_x, (void **)&s->pf_xn, (void **)&s->pf_q, (void **)&s->pf_k, (void **)&s->pf_v, (void **)&s->pf_vo,
-                         (void **)&s->pf_g1, (void **)&s->pf_g2, (void **)&s->pf_xh, (void **)&s->pf_xl};
+                         (void **)&s->pf_g1, (void **)&s->pf_g2, (void **)&s->pf_xh, (void **)&s->pf_xl, (void **)&s->pf_xs};
         const size_t halfs = gemm_k_padded((uint32_t)(F > D ? F : D)) * 2;   // an activation half: padded K, 2 bytes each
-        const size_t sizes[] = {D * 4, D * 4, D * 4, D * 4, D * 4, D * 4, F * 4, F * 4, halfs, halfs};
+        const size_t sizes[] = {D * 4, D * 4, D * 4, D * 4, D * 4, D * 4, F * 4, F * 4, halfs, halfs, 4};
         s->pf_cap = 0;
-        for (int i = 0; i < 10; i++) {
+        for (int i = 0; i < 11; i++) {
             (void)hipFree(*bufs[i]);
             *bufs[i] = nullptr;
             hipError_t e = hipMalloc(bufs[i], sizes[i] * cap);
@@ -1600,24 +1607,29 @@ static int prefill_reserve(lv_session *s, uint32_t n)
 }
 
 // x += pending K slices, xn = normalize(x) * w, halves of xn for the next GEMM: one kernel where the
-// row fits its registers, else the three separate ones.  xn (fp32) is written only when want_xn.
+// row fits its registers, else the three separate ones.  xn (fp32) is written only when want_xn.  *xscale: the per-token
+// scale the GEMMs that read these halves have to apply (null when the halves are unscaled).
 static int launch_prefill_norm(hipStream_t st, lv_session *s, const float *w, uint32_t n, uint32_t D, float *const parts[kGemmMaxMats],
-                               uint32_t pending, bool want_xn)
+                               uint32_t pending, bool want_xn, const float **xscale)
 {
+    *xscale = nullptr;
     const uint32_t n_pad = (n + kGemmTile - 1) / kGemmTile * kGemmTile;
     if (D <= 8192 && D % 8 == 0) {
         PrefillNormArgs a{};
         a.x = s->pf_x; a.nparts = pending; a.w = w; a.xn = want_xn ? s->pf_xn : nullptr; a.xh = s->pf_xh; a.xl = s->pf_xl; a.dim = D; a.n = n;
         a.Kp = gemm_k_padded(D);
+        a.xscale = s->pf_xs;
         for (uint32_t i = 0; i < pending; i++) a.parts[i] = parts[i];
         prefill_norm_kernel<<<dim3(n_pad), dim3(256), 0, st>>>(a);
         HIP_TRY(hipGetLastError());
+        *xscale = s->pf_xs;
         return LV_OK;
     }
     if (pending) LV_TRY(launch_gemm_reduce(st, s->pf_x, D, parts, pending, D, n, true));
     normalize_kernel<<<dim3(n), dim3(256), 0, st>>>(s->pf_xn, s->pf_x, w, D);
     HIP_TRY(hipGetLastError());
-    return launch_split(st, s->pf_xh, s->pf_xl, s->pf_xn, n, D);
+    *xscale = s->pf_xs;
+    return launch_split(st, s->pf_xh, s->pf_xl, s->pf_xs, s->pf_xn, n, D);
 }
 
 // Rows idx0 .. idx0+n-1 of the step at once (llava_layer.cpp:39-75 with batch > 1).  Row z sees cache rows
@@ -1647,40 +1659,42 @@ static int record_prefill(lv_session *s, uint32_t idx0, uint32_t n, bool with_he
     for (uint32_t li = 0; li < hp.layers; li++) {
         const LayerWeights &lw = m->layers[li];
         const bool qkv_same = gemm_same(lw.wq, lw.wk) && gemm_same(lw.wq, lw.wv), gate_same = gemm_same(lw.w3, lw.w1);
-        LV_TRY(launch_prefill_norm(st, s, lw.attn_norm, n, D, parts, pending, !qkv_same));
+        const float *xscale = nullptr;
+        LV_TRY(launch_prefill_norm(st, s, lw.attn_norm, n, D, parts, pending, !qkv_same, &xscale));
         pending = 0;
         if (qkv_same) {
             float *const outs[3] = {s->pf_q, s->pf_k, s->pf_v};
             const lv_matrix *const ws[3] = {&lw.wq, &lw.wk, &lw.wv};
-            LV_TRY(launch_gemm_multi(st, outs, D, ws, 3, n, s->pf_xh, s->pf_xl, false));
+            LV_TRY(launch_gemm_multi(st, outs, D, ws, 3, n, s->pf_xh, s->pf_xl, false, xscale));
         } else {
-            LV_TRY(launch_gemm_presplit(st, s->pf_q, D, lw.wq, n, s->pf_xh, s->pf_xl, false));
-            LV_TRY(launch_gemm_presplit(st, s->pf_k, D, lw.wk, n, s->pf_xh, s->pf_xl, false));
-            LV_TRY(launch_gemm_presplit(st, s->pf_v, D, lw.wv, n, s->pf_xh, s->pf_xl, false));
+            LV_TRY(launch_gemm_presplit(st, s->pf_q, D, lw.wq, n, s->pf_xh, s->pf_xl, false, xscale));
+            LV_TRY(launch_gemm_presplit(st, s->pf_k, D, lw.wk, n, s->pf_xh, s->pf_xl, false, xscale));
+            LV_TRY(launch_gemm_presplit(st, s->pf_v, D, lw.wv, n, s->pf_xh, s->pf_xl, false, xscale));
         }
         kv_append2_kernel<<<dim3(kv_grid.x, kv_grid.y, 2), dim3(256), 0, st>>>(kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->pf_k, s->pf_v, pos_ptr, idx0, D, s->backlog);
         HIP_TRY(hipGetLastError());
         LV_TRY(launch_attention_batch(st, s->pf_vo, kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->pf_q, s->trig_abs, pos_ptr, idx0, n, s->backlog,
                                       hp.heads, hp.rot));
-        LV_TRY(launch_split(st, s->pf_xh, s->pf_xl, s->pf_vo, n, D));
-        LV_TRY(launch_gemm_sliced(st, s->pf_x, D, lw.wo, n, s->pf_xh, s->pf_xl, true, parts, &pending));
-        LV_TRY(launch_prefill_norm(st, s, lw.ffn_norm, n, D, parts, pending, !gate_same));
+        LV_TRY(launch_split(st, s->pf_xh, s->pf_xl, nullptr, s->pf_vo, n, D));
+        LV_TRY(launch_gemm_sliced(st, s->pf_x, D, lw.wo, n, s->pf_xh, s->pf_xl, nullptr, true, parts, &pending));
+        LV_TRY(launch_prefill_norm(st, s, lw.ffn_norm, n, D, parts, pending, !gate_same, &xscale));
         pending = 0;
         if (gate_same) {
             float *const outs[2] = {s->pf_g1, s->pf_g2};
             const lv_matrix *const ws[2] = {&lw.w3, &lw.w1};
-            LV_TRY(launch_gemm_multi(st, outs, F, ws, 2, n, s->pf_xh, s->pf_xl, false));
+            LV_TRY(launch_gemm_multi(st, outs, F, ws, 2, n, s->pf_xh, s->pf_xl, false, xscale));
         } else {
-            LV_TRY(launch_gemm_presplit(st, s->pf_g1, F, lw.w3, n, s->pf_xh, s->pf_xl, false));
-            LV_TRY(launch_gemm_presplit(st, s->pf_g2, F, lw.w1, n, s->pf_xh, s->pf_xl, false));
+            LV_TRY(launch_gemm_presplit(st, s->pf_g1, F, lw.w3, n, s->pf_xh, s->pf_xl, false, xscale));
+            LV_TRY(launch_gemm_presplit(st, s->pf_g2, F, lw.w1, n, s->pf_xh, s->pf_xl, false, xscale));
         }
         {   // SwiGLU straight into the fp16 halves the down projection reads
             const uint32_t Fp = gemm_k_padded(F);
             const dim3 grid(Fp / 64, (n + kGemmTile - 1) / kGemmTile * kGemmTile / 32);
+            if (F % 8) return fail(LV_ERR_ARG, "prompt batch: ff size %u", F);
             silu_split_kernel<<<grid, dim3(256), 0, st>>>(s->pf_xh, s->pf_xl, s->pf_g1, s->pf_g2, n, F, Fp);
             HIP_TRY(hipGetLastError());
         }
-        LV_TRY(launch_gemm_sliced(st, s->pf_x, D, lw.w2, n, s->pf_xh, s->pf_xl, true, parts, &pending));
+        LV_TRY(launch_gemm_sliced(st, s->pf_x, D, lw.w2, n, s->pf_xh, s->pf_xl, nullptr, true, parts, &pending));
     }
     if (pending) LV_TRY(launch_gemm_reduce(st, s->pf_x, D, parts, pending, D, n, true));
     if (with_head) {

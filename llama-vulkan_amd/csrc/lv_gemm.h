@@ -75,9 +75,104 @@ __device__ __forceinline__ void gemm_split8(uint4 &h, uint4 &l, const float (&f)
     l = make_uint4(lw[0], lw[1], lw[2], lw[3]);
 }
 
-// Thread -> (token, chunk of 8 k) for the elementwise producers: a wave covers 8 tokens x 8 chunks, so that it reads
-// 256 consecutive bytes of each token's fp32 row and writes, per chunk, the 128 consecutive bytes of its 8 tokens.
-// grid (Kp / 64, n_pad / 32), 256 threads.
+// The producers of activation halves work a token row at a time: one 256-thread workgroup per row of the padded batch.
+// Workgroups are dealt to the 8 XCDs in turn; the row a workgroup takes is chosen so that the 8 tokens whose 16-byte chunks
+// share a 128-byte line are written through one XCD's L2.
+__device__ __forceinline__ uint32_t gemm_producer_row(uint32_t b) { return (b >> 6) * 64 + (b & 7) * 8 + ((b >> 3) & 7); }   // n_pad is a multiple of 128
+
+// The halves are written for 2^S * x, S chosen per row so that the largest element lies in [2^14, 2^15): the low half of an
+// element then stays a normal fp16 number down to 2^-14 of the row's largest (unscaled, the low half of anything below
+// 0.125 is a subnormal and the pair carries an absolute error of 2^-25), and a row cannot overflow fp16 whatever its
+// size.  xscale[row] = 2^-S, which the GEMM multiplies into its result: powers of two, nothing is rounded.
+// Returns 2^S for a row whose largest magnitude is `big`; *down = 2^-S.  1 for an all-zero or non-finite row.
+__device__ __forceinline__ float gemm_row_scale(float big, float *down)
+{
+    const int eb = (int)((__float_as_uint(big) >> 23) & 0xffu);
+    const int S = (eb == 0 || eb == 255) ? 0 : max(-100, min(100, 14 - (eb - 127)));
+    *down = __uint_as_float((uint32_t)(127 - S) << 23);
+    return __uint_as_float((uint32_t)(127 + S) << 23);
+}
+
+// One row of activations -> its two halves and its scale.  value(f, i) yields the 8 elements of chunk i (i < K / 8).
+// PER > 0: the row (at most 256 * 8 * PER elements) is evaluated once and kept in registers; PER = 0: any length, evaluated
+// twice (largest magnitude first, then the halves; the second pass finds its inputs in L2).
+template <int PER, class Value>
+__device__ __forceinline__ void gemm_write_row(uint16_t *__restrict__ xh, uint16_t *__restrict__ xl, float *__restrict__ xscale, uint32_t row, bool live,
+                                               uint32_t K, uint32_t Kp, float *lds, Value value)
+{
+    const uint32_t n8 = K / 8, chunks = Kp / 8;
+    float big = 0.f;
+    float keep[PER > 0 ? PER : 1][8];
+    if constexpr (PER > 0) {
+#pragma unroll
+        for (int j = 0; j < PER; j++) {
+            const uint32_t i = threadIdx.x + j * 256;
+#pragma unroll
+            for (int e = 0; e < 8; e++) keep[j][e] = 0.f;
+            if (live && i < n8) value(keep[j], i);
+#pragma unroll
+            for (int e = 0; e < 8; e++) big = fmaxf(big, fabsf(keep[j][e]));
+        }
+    } else {
+        if (live)
+            for (uint32_t i = threadIdx.x; i < n8; i += 256) {
+                float f[8];
+                value(f, i);
+#pragma unroll
+                for (int e = 0; e < 8; e++) big = fmaxf(big, fabsf(f[e]));
+            }
+    }
+    big = block_max_256(big, lds);
+    float down;
+    const float up = gemm_row_scale(big, &down);
+    if (threadIdx.x == 0) xscale[row] = down;
+    auto put = [&](uint32_t i, const float (&f)[8]) {
+        float g[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) g[e] = f[e] * up;
+        uint4 h, l;
+        gemm_split8(h, l, g);
+        const size_t o = gemm_x_offset(row, i * 8, Kp);
+        *reinterpret_cast<uint4 *>(xh + o) = h;
+        *reinterpret_cast<uint4 *>(xl + o) = l;
+    };
+    if constexpr (PER > 0) {
+#pragma unroll
+        for (int j = 0; j < PER; j++) {
+            const uint32_t i = threadIdx.x + j * 256;
+            if (i < chunks) put(i, keep[j]);
+        }
+    } else {
+        for (uint32_t i = threadIdx.x; i < chunks; i += 256) {
+            float f[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            if (live && i < n8) value(f, i);
+            put(i, f);
+        }
+    }
+}
+
+// x[n][K] fp32 -> xh, xl (tile order, n_pad tokens x Kp; everything outside n x K is written as zero), xscale[n_pad].
+// K a multiple of 8; with PER > 0, Kp <= 2048 * PER.  For inputs of unknown size (lv_kernel_gemm's activations).
+template <int PER>
+__global__ __launch_bounds__(256) void split_rows_kernel(uint16_t *__restrict__ xh, uint16_t *__restrict__ xl, float *__restrict__ xscale,
+                                                          const float *__restrict__ x, uint32_t n, uint32_t K, uint32_t Kp)
+{
+    __shared__ float lds[4];
+    const uint32_t row = gemm_producer_row(blockIdx.x);
+    const bool live = row < n;
+    const float4 *src = reinterpret_cast<const float4 *>(x + (size_t)(live ? row : 0) * K);
+    gemm_write_row<PER>(xh, xl, xscale, row, live, K, Kp, lds, [&](float (&f)[8], uint32_t i) {
+        const float4 a = src[2 * i], b = src[2 * i + 1];
+        f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+    });
+}
+
+// The two elementwise producers inside a prompt batch write unscaled halves (no xscale): attention outputs and SwiGLU
+// products are of the size of their rows' largest elements often enough that the 2^-25 absolute error of an unscaled pair is
+// of the order of fp32 rounding, and a pass over the row for its maximum costs more than it gains (measured: the same
+// logit errors, the prompt 3 % slower, because a row at a time means 16-byte writes 2 KB apart).
+// Thread -> (token, chunk of 8 k): a wave covers 8 tokens x 8 chunks, so that it reads 256 consecutive bytes of each
+// token's fp32 row and writes, per chunk, the 128 consecutive bytes of its 8 tokens.  grid (Kp / 64, n_pad / 32), 256 threads.
 __device__ __forceinline__ void gemm_producer_coords(uint32_t &token, uint32_t &k)
 {
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -93,7 +188,7 @@ __global__ __launch_bounds__(256) void split_half_kernel(uint16_t *__restrict__ 
     gemm_producer_coords(token, k);
     if (k >= Kp) return;
     float f[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    if (token < n && k < K) {       // K is a multiple of 32: a chunk of 8 lies inside or outside
+    if (token < n && k < K) {       // K is a multiple of 8: a chunk lies inside or outside
         const float4 a = *reinterpret_cast<const float4 *>(x + (size_t)token * K + k), b = *reinterpret_cast<const float4 *>(x + (size_t)token * K + k + 4);
         f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
     }
@@ -105,7 +200,7 @@ __global__ __launch_bounds__(256) void split_half_kernel(uint16_t *__restrict__ 
 }
 
 // ff[n][F] = a * b / (exp(-b) + 1) (matmul_silu_ff.comp:96 with a = W3 x, b = W1 x), written as the two fp16 halves
-// the down projection's GEMM reads (same layout and grid as split_half_kernel)
+// the down projection's GEMM reads (the fp32 product is never stored); layout and grid of split_half_kernel
 __global__ __launch_bounds__(256) void silu_split_kernel(uint16_t *__restrict__ xh, uint16_t *__restrict__ xl, const float *__restrict__ a,
                                                           const float *__restrict__ b, uint32_t n, uint32_t K, uint32_t Kp)
 {
@@ -138,6 +233,7 @@ struct GemmArgs {
     uint32_t n;                         // tokens
     uint32_t ldo;                       // floats between output rows
     int accumulate;                     // out += instead of out =
+    const float *xscale;                // null, or [n_pad]: the activation halves of token t stand for x / xscale[t] (a power of two)
     // 0: nz matrices.  Otherwise the launch splits K: w16[] all name one matrix, slice y multiplies the
     // K range y*slice_k .. (y+1)*slice_k-1 (slice_k a multiple of 64) into outs[y], and gemm_reduce_kernel adds the slices
     // up (a matrix with few rows and a long K, like the down projection, fills the CUs that way)
@@ -223,9 +319,8 @@ __global__ __launch_bounds__(256) void expand_codes_kernel(uint16_t *__restrict_
 // The steps between two GEMMs of a prompt batch as one pass over a token row: x += the K slices of the product
 // before (same order as gemm_reduce_kernel: slices first, then x), xn = normalize(x) * w (normalize_kernel's
 // arithmetic), and xn split in the two fp16 halves the next GEMM reads (tile order, padded to Kp with zeros).
-// One 256-thread workgroup per row of the padded batch; rows n.. are written as zeros.  dim <= 8192, a multiple of 8.
-// Workgroups are dealt to the 8 XCDs in turn; the row a workgroup takes is chosen so that the 8 tokens whose chunks
-// share a 128-byte line are written through one XCD's L2.
+// One 256-thread workgroup per row of the padded batch (rows as in gemm_producer_row, halves scaled as in gemm_row_scale);
+// rows n.. are written as zeros.  dim <= 8192, a multiple of 8.
 struct PrefillNormArgs {
     float *x;                              // [n][dim] residual stream, updated when nparts > 0
     const float *parts[kGemmMaxMats];      // [n][dim] each
@@ -233,13 +328,14 @@ struct PrefillNormArgs {
     const float *w;                        // norm weights
     float *xn;                             // [n][dim] or null: the normalised row as fp32 (for a GEMV-type consumer)
     uint16_t *xh, *xl;                     // tile order, n_pad x Kp
+    float *xscale;                         // [n_pad]: 2^-S of the row
     uint32_t dim, n, Kp;
 };
 __global__ __launch_bounds__(256) void prefill_norm_kernel(PrefillNormArgs a)
 {
     __shared__ float lds[4];
     constexpr int PER = 4;                 // chunks of 8 per thread
-    const uint32_t b = blockIdx.x, row = (b >> 6) * 64 + (b & 7) * 8 + ((b >> 3) & 7);     // n_pad is a multiple of 128
+    const uint32_t row = gemm_producer_row(blockIdx.x);
     const uint32_t dim = a.dim, n8 = dim / 8;
     const bool live = row < a.n;
     const size_t ro = (size_t)(live ? row : 0) * dim;
@@ -284,17 +380,31 @@ __global__ __launch_bounds__(256) void prefill_norm_kernel(PrefillNormArgs a)
     }
     const float inv = rsqrtf(block_sum_256(q, lds) / (float)dim);
     const uint32_t chunks = a.Kp / 8;
+    float big = 0.f;
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+        const bool in = live && threadIdx.x + j * 256 < n8;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            v[j][e] = in ? (v[j][e] * wv[j][e]) * inv : 0.f;   // padding rows and columns: zero
+            big = fmaxf(big, fabsf(v[j][e]));
+        }
+    }
+    big = block_max_256(big, lds);
+    float down;
+    const float up = gemm_row_scale(big, &down);
+    if (threadIdx.x == 0) a.xscale[row] = down;
 #pragma unroll
     for (int j = 0; j < PER; j++) {
         const uint32_t i = threadIdx.x + j * 256;
         if (i >= chunks) continue;
+        if (live && i < n8 && a.xn) {
+            reinterpret_cast<float4 *>(a.xn + ro)[i * 2] = make_float4(v[j][0], v[j][1], v[j][2], v[j][3]);
+            reinterpret_cast<float4 *>(a.xn + ro)[i * 2 + 1] = make_float4(v[j][4], v[j][5], v[j][6], v[j][7]);
+        }
         float f[8];
 #pragma unroll
-        for (int e = 0; e < 8; e++) f[e] = (live && i < n8) ? (v[j][e] * wv[j][e]) * inv : 0.f;   // padding rows and columns: zero
-        if (live && i < n8 && a.xn) {
-            reinterpret_cast<float4 *>(a.xn + ro)[i * 2] = make_float4(f[0], f[1], f[2], f[3]);
-            reinterpret_cast<float4 *>(a.xn + ro)[i * 2 + 1] = make_float4(f[4], f[5], f[6], f[7]);
-        }
+        for (int e = 0; e < 8; e++) f[e] = v[j][e] * up;
         uint4 h, l;
         gemm_split8(h, l, f);
         const size_t o = gemm_x_offset(row, i * 8, a.Kp);
@@ -449,6 +559,16 @@ __global__ __launch_bounds__(512) void gemm_kernel(GemmArgs a)
     // D[i][j]: i = token within the 32-tile, j = weight row; lane l holds j = l%32 and, in register r,
     // i = 8*(r/4) + 4*(l/32) + r%4
     float *const out = a.outs[z];
+    // the per-token scales of this lane's 32 tokens, fetched before the first store (the stores may alias them for all the
+    // compiler knows, and a load behind every store costs the launch 6 us)
+    float4 ts[2][4];
+#pragma unroll
+    for (int ti = 0; ti < 2; ti++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            ts[ti][q] = make_float4(1.f, 1.f, 1.f, 1.f);
+            if (a.xscale) ts[ti][q] = *reinterpret_cast<const float4 *>(a.xscale + tt * TN + wm * 64 + ti * 32 + 8 * q + 4 * lhi);   // n_pad entries: in range
+        }
 #pragma unroll
     for (int ti = 0; ti < 2; ti++)
 #pragma unroll
@@ -457,9 +577,12 @@ __global__ __launch_bounds__(512) void gemm_kernel(GemmArgs a)
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const uint32_t n = tt * TN + wm * 64 + ti * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
+                const float4 t4 = ts[ti][r / 4];
+                const float sc = (r % 4) == 0 ? t4.x : (r % 4) == 1 ? t4.y : (r % 4) == 2 ? t4.z : t4.w;
                 if (n < a.n && m < a.rows) {
                     float *dst = out + (size_t)n * a.ldo + m;
-                    *dst = a.accumulate ? *dst + acc[ti][tj][r] : acc[ti][tj][r];
+                    const float v = acc[ti][tj][r] * sc;
+                    *dst = a.accumulate ? *dst + v : v;
                 }
             }
         }

@@ -249,6 +249,16 @@ __device__ __forceinline__ float block_sum_256(float v, float *lds /* >= 4 float
     return (lds[0] + lds[1]) + (lds[2] + lds[3]);
 }
 
+__device__ __forceinline__ float block_max_256(float v, float *lds /* >= 4 floats */)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    __syncthreads();  // protect lds reuse between consecutive calls
+    if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return fmaxf(fmaxf(lds[0], lds[1]), fmaxf(lds[2], lds[3]));
+}
+
 // The row is read once, as 128-bit loads that are all in flight together, and kept in registers for the three passes
 // (up to 8192 floats, a multiple of 4); longer or odd rows walk memory three times.
 __global__ __launch_bounds__(256) void normalize_kernel(float *__restrict__ out, const float *__restrict__ x,

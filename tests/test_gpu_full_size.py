@@ -256,12 +256,12 @@ def test_13b_q8_0_prompt_of_512_as_one_batch(lva, orc, ctx):
     head_got = head.logits()
     # This model is the least forgiving of the configurations: q8_0 codes up to 127 give every layer weights of order 1,
     # attention scores so large that the softmax picks single rows, and logits up to 9.  The persistent kernel, whose
-    # arithmetic is fp32 throughout, leaves one or two of the 32000 logits a hair beyond the tolerance here (0.011 against
-    # 0.0108); the batch path (activations as a pair of halves) a few dozen, none beyond 0.016.  Hence: all within
-    # twice the tolerance, at most 0.5 % beyond the tolerance itself, the greedy token identical.
+    # arithmetic is fp32 throughout, leaves one of the 32000 logits a hair beyond the tolerance here (0.0110 against
+    # 0.0108); the batch path about ten, none beyond 0.0135.  Hence: all within 1.5 x the tolerance, at most 32 (0.1 %)
+    # beyond the tolerance itself, the greedy token identical.
     err, tol = np.abs(head_got - head_want), 1e-2 + 1e-3 * np.abs(head_want)
-    assert np.all(err <= 2 * tol), float(np.max(err))
-    assert int(np.sum(err > tol)) <= 160, int(np.sum(err > tol))
+    assert np.all(err <= 1.5 * tol), float(np.max(err))
+    assert int(np.sum(err > tol)) <= 32, int(np.sum(err > tol))
     assert head.argmax() == orc.greedy(head_want)
     for layer, bound in ((0, 2.0 ** -10), (19, 4e-3), (39, 4e-3)):
         for which in (0, 1):
