@@ -55,6 +55,14 @@ __device__ __forceinline__ void wide_lds_barrier()
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
+// The input vector sits in LDS block by block (32 floats = 128 bytes) and lane l of a wave reads block 64 * slab + l: in
+// plain order the 64 lanes of a 128-bit read would all fall on the same four banks.  Inside each block the eight 16-byte
+// groups are therefore rotated by the block index: offset of the four floats starting at element i (a multiple of 4).
+__device__ __forceinline__ uint32_t wide_xs_offset(uint32_t i)
+{
+    return (i & ~31u) | ((((i >> 2) + (i >> 5)) & 7u) << 2);
+}
+
 // sum over the workgroup through kWideWaves floats of LDS (one barrier; the caller alternates scratch areas)
 __device__ __forceinline__ float wide_block_sum(float v, float *scratch, int w, int lane)
 {
@@ -107,7 +115,7 @@ __device__ __forceinline__ void gemv_wide_body(const GemvArgs &a, uint32_t rows_
         for (uint32_t i = threadIdx.x * 4; i < K; i += NW * 64 * 4) {
             const float4 v = *reinterpret_cast<const float4 *>(xz + i), wv = *reinterpret_cast<const float4 *>(a.norm_w + i);
             s += (v.x + v.y) + (v.z + v.w);
-            *reinterpret_cast<float4 *>(xs + i) = make_float4(v.x * wv.x, v.y * wv.y, v.z * wv.z, v.w * wv.w);
+            *reinterpret_cast<float4 *>(xs + wide_xs_offset(i)) = make_float4(v.x * wv.x, v.y * wv.y, v.z * wv.z, v.w * wv.w);
         }
         const float mean = wide_block_sum(s, stat, w, lane) / (float)K;
         float qd = 0.f;
@@ -118,15 +126,16 @@ __device__ __forceinline__ void gemv_wide_body(const GemvArgs &a, uint32_t rows_
         }
         inv = rsqrtf(wide_block_sum(qd, stat + 16, w, lane) / (float)K);   // its barrier also publishes xs
     } else {
-        for (uint32_t i = threadIdx.x * 4; i < K; i += NW * 64 * 4) *reinterpret_cast<float4 *>(xs + i) = *reinterpret_cast<const float4 *>(xz + i);
+        for (uint32_t i = threadIdx.x * 4; i < K; i += NW * 64 * 4) *reinterpret_cast<float4 *>(xs + wide_xs_offset(i)) = *reinterpret_cast<const float4 *>(xz + i);
         wide_lds_barrier();
     }
     float xr[32], xsum = 0.f;
     {
-        const float4 *src = reinterpret_cast<const float4 *>(xs + (size_t)(lane_ok ? blk_col : 0) * 32);
+        const uint32_t blk = lane_ok ? blk_col : 0;
+        const float4 *src = reinterpret_cast<const float4 *>(xs + (size_t)blk * 32);
 #pragma unroll
         for (int j = 0; j < 8; j++) {
-            float4 v = src[j];
+            float4 v = src[(j + blk) & 7];
             if (!lane_ok) v = make_float4(0.f, 0.f, 0.f, 0.f);
             xr[4 * j] = v.x; xr[4 * j + 1] = v.y; xr[4 * j + 2] = v.z; xr[4 * j + 3] = v.w;
             xsum += (v.x + v.y) + (v.z + v.w);
