@@ -14,13 +14,13 @@ def _abs_dot_bound(orc, blocks, ftype, rows, cols, x):
 
 @pytest.mark.parametrize("ftype_name", ["q4_0", "q8_0"])
 @pytest.mark.parametrize("rows,cols,batch,accumulate", [
-    (128, 64, 128, False),       # exactly one tile, one K step
+    (128, 64, 128, False),       # half a row tile, one token tile, two K steps (the shortest K the pipeline sees)
     (256, 4096, 130, False),     # a second, almost empty token tile
     (704, 256, 17, True),        # rows not a multiple of the tile, residual add
-    (96, 1376, 200, False),      # K = 43 blocks: a half K step at the end, fewer rows than a tile
-    (4096, 4096, 512, True),     # the 7B attention shape at a 512-token prompt batch (K cut in two slices)
-    (5120, 3168, 512, True),     # 160 tiles for 256 CUs: K cut in three slices of 17, 17 and 15.5 steps, then reduced
-    (8264, 160, 400, True),      # more 128-row tiles than CUs: the 256-row form (q8_0), ragged in rows, K and tokens
+    (96, 1376, 200, False),      # K = 43 blocks, padded to 44 with zeros; fewer rows than a tile
+    (4096, 4096, 512, True),     # the 7B attention shape at a 512-token prompt batch (K cut in four slices, then reduced)
+    (5120, 3168, 512, True),     # 80 tiles for 256 CUs: K cut in three slices of 17, 17 and 15.5 steps of 64, then reduced
+    (8264, 160, 400, True),      # 33 row tiles (five of the eight XCDs get one more), ragged in rows, K and tokens
 ])
 def test_gemm_matches_oracle(lva, orc, ctx, ftype_name, rows, cols, batch, accumulate):
     ftype = lva.LV_Q4_0 if ftype_name == "q4_0" else lva.LV_Q8_0
@@ -44,6 +44,30 @@ def test_gemm_matches_oracle(lva, orc, ctx, ftype_name, rows, cols, batch, accum
     one = ctx.to_host(dout2, (batch, rows), np.float32)[:nb]
     assert float(np.max(np.abs(one.astype(np.float64) - got[:nb]) / bound[:nb])) <= 1.5
     for p in (dx, dout, dout2):
+        ctx.free(p)
+    ctx.matrix_free(m)
+
+
+@pytest.mark.parametrize("scale", [1e-6, 1e-3, 3e4])
+def test_gemm_holds_its_bound_at_any_activation_scale(lva, orc, ctx, scale):
+    """the activation halves are written scaled by a power of two per token row, so the low half of an element stays a normal
+    fp16 number whether the row is of order 1e-6 or 3e4 (unscaled, everything below 0.125 would lose its low bits and
+    anything above 65504 would overflow); rows of very different sizes in one batch"""
+    rows, cols, batch = 512, 1024, 96
+    blocks = lva.synth_quant(lva.LV_Q8_0, rows, cols, seed=71)
+    x = lva.synth_normal(batch, cols, seed=72) * np.float32(scale)
+    x[1] *= np.float32(1e3)                               # one row a thousand times larger than its neighbours
+    x[2] = 0.0                                            # an all-zero row
+    m = ctx.matrix(blocks, lva.LV_Q8_0, rows, cols)
+    dx, dout = ctx.to_device(x), ctx.alloc(batch * rows * 4)
+    lva.check(ctx.lib.lv_kernel_gemm(ctx.h, dout, m, dx, batch, 0))
+    got = ctx.to_host(dout, (batch, rows), np.float32)
+    want = orc.gemv(blocks, lva.LV_Q8_0, rows, cols, x)
+    bound = 1e-5 * _abs_dot_bound(orc, blocks, lva.LV_Q8_0, rows, cols, x)
+    assert np.all(got[2] == 0.0)
+    live = bound > 0
+    assert float(np.max(np.abs(got.astype(np.float64) - want)[live] / bound[live])) <= 1.0
+    for p in (dx, dout):
         ctx.free(p)
     ctx.matrix_free(m)
 
