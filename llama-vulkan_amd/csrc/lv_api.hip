@@ -1915,6 +1915,15 @@ extern "C" int lv_trace_read(lv_session *s, uint32_t layer, int which, float *ds
 }
 
 #ifdef LV_MEGA_TIMING
+// timing builds only: {shader cycles, 100 MHz wall ticks, K steps} of workgroup 0 of the last gemm_kernel launch
+extern "C" int lv_debug_gemm_clock(unsigned long long *dst)
+{
+    if (!dst) return LV_ERR_ARG;
+    HIP_TRY(hipDeviceSynchronize());
+    HIP_TRY(hipMemcpyFromSymbol(dst, HIP_SYMBOL(gemm_clock_words), sizeof(gemm_clock_words)));
+    return LV_OK;
+}
+
 // debugging aid of timing builds only: the persistent kernel's phase timestamps
 extern "C" int lv_debug_status_words(lv_session *s, uint32_t *dst, uint32_t n)
 {

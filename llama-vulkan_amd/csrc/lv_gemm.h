@@ -413,6 +413,12 @@ __global__ __launch_bounds__(256) void prefill_norm_kernel(PrefillNormArgs a)
     }
 }
 
+#ifdef LV_MEGA_TIMING
+// timing builds only: workgroup 0 of the last gemm_kernel launch leaves the shader cycles and the 100 MHz wall ticks of its
+// K loop and the number of steps here (lv_debug_gemm_clock reads them): the shader clock under this load, cycles per step
+__device__ unsigned long long gemm_clock_words[3];
+#endif
+
 // One workgroup: 128 tokens x 256 weight rows over a range of K.  The grid enumerates (matrix or K slice, row tile, token
 // tile) so that the token tiles of one row tile run on one XCD (workgroups are dealt to the 8 XCDs in turn) and find its
 // weights in that XCD's L2, and so that the XCDs get equal numbers of workgroups.
@@ -536,6 +542,9 @@ __global__ __launch_bounds__(512) void gemm_kernel(GemmArgs a)
         c3 = T[3];
         dc[0] = cur.d[0]; dc[1] = cur.d[1];
     };
+#ifdef LV_MEGA_TIMING
+    const unsigned long long clk0 = clock64(), wall0 = wall_clock64();
+#endif
     Frag FA, FB;
 #pragma unroll
     for (int s = 0; s < NST; s++)
@@ -555,6 +564,13 @@ __global__ __launch_bounds__(512) void gemm_kernel(GemmArgs a)
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[1][1][r] = fmaf(c3[r], dc[1], acc[1][1][r]);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // the repeats past the end have landed before the workgroup gives up its LDS
+#ifdef LV_MEGA_TIMING
+    if (blockIdx.x == 0 && tid == 0) {
+        gemm_clock_words[0] = clock64() - clk0;
+        gemm_clock_words[1] = wall_clock64() - wall0;
+        gemm_clock_words[2] = steps;
+    }
+#endif
 
     // D[i][j]: i = token within the 32-tile, j = weight row; lane l holds j = l%32 and, in register r,
     // i = 8*(r/4) + 4*(l/32) + r%4

@@ -14,6 +14,7 @@
     python llama-vulkan_amd/measure.py gemm          isolated 512-token GEMMs at the 13B shapes, q8_0 (for kernel traces and counters)
     python llama-vulkan_amd/measure.py handover      phases of the persistent kernel inside a layer (7B q4_0, position 511; timing build)
     python llama-vulkan_amd/measure.py handover-q8   the same for 7B q8_0 at position 2047
+    python llama-vulkan_amd/measure.py gemm-clock    shader clock and cycles per K step of gemm_kernel during the 13B q8_0 prompt (timing build)
     python llama-vulkan_amd/measure.py copy          1 GiB device-to-device copy: achievable bandwidth, counter calibration
     python llama-vulkan_amd/measure.py all
 
@@ -247,6 +248,34 @@ def handover_case(name, wtype, seed, backlog, last):
     ctx.close()
 
 
+def gemm_clock_case():
+    """Loads the timing build and evaluates the 13B q8_0 512-token prompt eight times; after each pass reads what workgroup 0
+    of the last gemm_kernel launch (the last layer's down projection: a K slice of 4608 = 144 steps) measured around its K
+    loop: shader cycles (clock64) against the 100 MHz wall clock = the shader clock the launch ran at, and cycles per step
+    (the MFMAs of a SIMD's two waves take 1024)."""
+    import ctypes as C
+    lva._libs["libllava_hip.so"] = C.CDLL(os.path.join(HERE, "libllava_hip_timing.so"), mode=C.RTLD_GLOBAL)
+    ctx = lva.Context(0)
+    shape = SHAPES["13b"]
+    model = lva.Model(ctx, model_file("13b", lva.LV_Q8_0, 3))
+    s = lva.Session(model, 512)
+    prompt = lva.synth_tokens(512, 3, shape["vocab"], seed=3)
+    s.begin(prompt, 0)
+    s.wait()
+    words = (C.c_ulonglong * 3)()
+    for rep in range(8):
+        s.timer_start()
+        s.begin(prompt, 0)
+        ms = s.timer_stop()
+        lva.check(ctx.lib.lv_debug_gemm_clock(words))
+        cycles, ticks, steps = words[0], words[1], words[2]
+        emit(case="gemm-clock", pass_ms=round(ms, 2), steps=int(steps), shader_cycles=int(cycles), wall_us=round(ticks / 100.0, 1),
+             shader_MHz=round(cycles / (ticks / 100.0)), cycles_per_step=round(cycles / max(steps, 1)))
+    s.close()
+    model.close()
+    ctx.close()
+
+
 def gemm_cases(ctx):
     """lv_kernel_gemm allocates its workspace and splits the activations in every call, so the time of a call is not the
     kernel's: this case exists to put gemm_kernel launches of known shape under rocprofv3 (kernel trace, counters)"""
@@ -268,6 +297,8 @@ def gemm_cases(ctx):
 
 def main():
     which = sys.argv[1] if len(sys.argv) > 1 else "all"
+    if which == "gemm-clock":
+        return gemm_clock_case()
     if which == "handover":
         return handover_case("handover", lva.LV_Q4_0, 0, 512, 511)
     if which == "handover-q8":
