@@ -14,6 +14,7 @@ def _abs_dot_bound(orc, blocks, ftype, rows, cols, x):
 
 @pytest.mark.parametrize("ftype_name", ["q4_0", "q8_0"])
 @pytest.mark.parametrize("rows,cols,batch,accumulate", [
+    (64, 32, 5, False),          # one quant block per row: K padded to 64 with zeros, a handful of tokens
     (128, 64, 128, False),       # half a row tile, one token tile, two K steps (the shortest K the pipeline sees)
     (256, 4096, 130, False),     # a second, almost empty token tile
     (704, 256, 17, True),        # rows not a multiple of the tile, residual add
