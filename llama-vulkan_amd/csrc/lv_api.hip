@@ -749,10 +749,8 @@ static int dispatch_gemm(hipStream_t st, GemmArgs a, const lv_matrix &w, uint32_
     a.rows = w.view.rows; a.K = w.view.cols;
     for (uint32_t i = 0; i < nz; i++)
         if (!a.w16[i]) return fail(LV_ERR_STATE, "gemm: the matrix has no prompt copy");
-    static std::once_flag lds_once;
-    static hipError_t lds_rc = hipSuccess;
-    std::call_once(lds_once, [] { lds_rc = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLdsBytes); });
-    HIP_TRY(lds_rc);
+    // 132 KB of dynamic LDS need the attribute on the device the launch goes to; setting it is a host-side table entry
+    HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLdsBytes));
     const uint32_t token_tiles = (a.n + kGemmTile - 1) / kGemmTile, row_tiles = (a.rows + kGemmRows - 1) / kGemmRows;
     a.nz = nz;
     const dim3 grid((row_tiles * nz + 7) / 8 * 8 * token_tiles);
