@@ -68,6 +68,11 @@ struct lv_ctx {
     float *attn_part = nullptr;
     uint32_t *attn_counters = nullptr;
     size_t attn_part_floats = 0, attn_counter_words = 0;
+    // and for its batched form (batch >= kPrefillMin): absolute-position table and operand planes
+    float2 *trig_abs = nullptr;
+    uint32_t trig_abs_rows = 0, trig_abs_rot = 0;
+    uint16_t *attn_planes = nullptr;
+    size_t attn_plane_halfs = 0;
     hipEvent_t ev_start = nullptr, ev_stop = nullptr;
     struct AttnScratch *scratch = nullptr;   // this device's copy of the file-scope scratch array (lv_kernel_attention_static)
     // Persistent decode kernels of different sessions (one per thread, llava_context.h:47-49 has the same pools and
@@ -164,6 +169,9 @@ struct lv_session {
     float *pf_x = nullptr, *pf_xn = nullptr, *pf_q = nullptr, *pf_k = nullptr, *pf_v = nullptr, *pf_vo = nullptr, *pf_g1 = nullptr, *pf_g2 = nullptr;
     uint16_t *pf_xh = nullptr, *pf_xl = nullptr;
     float *pf_xs = nullptr;   // per token: the power of two the halves written by prefill_norm_kernel are scaled down by
+    // operand planes of the batched attention (one layer's worth, rewritten per layer): four of attn_plane_halfs() each
+    uint16_t *pf_planes = nullptr;
+    size_t pf_plane_halfs = 0;
     float *xchg[2] = {nullptr, nullptr};  // hand-over buffer sets of the persistent kernel
     uint32_t xchg_turn = 0;
     uint32_t *status_host = nullptr;      // pinned, written by the persistent kernel: [0] a poll expired, [kStatusToken] greedy pick
@@ -237,6 +245,8 @@ extern "C" int lv_ctx_destroy(lv_ctx *c)
     (void)hipFree(c->trig);
     (void)hipFree(c->attn_part);
     (void)hipFree(c->attn_counters);
+    (void)hipFree(c->trig_abs);
+    (void)hipFree(c->attn_planes);
     if (c->ev_start) (void)hipEventDestroy(c->ev_start);
     if (c->ev_stop) (void)hipEventDestroy(c->ev_stop);
     if (c->mega_done) (void)hipEventDestroy(c->mega_done);
@@ -595,6 +605,8 @@ static int launch_gemv3(hipStream_t st, float *const out[3], const lv_matrix *co
     return LV_OK;
 }
 
+constexpr uint32_t kPrefillMin = 16;       // below this the rows of a step go through the one-token kernels
+
 static size_t attn_part_floats(uint32_t batch, uint32_t heads, uint32_t splits, uint32_t rot)
 {
     return (size_t)batch * heads * splits * (rot + 1);
@@ -620,19 +632,40 @@ static int launch_attention(hipStream_t st, float *out, const uint16_t *kc, cons
     return LV_OK;
 }
 
-static int launch_attention_batch(hipStream_t st, float *out, const uint16_t *kc, const uint16_t *vc, const float *q, const float2 *trig_abs,
-                                  const uint32_t *pos_ptr, uint32_t pos_add, uint32_t n, uint32_t backlog, uint32_t heads, uint32_t rot)
+// Batched (prompt) attention of one layer: the operand planes of positions 0 .. pos + n - 1, then the attention kernel.
+// `planes`: four planes of attn_plane_halfs(backlog, heads, rot) halfs.  kin / vin: the batch's K and V rows, not yet in the cache
+// (the first kernel appends them), or null when the cache already holds them.  The result goes to `out` (fp32 rows) and/or to the
+// activation halves xh / xl (tile order, width Kp; the rows up to the next multiple of 128 are written as zeros).
+static int launch_attention_batch(hipStream_t st, float *out, uint16_t *xh, uint16_t *xl, uint32_t Kp, uint16_t *planes, uint16_t *kc,
+                                  uint16_t *vc, const float *kin, const float *vin, const float *q, const float2 *trig_abs, const uint32_t *pos_ptr, uint32_t pos_add, uint32_t n,
+                                  uint32_t backlog, uint32_t heads, uint32_t rot)
 {
+    const size_t ph = attn_plane_halfs(backlog, heads, rot);
+    AttnPrepArgs p{};
+    p.pl.kh = planes; p.pl.kl = planes + ph; p.pl.v1 = planes + 2 * ph; p.pl.v2 = planes + 3 * ph;
+    p.kcache = kc; p.vcache = vc; p.kin = kin; p.vin = vin; p.trig_abs = trig_abs; p.pos_ptr = pos_ptr; p.pos_add = pos_add; p.n = n; p.heads = heads; p.backlog = backlog;
     AttnBatchArgs a{};
-    a.out = out; a.kcache = kc; a.vcache = vc; a.q = q; a.trig_abs = trig_abs; a.pos_ptr = pos_ptr; a.pos_add = pos_add;
+    a.out = out; a.xh = xh; a.xl = xl; a.Kp = Kp; a.pl = p.pl; a.q = q; a.trig_abs = trig_abs; a.pos_ptr = pos_ptr; a.pos_add = pos_add;
     a.n = n; a.heads = heads; a.backlog = backlog;
-    const dim3 grid(heads, (n + kAttnBatchQ - 1) / kAttnBatchQ);
+    const dim3 pgrid(heads, attn_rows64(backlog) / kAttnBatchK);
+    const uint32_t n_pad = xh ? (n + kGemmTile - 1) / kGemmTile * kGemmTile : n;
+    const dim3 grid(heads, (n_pad + kAttnBatchQ - 1) / kAttnBatchQ);
+    const size_t lds = (size_t)1024 * rot;
+    // more than 64 KB of dynamic LDS has to be allowed per function, on the device that launches it
+#define LV_ATTN_BATCH(R)                                                                                                              \
+    case R:                                                                                                                           \
+        attention_prepare_kernel<R><<<pgrid, dim3(256), 0, st>>>(p);                                                                  \
+        HIP_TRY(hipGetLastError());                                                                                                   \
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(attention_batch_kernel<R>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
+        attention_batch_kernel<R><<<grid, dim3(256), lds, st>>>(a);                                                                   \
+        break;
     switch (rot) {
-    case 32: attention_batch_kernel<32><<<grid, dim3(256), 0, st>>>(a); break;
-    case 64: attention_batch_kernel<64><<<grid, dim3(256), 0, st>>>(a); break;
-    case 128: attention_batch_kernel<128><<<grid, dim3(256), 0, st>>>(a); break;
+        LV_ATTN_BATCH(32)
+        LV_ATTN_BATCH(64)
+        LV_ATTN_BATCH(128)
     default: return fail(LV_ERR_ARG, "attention: head size %u (32, 64 and 128 are built)", rot);
     }
+#undef LV_ATTN_BATCH
     HIP_TRY(hipGetLastError());
     return LV_OK;
 }
@@ -910,6 +943,28 @@ extern "C" int lv_kernel_attention(lv_ctx *c, float *out, const void *kcache, co
     if ((uint64_t)pos + batch > backlog) return fail(LV_ERR_RANGE, "lv_kernel_attention: rows %u+%u of %u", pos, batch, backlog);
     if (rot != 32 && rot != 64 && rot != 128) return fail(LV_ERR_ARG, "lv_kernel_attention: head size %u", rot);
     HIP_TRY(hipSetDevice(c->device));
+    if (batch >= kPrefillMin) {    // the kernels a prompt batch goes through
+        if (c->trig_abs_rot != rot || c->trig_abs_rows < backlog) {
+            HIP_TRY(hipStreamSynchronize(c->stream));
+            (void)hipFree(c->trig_abs);
+            c->trig_abs = nullptr;
+            c->trig_abs_rows = c->trig_abs_rot = 0;
+            LV_TRY(upload_trig(&c->trig_abs, backlog, rot, c->stream, true));
+            c->trig_abs_rows = backlog;
+            c->trig_abs_rot = rot;
+        }
+        const size_t planes = 4 * attn_plane_halfs(backlog, heads, rot);
+        if (c->attn_plane_halfs < planes) {
+            HIP_TRY(hipStreamSynchronize(c->stream));
+            (void)hipFree(c->attn_planes);
+            c->attn_planes = nullptr;
+            c->attn_plane_halfs = 0;
+            HIP_TRY(hipMalloc(reinterpret_cast<void **>(&c->attn_planes), planes * 2));
+            c->attn_plane_halfs = planes;
+        }
+        return launch_attention_batch(c->stream, out, nullptr, nullptr, 0, c->attn_planes, static_cast<uint16_t *>(const_cast<void *>(kcache)),
+                                      static_cast<uint16_t *>(const_cast<void *>(vcache)), nullptr, nullptr, q, c->trig_abs, nullptr, pos, batch, backlog, heads, rot);
+    }
     if (c->trig_rot != rot || c->trig_rows < backlog) {
         HIP_TRY(hipStreamSynchronize(c->stream));
         (void)hipFree(c->trig);
@@ -1248,7 +1303,7 @@ extern "C" int lv_session_destroy(lv_session *s)
     drop_graph(s);
     void *dev[] = {s->kv, s->trig, s->trig_abs, s->x, s->xn, s->q, s->k, s->v, s->vo, s->ff, s->logits, s->attn_part, s->attn_counters,
                    s->cfg, s->argmax_dev, s->trace_buf, s->trace_attn, s->pf_x, s->pf_xn, s->pf_q, s->pf_k, s->pf_v, s->pf_vo, s->pf_g1, s->pf_g2,
-                   s->pf_xh, s->pf_xl, s->pf_xs};
+                   s->pf_xh, s->pf_xl, s->pf_xs, s->pf_planes};
     for (void *p : dev) (void)hipFree(p);
     (void)hipFree(s->xchg[0]);
     (void)hipFree(s->xchg[1]);
@@ -1579,7 +1634,6 @@ static bool ensure_prompt_copy(lv_model *m)
 }
 
 constexpr uint32_t kPrefillChunk = 512;    // tokens evaluated together (bounds the workspace)
-constexpr uint32_t kPrefillMin = 16;       // below this the rows go through the one-token kernels
 
 static int prefill_reserve(lv_session *s, uint32_t n)
 {
@@ -1600,6 +1654,16 @@ static int prefill_reserve(lv_session *s, uint32_t n)
             if (e != hipSuccess) return fail(e == hipErrorOutOfMemory ? LV_ERR_OOM : LV_ERR_HIP, "prompt workspace: %s", hipGetErrorString(e));
         }
         s->pf_cap = cap;
+    }
+    const size_t planes = 4 * attn_plane_halfs(s->backlog, hp.heads, hp.rot);
+    if (planes > s->pf_plane_halfs) {
+        HIP_TRY(hipStreamSynchronize(s->stream));
+        (void)hipFree(s->pf_planes);
+        s->pf_planes = nullptr;
+        s->pf_plane_halfs = 0;
+        hipError_t e = hipMalloc(reinterpret_cast<void **>(&s->pf_planes), planes * 2);
+        if (e != hipSuccess) return fail(e == hipErrorOutOfMemory ? LV_ERR_OOM : LV_ERR_HIP, "prompt workspace: %s", hipGetErrorString(e));
+        s->pf_plane_halfs = planes;
     }
     return LV_OK;
 }
@@ -1649,7 +1713,6 @@ static int record_prefill(lv_session *s, uint32_t idx0, uint32_t n, bool with_he
         embed_quant_kernel<8><<<dim3((D / 32 + 63) / 64, n), dim3(64), 0, st>>>(s->pf_x, m->tok_quant.view, tok_ptr);
     HIP_TRY(hipGetLastError());
 
-    const dim3 kv_grid((D + 255) / 256, n);
     // q, k and v buffers of a layer are free once attention has run: they take the K slices of the output projection
     // and of the down projection; `pending` of them wait to be added to the residual stream by the next norm
     float *const parts[kGemmMaxMats] = {s->pf_q, s->pf_k, s->pf_v, s->pf_vo};
@@ -1669,11 +1732,15 @@ static int record_prefill(lv_session *s, uint32_t idx0, uint32_t n, bool with_he
             LV_TRY(launch_gemm_presplit(st, s->pf_k, D, lw.wk, n, s->pf_xh, s->pf_xl, false, xscale));
             LV_TRY(launch_gemm_presplit(st, s->pf_v, D, lw.wv, n, s->pf_xh, s->pf_xl, false, xscale));
         }
-        kv_append2_kernel<<<dim3(kv_grid.x, kv_grid.y, 2), dim3(256), 0, st>>>(kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->pf_k, s->pf_v, pos_ptr, idx0, D, s->backlog);
-        HIP_TRY(hipGetLastError());
-        LV_TRY(launch_attention_batch(st, s->pf_vo, kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->pf_q, s->trig_abs, pos_ptr, idx0, n, s->backlog,
-                                      hp.heads, hp.rot));
-        LV_TRY(launch_split(st, s->pf_xh, s->pf_xl, nullptr, s->pf_vo, n, D));
+        // the batch's K and V rows go to the cache in the first of the attention kernels
+        if (D % kGemmK == 0) {     // the attention kernel writes the halves the output projection reads
+            LV_TRY(launch_attention_batch(st, nullptr, s->pf_xh, s->pf_xl, D, s->pf_planes, kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->pf_k, s->pf_v, s->pf_q, s->trig_abs,
+                                          pos_ptr, idx0, n, s->backlog, hp.heads, hp.rot));
+        } else {                   // a padded K: the split kernel writes the zero columns as well
+            LV_TRY(launch_attention_batch(st, s->pf_vo, nullptr, nullptr, 0, s->pf_planes, kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->pf_k, s->pf_v, s->pf_q, s->trig_abs,
+                                          pos_ptr, idx0, n, s->backlog, hp.heads, hp.rot));
+            LV_TRY(launch_split(st, s->pf_xh, s->pf_xl, nullptr, s->pf_vo, n, D));
+        }
         LV_TRY(launch_gemm_sliced(st, s->pf_x, D, lw.wo, n, s->pf_xh, s->pf_xl, nullptr, true, parts, &pending));
         LV_TRY(launch_prefill_norm(st, s, lw.ffn_norm, n, D, parts, pending, !gate_same, &xscale));
         pending = 0;

@@ -5,217 +5,332 @@
 // Arithmetic.  mhsa.comp:45-58 rotates every (query, position) pair by the relative angle delta * theta_i:
 //     s = sum_i cos(delta theta_i) (qx kx + qy ky) + sin(delta theta_i) (qx ky - qy kx),   delta = pos_q - pos_k.
 // That is Re[conj(q') k'] with q' = e^{i pos_q theta} q and k' = e^{i pos_k theta} k: rotating each query row and each
-// cache row ONCE by its own position turns the score into a plain dot product, which the matrix cores take (fp32 MFMA:
-// products and sums in fp32).  The rotation angles come from a table of cos/sin(p * theta_i) with theta_i rounded to
-// fp32 as the shader's pow() result is and the product taken exactly; the shader rounds delta * theta_i to fp32 before
-// its cos/sin, so the two differ by that one rounding of the angle (below 1.3e-4 rad at a distance of 2047, far inside
-// the tolerance that GLSL's own cos/sin precision needs).  The one-query kernels keep the per-pair form.
-// Then e = exp(s / sqrt(R)) without max subtraction (softmax.comp:33), out = sum e V / sum e (kqv_matching.comp:35-41),
-// K and V read back from the fp16 cache.  Without a running maximum there is nothing to rescale: both sums simply
-// accumulate over the tiles.
+// cache row ONCE by its own position turns the score into a plain dot product.  The rotation angles come from a table of
+// cos/sin(p * theta_i) with theta_i rounded to fp32 as the shader's pow() result is and the product taken exactly; the
+// shader rounds delta * theta_i to fp32 before its cos/sin, so the two differ by that one rounding of the angle (below
+// 1.3e-4 rad at a distance of 2047, far inside the tolerance that GLSL's own cos/sin precision needs).  The one-query
+// kernels keep the per-pair form.  Then e = exp(s / sqrt(R)) without max subtraction (softmax.comp:33),
+// out = sum e V / sum e (kqv_matching.comp:35-41), K and V read back from the fp16 cache.  Without a running maximum there
+// is nothing to rescale: both sums simply accumulate over the tiles.
 //
-// One workgroup = one head x 64 query rows, four waves = 2 query tiles x 2 position tiles of 32; the cache is walked
-// in tiles of 64 positions staged through LDS (K rotated, as fp32, x and y components apart; V transposed, fp16, even
-// and odd positions apart: both so that an MFMA operand is a run of consecutive LDS words per lane; the 8-byte units
-// of a V row are permuted so that the stores of the staging spread over the banks).
+// Matrix cores at fp32 accuracy.  Both products run on the 16-bit MFMAs (sixteen times the rate of the fp32 ones) with
+// their fp32 operands cut into 16-bit pieces whose products the MFMA forms exactly and adds in fp32:
+//   scores  q' = qh + ql and k' = kh + kl as fp16 pairs (22 bits); qh kh + ql kh + qh kl, the dropped ql kl is 2^-22 of a term;
+//   sums    e = e1 + e2 + e3 as bf16 (an exact cut of the 24 bits; bf16 has fp32's range, and e is not bounded by anything
+//           smaller) and the fp16 cache value v = v1 + v2 as bf16 (exact: 11 bits in 8 + 3);
+//           e1 v1 + e1 v2 + e2 v1 + e2 v2 + e3 v1, the dropped e3 v2 is 2^-24 of a term.
+// attention_prepare_kernel writes the four position-only operand planes of a layer once (kh, kl: rotated K, row-major;
+// v1, v2: V transposed, positions along a row, the 16 positions of a group in the order the MFMA's k index wants them),
+// so that the attention kernel's inner loop has no conversion in it.
+//
+// One workgroup = one head x 64 query rows, four waves = 2 query tiles x 2 position tiles of 32; the cache is walked in
+// tiles of 64 positions.  A tile's four planes (64 KB at R = 128) go to LDS by direct loads one step ahead of their use
+// (two buffers, one barrier per step).  The score MFMA is taken transposed (positions x queries), which leaves a lane
+// holding 16 positions of ONE query: exactly the A operand of the second product, with no trip through LDS.
+// The 16-byte chunks of a plane's rows are permuted in LDS (chunk ^ row bits) so that the 32 lanes of an operand read,
+// which walk down the rows at one chunk, spread over the banks.
 #pragma once
 
-#include "lv_kernels.h"
+#include "lv_gemm.h"
 
 namespace lv {
 
 constexpr int kAttnBatchQ = 64;   // query rows per workgroup
 constexpr int kAttnBatchK = 64;   // cache positions per tile
 
+typedef __bf16 lv_b8 __attribute__((ext_vector_type(8)));
+
+// the prepared operand planes of one layer
+struct AttnPlanes {
+    uint16_t *kh, *kl;      // [rows64][H*R] fp16: rotated K, high and low halves (rows64 = backlog rounded up to 64)
+    uint16_t *v1, *v2;      // [H*R][rows64] bf16: V transposed, high and low parts; position order within 16: see attn_slot_pos
+};
+
+// position (within its group of 16) held by slot i of a transposed V row: slots 0-3 = positions 0-3, 4-7 = 8-11,
+// 8-11 = 4-7, 12-15 = 12-15 (bits 2 and 3 swapped).  A lane of the score MFMA's result holds, in registers 8t .. 8t+7,
+// positions 16t + {0-3, 8-11} (lanes 0-31) or 16t + {4-7, 12-15} (lanes 32-63): with this order each is one 16-byte chunk.
+__host__ __device__ constexpr int attn_slot_pos(int i) { return (i & 3) | ((i & 4) << 1) | ((i & 8) >> 1); }
+
+__host__ __device__ constexpr uint32_t attn_rows64(uint32_t backlog) { return (backlog + 63) / 64 * 64; }
+// halfs of one plane
+__host__ __device__ constexpr size_t attn_plane_halfs(uint32_t backlog, uint32_t heads, uint32_t rot) { return (size_t)attn_rows64(backlog) * heads * rot; }
+
+struct AttnPrepArgs {
+    AttnPlanes pl;
+    uint16_t *kcache, *vcache;          // [backlog][H*R] fp16
+    const float *kin, *vin;             // or null: the batch's own K and V rows [n][H*R], which this kernel then also appends to the
+                                        // cache (copy_to_cache.comp:29-37: rounded to fp16) and uses as rounded
+    const float2 *trig_abs;             // [backlog][R/2] (cos, sin) of p * theta_i
+    const uint32_t *pos_ptr;
+    uint32_t pos_add;                   // row 0 of the batch sits at *pos_ptr + pos_add
+    uint32_t n, heads, backlog;
+};
+
+// planes of positions 0 .. pos + n - 1 of one layer; grid (heads, tiles of 64 positions), tiles past the last position return.
+// Given the batch's fresh K and V rows it is also the cache append of the batch.
+template <int R>
+__global__ __launch_bounds__(256) void attention_prepare_kernel(AttnPrepArgs a)
+{
+    constexpr int TK = kAttnBatchK, C8 = R / 8, VS = R + 2;     // VS: row stride of the staged V tile in halfs
+    __shared__ uint32_t vs[TK * VS / 2];
+    const uint32_t h = blockIdx.x, k0 = blockIdx.y * TK;
+    const uint32_t D = a.heads * R, rows64 = attn_rows64(a.backlog);
+    const uint32_t pos0 = (a.pos_ptr ? *a.pos_ptr : 0u) + a.pos_add;
+    const uint32_t rows = min(pos0 + a.n, a.backlog);           // positions 0 .. rows-1 hold data
+    if (k0 >= rows) return;
+    const int t = threadIdx.x;
+    for (int g = t; g < C8 * TK; g += 256) {
+        const int c8 = g % C8, row = g / C8;
+        const uint32_t p = k0 + row;
+        float f[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        uint4 vraw = make_uint4(0u, 0u, 0u, 0u);                // rows past the data: zeros, which the masked sums can take
+        if (p < rows) {
+            const size_t o = (size_t)p * D + (size_t)h * R + c8 * 8;
+            uint4 kraw;
+            if (a.kin && p >= pos0) {
+                const size_t oi = (size_t)(p - pos0) * D + (size_t)h * R + c8 * 8;
+                const float4 k0v = *reinterpret_cast<const float4 *>(a.kin + oi), k1v = *reinterpret_cast<const float4 *>(a.kin + oi + 4);
+                const float4 v0v = *reinterpret_cast<const float4 *>(a.vin + oi), v1v = *reinterpret_cast<const float4 *>(a.vin + oi + 4);
+                auto pack = [](float lo, float hi) { return (uint32_t)float_to_half_bits(lo) | ((uint32_t)float_to_half_bits(hi) << 16); };
+                kraw = make_uint4(pack(k0v.x, k0v.y), pack(k0v.z, k0v.w), pack(k1v.x, k1v.y), pack(k1v.z, k1v.w));
+                vraw = make_uint4(pack(v0v.x, v0v.y), pack(v0v.z, v0v.w), pack(v1v.x, v1v.y), pack(v1v.z, v1v.w));
+                *reinterpret_cast<uint4 *>(a.kcache + o) = kraw;
+                *reinterpret_cast<uint4 *>(a.vcache + o) = vraw;
+            } else {
+                kraw = *reinterpret_cast<const uint4 *>(a.kcache + o);
+                vraw = *reinterpret_cast<const uint4 *>(a.vcache + o);
+            }
+            const float4 cs0 = *reinterpret_cast<const float4 *>(a.trig_abs + (size_t)p * (R / 2) + c8 * 4);
+            const float4 cs1 = *reinterpret_cast<const float4 *>(a.trig_abs + (size_t)p * (R / 2) + c8 * 4 + 2);
+            const uint32_t kw[4] = {kraw.x, kraw.y, kraw.z, kraw.w};
+            const float c[4] = {cs0.x, cs0.z, cs1.x, cs1.z}, s[4] = {cs0.y, cs0.w, cs1.y, cs1.w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                // e^{i phi} (x + i y) = (x c - y s) + i (x s + y c)
+                const float x = half_bits_to_float((uint16_t)(kw[j] & 0xffffu)), y = half_bits_to_float((uint16_t)(kw[j] >> 16));
+                f[2 * j] = x * c[j] - y * s[j];
+                f[2 * j + 1] = x * s[j] + y * c[j];
+            }
+        }
+        uint4 hi, lo;
+        gemm_split8(hi, lo, f);
+        const size_t ok = (size_t)p * D + (size_t)h * R + c8 * 8;   // p < rows64: the planes have that many rows
+        *reinterpret_cast<uint4 *>(a.pl.kh + ok) = hi;
+        *reinterpret_cast<uint4 *>(a.pl.kl + ok) = lo;
+        uint32_t *vrow = vs + (row * VS + c8 * 8) / 2;
+        vrow[0] = vraw.x; vrow[1] = vraw.y; vrow[2] = vraw.z; vrow[3] = vraw.w;
+    }
+    __syncthreads();
+    const uint16_t *vh = reinterpret_cast<const uint16_t *>(vs);
+    for (int g = t; g < R * 8; g += 256) {
+        const int c = g % 8, dim = g / 8;                       // chunk c of the tile's row of this dim: slots 8c .. 8c+7
+        uint32_t w1[4], w2[4];
+#pragma unroll
+        for (int e = 0; e < 8; e += 2) {
+            uint32_t b1[2], b2[2];
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                const int slot = 8 * c + e + u, pos = (slot & ~15) + attn_slot_pos(slot & 15);
+                const float v = half_bits_to_float(vh[pos * VS + dim]);
+                b1[u] = __float_as_uint(v) & 0xffff0000u;
+                b2[u] = __float_as_uint(v - __uint_as_float(b1[u]));    // three bits at most: the cut to bf16 below loses nothing
+            }
+            w1[e / 2] = (b1[0] >> 16) | b1[1];
+            w2[e / 2] = (b2[0] >> 16) | (b2[1] & 0xffff0000u);
+        }
+        const size_t o = ((size_t)h * R + dim) * rows64 + k0 + 8 * c;
+        *reinterpret_cast<uint4 *>(a.pl.v1 + o) = make_uint4(w1[0], w1[1], w1[2], w1[3]);
+        *reinterpret_cast<uint4 *>(a.pl.v2 + o) = make_uint4(w2[0], w2[1], w2[2], w2[3]);
+    }
+}
+
 struct AttnBatchArgs {
-    float *out;             // [n][H*R]
-    const uint16_t *kcache; // [backlog][H*R] fp16
-    const uint16_t *vcache;
+    float *out;             // [n][H*R], or null
+    uint16_t *xh, *xl;      // or: the result as the two fp16 halves the output projection's GEMM reads (tile order, width Kp,
+                            // rows n .. n_pad-1 zero), or null
+    AttnPlanes pl;
     const float *q;         // [n][H*R]
     const float2 *trig_abs; // [backlog][R/2] (cos, sin) of p * theta_i
     const uint32_t *pos_ptr;
     uint32_t pos_add;       // row z of the batch sits at *pos_ptr + pos_add + z
-    uint32_t n, heads, backlog;
+    uint32_t n, heads, backlog, Kp;
 };
 
-typedef float lv_f32x16 __attribute__((ext_vector_type(16)));
-
+// LDS chunk permutation of the K planes: rows of 2R bytes; eight consecutive rows at one chunk must fall into eight
+// different 16-byte columns of the 128-byte bank row
 template <int R>
-struct AttnBatchLds {
-    static constexpr int KP = R / 2 + 4;     // row stride of kx / ky in floats (16-byte aligned, rows start in different banks)
-    static constexpr int VP = kAttnBatchK / 2 + 8;   // row stride of vt in halfs
-    static constexpr int PP = 16 + 4;        // row stride of the probability tiles in floats
-    float kx[kAttnBatchK][KP], ky[kAttnBatchK][KP];   // rotated K: components 2i and 2i+1 of the pairs
-    uint16_t vt[2][R][VP];                   // V transposed: [position parity][dim][position / 2], 8-byte units permuted:
-    // unit u (positions / 2 = 4u .. 4u+3) of the row of a dim in group c8 = dim / 8 is stored at unit u ^ (c8 & 7)
-    __device__ static constexpr int vt_unit(int u, int c8) { return u ^ (c8 & 7); }
-    float ps[4][2][32][PP];                  // per wave: exp(score) [position parity][query row][position / 2]
-    float den[2][2][32];                     // [position tile][query tile][query row]
-};
+__device__ __forceinline__ int attn_kswz(int row) { return R >= 64 ? (row & 7) : ((row >> 1) & 3); }
 
+// grid (heads, query tiles of 64 over the padded batch); dynamic LDS: 1024 R bytes
 template <int R>
 __global__ __launch_bounds__(256) void attention_batch_kernel(AttnBatchArgs a)
 {
     constexpr int TQ = kAttnBatchQ, TK = kAttnBatchK;
-    constexpr int KS = R / 2;     // MFMA steps of a score tile (2 k each)
-    constexpr int DT = R / 32;    // 32-wide tiles of the head dimension
-    using L = AttnBatchLds<R>;
-    __shared__ __attribute__((aligned(16))) L l;
+    constexpr int KS = R / 16;                  // MFMA steps of a score tile (16 k each)
+    constexpr int DT = R / 32;                  // 32-wide tiles of the head dimension
+    constexpr int PLANE = TK * R * 2;           // bytes of one plane of a tile (K: 64 rows of 2R bytes; V: R rows of 128 bytes)
+    constexpr int STAGE = 4 * PLANE;            // kh, kl, v1, v2
+    constexpr int NI = PLANE / 1024;            // direct loads (1 KB per wave instruction) per plane
+    constexpr int XS = R + 4;                   // row stride of the result exchange in floats
+    static_assert(TQ * XS * 4 <= 2 * STAGE, "the result exchange reuses the tile buffers");
+    extern __shared__ __attribute__((aligned(16))) uint8_t attn_lds[];
+    __shared__ float den_s[2][2][32];           // [position tile][query tile][query row]
     // the last query tile walks the most cache tiles: it is dispatched first, so the short ones fill the tail
     const uint32_t h = blockIdx.x, z0 = (gridDim.y - 1 - blockIdx.y) * TQ;
-    const uint32_t H = a.heads, D = H * R;
+    const uint32_t H = a.heads, D = H * R, rows64 = attn_rows64(a.backlog);
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    if (z0 >= a.n) {        // rows of the padded batch: zero halves
+        if (a.xh)
+            for (int g = t; g < TQ * (R / 8); g += 256) {
+                const size_t o = gemm_x_offset(z0 + g / (R / 8), h * R + (g % (R / 8)) * 8, a.Kp);
+                *reinterpret_cast<uint4 *>(a.xh + o) = make_uint4(0u, 0u, 0u, 0u);
+                *reinterpret_cast<uint4 *>(a.xl + o) = make_uint4(0u, 0u, 0u, 0u);
+            }
+        return;
+    }
     const uint32_t pos0 = (a.pos_ptr ? *a.pos_ptr : 0u) + a.pos_add;  // cache position of batch row 0
-    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int qt = wave & 1, pt = wave >> 1;      // this wave's query tile and position sub-tile
     const int n32 = lane & 31, hh = lane >> 5;
     const uint32_t last_row = min(z0 + TQ, a.n) - 1;                  // last query row of the workgroup
     const uint32_t last_pos = min(pos0 + last_row, a.backlog - 1);    // newest position any of them sees
+    const uint32_t steps = last_pos / TK + 1;
 
-    // ---- this lane's query operands: row n32 of the wave's tile, rotated to its own position ------------------
-    // operand j of the score MFMAs is component 2j + hh of q' (hh = 0: x of pair j, hh = 1: y of pair j)
-    float qf[KS];
+    // ---- direct loads of the tile at k0 into buffer s: every wave issues NI / 4 (at least one) per plane ------------------
+    const uint8_t *const gkh = reinterpret_cast<const uint8_t *>(a.pl.kh), *const gkl = reinterpret_cast<const uint8_t *>(a.pl.kl);
+    const uint8_t *const gv1 = reinterpret_cast<const uint8_t *>(a.pl.v1), *const gv2 = reinterpret_cast<const uint8_t *>(a.pl.v2);
+    auto issue = [&](int s, uint32_t k0) {
+        uint8_t *buf = attn_lds + s * STAGE;
+#pragma unroll
+        for (int i0 = 0; i0 < NI; i0 += 4) {
+            const int i = i0 + wave;
+            if (NI < 4 && i >= NI) break;
+            const int byte = 1024 * i + 16 * lane;
+            const int row = byte / (2 * R), c = ((byte % (2 * R)) / 16) ^ attn_kswz<R>(row);
+            const size_t gk = ((size_t)(k0 + row) * D + (size_t)h * R + c * 8) * 2;
+            __builtin_amdgcn_global_load_lds((lv_glb_void *)(gkh + gk), (lv_lds_void *)(buf + 1024 * i), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((lv_glb_void *)(gkl + gk), (lv_lds_void *)(buf + PLANE + 1024 * i), 16, 0, 0);
+            const int dim = byte / 128, cv = (lane & 7) ^ (dim & 7);
+            const size_t gv = (((size_t)h * R + dim) * rows64 + k0 + 8 * cv) * 2;
+            __builtin_amdgcn_global_load_lds((lv_glb_void *)(gv1 + gv), (lv_lds_void *)(buf + 2 * PLANE + 1024 * i), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((lv_glb_void *)(gv2 + gv), (lv_lds_void *)(buf + 3 * PLANE + 1024 * i), 16, 0, 0);
+        }
+    };
+    issue(0, 0);
+
+    // ---- this lane's query operands: row n32 of the wave's tile, rotated to its own position, as fp16 pairs -------------
+    // operand j holds components 16 j + 8 hh .. + 7 of q' (pairs 8 j + 4 hh .. + 3)
+    lv_h8 qh[KS], ql[KS];
+    const uint32_t zq = z0 + 32 * qt + n32;
+    const bool zok = zq < a.n;
     {
-        const uint32_t z = z0 + 32 * qt + n32;
-        const bool zok = z < a.n;
-        const uint32_t pq = min(pos0 + z, a.backlog - 1);
-        const float *qr = a.q + (size_t)(zok ? z : 0) * D + (size_t)h * R;
+        const uint32_t pq = min(pos0 + zq, a.backlog - 1);
+        const float *qr = a.q + (size_t)(zok ? zq : 0) * D + (size_t)h * R;
         const float2 *tr = a.trig_abs + (size_t)pq * (R / 2);
 #pragma unroll
-        for (int j = 0; j < KS; j += 2) {
-            const float4 q2 = *reinterpret_cast<const float4 *>(qr + 2 * j);      // pairs j, j + 1
-            const float4 cs = *reinterpret_cast<const float4 *>(tr + j);          // (c, s) of pairs j, j + 1
+        for (int j = 0; j < KS; j++) {
+            const float4 q0 = *reinterpret_cast<const float4 *>(qr + 16 * j + 8 * hh), q1 = *reinterpret_cast<const float4 *>(qr + 16 * j + 8 * hh + 4);
+            const float4 c0 = *reinterpret_cast<const float4 *>(tr + 8 * j + 4 * hh), c1 = *reinterpret_cast<const float4 *>(tr + 8 * j + 4 * hh + 2);
             // e^{i phi} (x + i y) = (x c - y s) + i (x s + y c)
-            const float x0 = q2.x * cs.x - q2.y * cs.y, y0 = q2.x * cs.y + q2.y * cs.x;
-            const float x1 = q2.z * cs.z - q2.w * cs.w, y1 = q2.z * cs.w + q2.w * cs.z;
-            qf[j] = zok ? (hh ? y0 : x0) : 0.f;
-            qf[j + 1] = zok ? (hh ? y1 : x1) : 0.f;
+            float f[8] = {q0.x * c0.x - q0.y * c0.y, q0.x * c0.y + q0.y * c0.x, q0.z * c0.z - q0.w * c0.w, q0.z * c0.w + q0.w * c0.z,
+                          q1.x * c1.x - q1.y * c1.y, q1.x * c1.y + q1.y * c1.x, q1.z * c1.z - q1.w * c1.w, q1.z * c1.w + q1.w * c1.z};
+            if (!zok) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) f[e] = 0.f;
+            }
+            uint4 hi, lo;
+            gemm_split8(hi, lo, f);
+            qh[j] = __builtin_bit_cast(lv_h8, hi);
+            ql[j] = __builtin_bit_cast(lv_h8, lo);
         }
     }
 
     const float scale = rsqrtf((float)R);
-    lv_f32x16 acc[DT];
+    lv_f16v acc[DT];
 #pragma unroll
     for (int d = 0; d < DT; d++)
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[d][r] = 0.f;
-    float den = 0.f;      // sum of this lane's probability operands: query row n32, positions of parity hh
+    float den = 0.f;      // sum of this lane's probabilities: query row n32, the positions this lane's registers hold
+    const uint32_t wave_last = pos0 + min(z0 + 32 * qt + 31, a.n - 1);   // newest position a query of this wave's tile sees
+    const uint32_t limit = pos0 + zq;                                     // newest position this lane's query sees
 
-    for (uint32_t k0 = 0; k0 <= last_pos; k0 += TK) {
-        __syncthreads();  // the previous tile is consumed
-        // ---- stage K (rotated, fp32) and V (transposed, fp16) of this tile ------------------------------------------
-        // a thread takes eight dims (c8) of four positions of one parity, base + par + 2m: their V halfs are neighbours
-        // in the transposed tile and go out as one 8-byte store per dim.  The 8-byte units of a vt row are permuted by
-        // the row's c8 (vt_unit), which spreads the stores of a wave's sixteen c8 over the banks.
-        for (int g = t; g < (R / 8) * 16; g += 256) {
-            const int c8 = g % (R / 8), rg = g / (R / 8), par = rg & 1, base = (rg >> 1) * 8;
-            uint4 kraw[4], vraw[4];
-            float4 cs0[4], cs1[4];
-#pragma unroll
-            for (int m = 0; m < 4; m++) {
-                const uint32_t p = min(k0 + base + par + 2 * m, a.backlog - 1);
-                kraw[m] = *reinterpret_cast<const uint4 *>(a.kcache + (size_t)p * D + (size_t)h * R + c8 * 8);
-                vraw[m] = *reinterpret_cast<const uint4 *>(a.vcache + (size_t)p * D + (size_t)h * R + c8 * 8);
-                cs0[m] = *reinterpret_cast<const float4 *>(a.trig_abs + (size_t)p * (R / 2) + c8 * 4);
-                cs1[m] = *reinterpret_cast<const float4 *>(a.trig_abs + (size_t)p * (R / 2) + c8 * 4 + 2);
-            }
-#pragma unroll
-            for (int m = 0; m < 4; m++) {
-                const int row = base + par + 2 * m;
-                const uint32_t kw[4] = {kraw[m].x, kraw[m].y, kraw[m].z, kraw[m].w};
-                const float c[4] = {cs0[m].x, cs0[m].z, cs1[m].x, cs1[m].z}, s[4] = {cs0[m].y, cs0[m].w, cs1[m].y, cs1[m].w};
-                float xr[4], yr[4];
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    const float x = half_bits_to_float((uint16_t)(kw[j] & 0xffffu)), y = half_bits_to_float((uint16_t)(kw[j] >> 16));
-                    xr[j] = x * c[j] - y * s[j];
-                    yr[j] = x * s[j] + y * c[j];
-                }
-                *reinterpret_cast<float4 *>(&l.kx[row][c8 * 4]) = make_float4(xr[0], xr[1], xr[2], xr[3]);
-                *reinterpret_cast<float4 *>(&l.ky[row][c8 * 4]) = make_float4(yr[0], yr[1], yr[2], yr[3]);
-            }
-            const uint32_t vw[4][4] = {{vraw[0].x, vraw[0].y, vraw[0].z, vraw[0].w}, {vraw[1].x, vraw[1].y, vraw[1].z, vraw[1].w},
-                                       {vraw[2].x, vraw[2].y, vraw[2].z, vraw[2].w}, {vraw[3].x, vraw[3].y, vraw[3].z, vraw[3].w}};
-            const int unit = L::vt_unit(rg >> 1, c8);
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                // dims c8*8 + 2j (low halfs) and + 2j + 1 (high halfs) at positions m = 0..3
-                const uint2 lo = make_uint2((vw[0][j] & 0xffffu) | (vw[1][j] << 16), (vw[2][j] & 0xffffu) | (vw[3][j] << 16));
-                const uint2 hi = make_uint2((vw[0][j] >> 16) | (vw[1][j] & 0xffff0000u), (vw[2][j] >> 16) | (vw[3][j] & 0xffff0000u));
-                *reinterpret_cast<uint2 *>(&l.vt[par][c8 * 8 + 2 * j][unit * 4]) = lo;
-                *reinterpret_cast<uint2 *>(&l.vt[par][c8 * 8 + 2 * j + 1][unit * 4]) = hi;
-            }
-        }
-        __syncthreads();
+    for (uint32_t it = 0; it < steps; it++) {
+        const uint32_t k0 = it * TK;
+        __syncthreads();      // this tile's loads have landed (the barrier waits for the loads in flight); the other buffer is consumed
+        if (it + 1 < steps) issue((it + 1) & 1, k0 + TK);
+        if (k0 + 32 * pt > wave_last) continue;       // every pair of this wave's 32 x 32 tile is masked
+        const uint8_t *kb = attn_lds + (it & 1) * STAGE, *vb = kb + 2 * PLANE;
 
-        // ---- scores of (query tile qt) x (positions k0 + 32 pt ..): S = Q' K'^T ----------------------------------------
-        lv_f32x16 sc;
+        // ---- scores, transposed: S^T = K' Q'^T; rows = positions k0 + 32 pt .., columns = queries ---------------------------
+        lv_f16v sc;
 #pragma unroll
         for (int r = 0; r < 16; r++) sc[r] = 0.f;
         {
-            const float *kr = hh ? &l.ky[32 * pt + n32][0] : &l.kx[32 * pt + n32][0];   // position n32 of the sub-tile
+            const int row = 32 * pt + n32;
+            const uint8_t *kr = kb + row * 2 * R;
+            const int sw = attn_kswz<R>(row);
 #pragma unroll
-            for (int j = 0; j < KS; j += 4) {
-                const float4 k4 = *reinterpret_cast<const float4 *>(kr + j);
-                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(qf[j], k4.x, sc, 0, 0, 0);
-                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(qf[j + 1], k4.y, sc, 0, 0, 0);
-                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(qf[j + 2], k4.z, sc, 0, 0, 0);
-                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(qf[j + 3], k4.w, sc, 0, 0, 0);
+            for (int j = 0; j < KS; j++) {
+                const int c = (2 * j + hh) ^ sw;
+                const lv_h8 ah = *reinterpret_cast<const lv_h8 *>(kr + c * 16), al = *reinterpret_cast<const lv_h8 *>(kr + PLANE + c * 16);
+                sc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, ql[j], sc, 0, 0, 0);
+                sc = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, qh[j], sc, 0, 0, 0);
+                sc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, qh[j], sc, 0, 0, 0);
             }
         }
-        // in sc a lane holds position n32 of the sub-tile and query rows i = 8 (r / 4) + 4 hh + r % 4
-        {
-            const uint32_t p = k0 + 32 * pt + n32;
-            float *prow = &l.ps[wave][n32 & 1][0][n32 >> 1];
+        // register r of sc: position k0 + 32 pt + 8 (r / 4) + 4 hh + r % 4, query n32 of the wave's tile
+        // ---- O += P V, sixteen positions (registers 8t .. 8t+7 of both lane halves) at a time --------------------------------
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int i = 8 * (r / 4) + 4 * hh + (r % 4);
-                const uint32_t z = z0 + 32 * qt + i;
-                const bool ok = z < a.n && p <= pos0 + z && p < a.backlog;
-                prow[i * L::PP] = ok ? __expf(sc[r] * scale) : 0.f;
+        for (int tt = 0; tt < 2; tt++) {
+            uint32_t w1[4], w2[4], w3[4];
+#pragma unroll
+            for (int e = 0; e < 8; e += 2) {
+                uint32_t b1[2], b2[2], b3[2];
+#pragma unroll
+                for (int u = 0; u < 2; u++) {
+                    const int r = 8 * tt + e + u;
+                    const uint32_t p = k0 + 32 * pt + 8 * (r / 4) + 4 * hh + (r % 4);
+                    const bool ok = zok && p <= limit && p < a.backlog;
+                    const float e0 = ok ? __expf(sc[r] * scale) : 0.f;
+                    den += e0;
+                    b1[u] = __float_as_uint(e0) & 0xffff0000u;
+                    const float r1 = e0 - __uint_as_float(b1[u]);
+                    b2[u] = __float_as_uint(r1) & 0xffff0000u;
+                    b3[u] = __float_as_uint(r1 - __uint_as_float(b2[u]));   // eight bits at most are left
+                }
+                w1[e / 2] = (b1[0] >> 16) | b1[1];
+                w2[e / 2] = (b2[0] >> 16) | b2[1];
+                w3[e / 2] = (b3[0] >> 16) | (b3[1] & 0xffff0000u);
             }
-        }
-        // ---- O += P V: the probabilities come back as the A operand (row = query n32, k = position 2j + hh) ------------
-        float pf[16];
-        {
-            const float *pr = &l.ps[wave][hh][n32][0];
+            const lv_b8 p1 = __builtin_bit_cast(lv_b8, make_uint4(w1[0], w1[1], w1[2], w1[3]));
+            const lv_b8 p2 = __builtin_bit_cast(lv_b8, make_uint4(w2[0], w2[1], w2[2], w2[3]));
+            const lv_b8 p3 = __builtin_bit_cast(lv_b8, make_uint4(w3[0], w3[1], w3[2], w3[3]));
 #pragma unroll
-            for (int j = 0; j < 16; j += 4) {
-                const float4 p4 = *reinterpret_cast<const float4 *>(pr + j);
-                pf[j] = p4.x; pf[j + 1] = p4.y; pf[j + 2] = p4.z; pf[j + 3] = p4.w;
-                den += (p4.x + p4.y) + (p4.z + p4.w);
-            }
-        }
-#pragma unroll
-        for (int d = 0; d < DT; d++) {
-            // B operand: V[position 32 pt + 2j + hh][dim 32 d + n32], sixteen consecutive halfs of the transposed tile
-            const int dim = 32 * d + n32;
-            uint32_t vw[8];
-#pragma unroll
-            for (int u = 0; u < 4; u++) {
-                const uint2 v2 = *reinterpret_cast<const uint2 *>(&l.vt[hh][dim][L::vt_unit(4 * pt + u, dim >> 3) * 4]);
-                vw[2 * u] = v2.x;
-                vw[2 * u + 1] = v2.y;
-            }
-#pragma unroll
-            for (int j = 0; j < 8; j++) {
-                acc[d] = __builtin_amdgcn_mfma_f32_32x32x2f32(pf[2 * j], half_bits_to_float((uint16_t)(vw[j] & 0xffffu)), acc[d], 0, 0, 0);
-                acc[d] = __builtin_amdgcn_mfma_f32_32x32x2f32(pf[2 * j + 1], half_bits_to_float((uint16_t)(vw[j] >> 16)), acc[d], 0, 0, 0);
+            for (int d = 0; d < DT; d++) {
+                const int dim = 32 * d + n32, c = (4 * pt + 2 * tt + hh) ^ (dim & 7);
+                const lv_b8 va = *reinterpret_cast<const lv_b8 *>(vb + dim * 128 + c * 16);
+                const lv_b8 vc = *reinterpret_cast<const lv_b8 *>(vb + PLANE + dim * 128 + c * 16);
+                acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(p3, va, acc[d], 0, 0, 0);
+                acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(p2, vc, acc[d], 0, 0, 0);
+                acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(p2, va, acc[d], 0, 0, 0);
+                acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(p1, vc, acc[d], 0, 0, 0);
+                acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(p1, va, acc[d], 0, 0, 0);
             }
         }
     }
 
     // ---- combine the two position tiles, divide, write -------------------------------------------------------------
-    den += __shfl_xor(den, 32, kWave);                    // both parities: all positions this wave saw, query row n32
-    if (hh == 0) l.den[pt][qt][n32] = den;
-    __syncthreads();                                      // also: every wave is done with kx / ky
-    static_assert(sizeof(l.kx) + sizeof(l.ky) >= (size_t)2 * DT * 16 * 64 * sizeof(float) && offsetof(L, ky) == offsetof(L, kx) + sizeof(l.kx),
-                  "the exchange area below spans kx and ky");
-    float *xch = &l.kx[0][0];                             // reused: [query tile][dim tile][register][lane]
+    // acc[d][r]: query row 8 (r / 4) + 4 hh + r % 4 of the wave's tile, dim 32 d + n32
+    den += __shfl_xor(den, 32, kWave);                    // both lane halves: all positions this wave saw, query row n32
+    if (hh == 0) den_s[pt][qt][n32] = den;
+    __syncthreads();                                      // also: every wave is done with the tile buffers
+    float *xch = reinterpret_cast<float *>(attn_lds);     // [query row of the workgroup][XS]
     if (pt == 1) {
 #pragma unroll
         for (int d = 0; d < DT; d++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) xch[((qt * DT + d) * 16 + r) * 64 + lane] = acc[d][r];
+            for (int r = 0; r < 16; r++) xch[(32 * qt + 8 * (r / 4) + 4 * hh + (r % 4)) * XS + 32 * d + n32] = acc[d][r];
     }
     __syncthreads();
     if (pt == 0) {
@@ -224,12 +339,33 @@ __global__ __launch_bounds__(256) void attention_batch_kernel(AttnBatchArgs a)
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int i = 8 * (r / 4) + 4 * hh + (r % 4);
-                const uint32_t z = z0 + 32 * qt + i;
-                if (z < a.n) {
-                    const float total = acc[d][r] + xch[((qt * DT + d) * 16 + r) * 64 + lane];
-                    a.out[(size_t)z * D + (size_t)h * R + 32 * d + n32] = total / (l.den[0][qt][i] + l.den[1][qt][i]);
-                }
+                float *x = &xch[(32 * qt + i) * XS + 32 * d + n32];
+                *x = (acc[d][r] + *x) / (den_s[0][qt][i] + den_s[1][qt][i]);
             }
+    }
+    __syncthreads();
+    for (int g = t; g < TQ * (R / 8); g += 256) {
+        const int row = g / (R / 8), c8 = g % (R / 8);
+        const uint32_t z = z0 + row;
+        const float4 x0 = *reinterpret_cast<const float4 *>(&xch[row * XS + c8 * 8]), x1 = *reinterpret_cast<const float4 *>(&xch[row * XS + c8 * 8 + 4]);
+        const bool live = z < a.n;
+        if (a.out && live) {
+            float *o = a.out + (size_t)z * D + (size_t)h * R + c8 * 8;
+            *reinterpret_cast<float4 *>(o) = x0;
+            *reinterpret_cast<float4 *>(o + 4) = x1;
+        }
+        if (a.xh) {
+            float f[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+            if (!live) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) f[e] = 0.f;
+            }
+            uint4 hi, lo;
+            gemm_split8(hi, lo, f);
+            const size_t o = gemm_x_offset(z, h * R + c8 * 8, a.Kp);
+            *reinterpret_cast<uint4 *>(a.xh + o) = hi;
+            *reinterpret_cast<uint4 *>(a.xl + o) = lo;
+        }
     }
 }
 

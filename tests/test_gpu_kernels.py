@@ -129,6 +129,10 @@ def test_kv_append_bit_exact(lva, orc, ctx, dim, batch, pos, backlog):
 @pytest.mark.parametrize("heads,rot,backlog,pos,batch", [
     (32, 128, 128, 0, 1), (32, 128, 128, 40, 1), (32, 128, 128, 127, 1), (4, 64, 128, 77, 1), (16, 32, 64, 63, 1),
     (40, 128, 256, 200, 1), (32, 128, 512, 511, 1), (4, 64, 128, 10, 4), (2, 128, 256, 250, 3),
+    # 16 rows and more: the kernels of a prompt batch (16-bit matrix-core products of split operands)
+    # (the oracle's tree sums want a power-of-two backlog, as the shaders do)
+    (4, 128, 256, 37, 100), (8, 64, 256, 0, 150), (5, 32, 128, 3, 120), (3, 128, 64, 0, 16), (2, 128, 512, 283, 17),
+    (2, 64, 32, 5, 20), (40, 128, 512, 0, 512),
 ])
 def test_attention_matches_oracle(lva, orc, ctx, heads, rot, backlog, pos, batch):
     dim = heads * rot
