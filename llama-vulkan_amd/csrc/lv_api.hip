@@ -95,6 +95,7 @@ struct lv_matrix {
 struct LayerWeights {
     lv_matrix wq, wk, wv, wo, w1, w2, w3;
     const float *attn_norm = nullptr, *ffn_norm = nullptr;
+    const uint16_t *gate_up16 = nullptr;   // pair copy of w3 and w1 (in place of their own prompt copies) where they can share one
 };
 
 struct lv_model {
@@ -168,6 +169,7 @@ struct lv_session {
     uint32_t pf_cap = 0;
     float *pf_x = nullptr, *pf_xn = nullptr, *pf_q = nullptr, *pf_k = nullptr, *pf_v = nullptr, *pf_vo = nullptr, *pf_g1 = nullptr, *pf_g2 = nullptr;
     uint16_t *pf_xh = nullptr, *pf_xl = nullptr;
+    uint16_t *pf_fh = nullptr, *pf_fl = nullptr;   // the feed-forward's inner activations (their producer still reads pf_xh / pf_xl)
     float *pf_xs = nullptr;   // per token: the power of two the halves written by prefill_norm_kernel are scaled down by
     // operand planes of the batched attention (one layer's worth, rewritten per layer): four of attn_plane_halfs() each
     uint16_t *pf_planes = nullptr;
@@ -769,9 +771,27 @@ static int launch_expand(hipStream_t st, uint16_t *dst, const lv_matrix &w)
 {
     const uint64_t threads = (uint64_t)gemm_rows_padded(w.view.rows) * (gemm_k_padded(w.view.cols) / 32);
     const dim3 grid((unsigned)((threads + 255) / 256));
-    if (w.ftype == LV_Q4_0) expand_codes_kernel<4><<<grid, dim3(256), 0, st>>>(dst, w.view);
-    else if (w.ftype == LV_Q8_0) expand_codes_kernel<8><<<grid, dim3(256), 0, st>>>(dst, w.view);
+    if (w.ftype == LV_Q4_0) expand_codes_kernel<4, false><<<grid, dim3(256), 0, st>>>(dst, w.view, w.view);
+    else if (w.ftype == LV_Q8_0) expand_codes_kernel<8, false><<<grid, dim3(256), 0, st>>>(dst, w.view, w.view);
     else return fail(LV_ERR_ARG, "gemm: matrix type %u", w.ftype);
+    HIP_TRY(hipGetLastError());
+    return LV_OK;
+}
+
+// The feed-forward's gate (W3) and up (W1) matrices as one pair copy (expand_codes_kernel<.., true>), whose GEMM applies
+// SwiGLU in its epilogue.  Possible when the two have one shape, type and kind of scale plane and 128 divides their rows.
+static bool gemm_same(const lv_matrix &a, const lv_matrix &b);
+static bool gemm_pairable(const lv_matrix &gate, const lv_matrix &up)
+{
+    return gemm_same(gate, up) && gate.view.rows % 128 == 0 && (gate.ftype == LV_Q4_0 || gate.ftype == LV_Q8_0);
+}
+static uint64_t pair_copy_halfs(const lv_matrix &gate) { return gemm_copy_halfs(2 * gate.view.rows, gate.view.cols); }
+static int launch_expand_pair(hipStream_t st, uint16_t *dst, const lv_matrix &gate, const lv_matrix &up)
+{
+    const uint64_t threads = (uint64_t)gemm_rows_padded(2 * gate.view.rows) * (gemm_k_padded(gate.view.cols) / 32);
+    const dim3 grid((unsigned)((threads + 255) / 256));
+    if (gate.ftype == LV_Q4_0) expand_codes_kernel<4, true><<<grid, dim3(256), 0, st>>>(dst, gate.view, up.view);
+    else expand_codes_kernel<8, true><<<grid, dim3(256), 0, st>>>(dst, gate.view, up.view);
     HIP_TRY(hipGetLastError());
     return LV_OK;
 }
@@ -783,11 +803,26 @@ static int dispatch_gemm(hipStream_t st, GemmArgs a, const lv_matrix &w, uint32_
     for (uint32_t i = 0; i < nz; i++)
         if (!a.w16[i]) return fail(LV_ERR_STATE, "gemm: the matrix has no prompt copy");
     // 132 KB of dynamic LDS need the attribute on the device the launch goes to; setting it is a host-side table entry
-    HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLdsBytes));
+    HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_kernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLdsBytes));
     const uint32_t token_tiles = (a.n + kGemmTile - 1) / kGemmTile, row_tiles = (a.rows + kGemmRows - 1) / kGemmRows;
     a.nz = nz;
     const dim3 grid((row_tiles * nz + 7) / 8 * 8 * token_tiles);
-    gemm_kernel<<<grid, dim3(512), kGemmLdsBytes, st>>>(a);
+    gemm_kernel<false><<<grid, dim3(512), kGemmLdsBytes, st>>>(a);
+    HIP_TRY(hipGetLastError());
+    return LV_OK;
+}
+
+// fh, fl (tile order, n_pad x gemm_k_padded(F)) = the halves of SwiGLU(x W3^T, x W1^T) for the pair copy `pair16` of two F x K matrices
+static int launch_gemm_silu(hipStream_t st, uint16_t *fh, uint16_t *fl, const uint16_t *pair16, uint32_t F, uint32_t K, uint32_t n,
+                            const uint16_t *xh, const uint16_t *xl, const float *xscale)
+{
+    GemmArgs a{};
+    a.xh = xh; a.xl = xl; a.n = n; a.xscale = xscale; a.w16[0] = pair16; a.rows = 2 * F; a.K = K; a.nz = 1;
+    a.fh = fh; a.fl = fl; a.fKp = gemm_k_padded(F);
+    HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLdsBytes));
+    const uint32_t token_tiles = (n + kGemmTile - 1) / kGemmTile, row_tiles = a.rows / kGemmRows;
+    const dim3 grid((row_tiles + 7) / 8 * 8 * token_tiles);
+    gemm_kernel<true><<<grid, dim3(512), kGemmLdsBytes, st>>>(a);
     HIP_TRY(hipGetLastError());
     return LV_OK;
 }
@@ -1303,7 +1338,7 @@ extern "C" int lv_session_destroy(lv_session *s)
     drop_graph(s);
     void *dev[] = {s->kv, s->trig, s->trig_abs, s->x, s->xn, s->q, s->k, s->v, s->vo, s->ff, s->logits, s->attn_part, s->attn_counters,
                    s->cfg, s->argmax_dev, s->trace_buf, s->trace_attn, s->pf_x, s->pf_xn, s->pf_q, s->pf_k, s->pf_v, s->pf_vo, s->pf_g1, s->pf_g2,
-                   s->pf_xh, s->pf_xl, s->pf_xs, s->pf_planes};
+                   s->pf_xh, s->pf_xl, s->pf_xs, s->pf_planes, s->pf_fh, s->pf_fl};
     for (void *p : dev) (void)hipFree(p);
     (void)hipFree(s->xchg[0]);
     (void)hipFree(s->xchg[1]);
@@ -1612,8 +1647,11 @@ static bool ensure_prompt_copy(lv_model *m)
     std::lock_guard<std::mutex> lock(m->prompt_mutex);
     if (m->prompt_state) return m->prompt_state > 0;
     uint64_t halfs = 0;
-    for (LayerWeights &lw : m->layers)
-        for (lv_matrix *x : {&lw.wq, &lw.wk, &lw.wv, &lw.wo, &lw.w1, &lw.w2, &lw.w3}) halfs += prompt_copy_halfs(*x);
+    for (LayerWeights &lw : m->layers) {
+        const bool pair = gemm_pairable(lw.w3, lw.w1);
+        for (lv_matrix *x : {&lw.wq, &lw.wk, &lw.wv, &lw.wo, &lw.w2}) halfs += prompt_copy_halfs(*x);
+        halfs += pair ? pair_copy_halfs(lw.w3) : prompt_copy_halfs(lw.w1) + prompt_copy_halfs(lw.w3);
+    }
     m->prompt_state = -1;
     if (hipMalloc(reinterpret_cast<void **>(&m->prompt_arena), halfs * 2) != hipSuccess) {
         (void)hipGetLastError();
@@ -1622,12 +1660,20 @@ static bool ensure_prompt_copy(lv_model *m)
     }
     uint16_t *at = m->prompt_arena;
     hipStream_t st = m->ctx->stream;
-    for (LayerWeights &lw : m->layers)
-        for (lv_matrix *x : {&lw.wq, &lw.wk, &lw.wv, &lw.wo, &lw.w1, &lw.w2, &lw.w3}) {
+    for (LayerWeights &lw : m->layers) {
+        const bool pair = gemm_pairable(lw.w3, lw.w1);
+        for (lv_matrix *x : {&lw.wq, &lw.wk, &lw.wv, &lw.wo, &lw.w2, &lw.w1, &lw.w3}) {
+            if (pair && (x == &lw.w1 || x == &lw.w3)) continue;
             if (launch_expand(st, at, *x) != LV_OK) return false;
             x->h16 = at;
             at += prompt_copy_halfs(*x);
         }
+        if (pair) {
+            if (launch_expand_pair(st, at, lw.w3, lw.w1) != LV_OK) return false;
+            lw.gate_up16 = at;
+            at += pair_copy_halfs(lw.w3);
+        }
+    }
     if (hipStreamSynchronize(st) != hipSuccess) return false;
     m->prompt_state = 1;
     return true;
@@ -1643,11 +1689,12 @@ static int prefill_reserve(lv_session *s, uint32_t n)
     if (cap > s->pf_cap) {
         HIP_TRY(hipStreamSynchronize(s->stream));
         void **bufs[] = {(void **)&s->pf_x, (void **)&s->pf_xn, (void **)&s->pf_q, (void **)&s->pf_k, (void **)&s->pf_v, (void **)&s->pf_vo,
-                         (void **)&s->pf_g1, (void **)&s->pf_g2, (void **)&s->pf_xh, (void **)&s->pf_xl, (void **)&s->pf_xs};
+                         (void **)&s->pf_g1, (void **)&s->pf_g2, (void **)&s->pf_xh, (void **)&s->pf_xl, (void **)&s->pf_xs,
+                         (void **)&s->pf_fh, (void **)&s->pf_fl};
         const size_t halfs = gemm_k_padded((uint32_t)(F > D ? F : D)) * 2;   // an activation half: padded K, 2 bytes each
-        const size_t sizes[] = {D * 4, D * 4, D * 4, D * 4, D * 4, D * 4, F * 4, F * 4, halfs, halfs, 4};
+        const size_t sizes[] = {D * 4, D * 4, D * 4, D * 4, D * 4, D * 4, F * 4, F * 4, halfs, halfs, 4, halfs, halfs};
         s->pf_cap = 0;
-        for (int i = 0; i < 11; i++) {
+        for (int i = 0; i < 13; i++) {
             (void)hipFree(*bufs[i]);
             *bufs[i] = nullptr;
             hipError_t e = hipMalloc(bufs[i], sizes[i] * cap);
@@ -1744,7 +1791,11 @@ static int record_prefill(lv_session *s, uint32_t idx0, uint32_t n, bool with_he
         LV_TRY(launch_gemm_sliced(st, s->pf_x, D, lw.wo, n, s->pf_xh, s->pf_xl, nullptr, true, parts, &pending));
         LV_TRY(launch_prefill_norm(st, s, lw.ffn_norm, n, D, parts, pending, !gate_same, &xscale));
         pending = 0;
-        if (gate_same) {
+        const uint16_t *fh = s->pf_xh, *fl = s->pf_xl;     // where the down projection finds its activations
+        if (lw.gate_up16) {        // SwiGLU in the GEMM's epilogue
+            LV_TRY(launch_gemm_silu(st, s->pf_fh, s->pf_fl, lw.gate_up16, F, D, n, s->pf_xh, s->pf_xl, xscale));
+            fh = s->pf_fh; fl = s->pf_fl;
+        } else if (gate_same) {
             float *const outs[2] = {s->pf_g1, s->pf_g2};
             const lv_matrix *const ws[2] = {&lw.w3, &lw.w1};
             LV_TRY(launch_gemm_multi(st, outs, F, ws, 2, n, s->pf_xh, s->pf_xl, false, xscale));
@@ -1752,14 +1803,14 @@ static int record_prefill(lv_session *s, uint32_t idx0, uint32_t n, bool with_he
             LV_TRY(launch_gemm_presplit(st, s->pf_g1, F, lw.w3, n, s->pf_xh, s->pf_xl, false, xscale));
             LV_TRY(launch_gemm_presplit(st, s->pf_g2, F, lw.w1, n, s->pf_xh, s->pf_xl, false, xscale));
         }
-        {   // SwiGLU straight into the fp16 halves the down projection reads
+        if (!lw.gate_up16) {   // SwiGLU straight into the fp16 halves the down projection reads
             const uint32_t Fp = gemm_k_padded(F);
             const dim3 grid(Fp / 64, (n + kGemmTile - 1) / kGemmTile * kGemmTile / 32);
             if (F % 8) return fail(LV_ERR_ARG, "prompt batch: ff size %u", F);
             silu_split_kernel<<<grid, dim3(256), 0, st>>>(s->pf_xh, s->pf_xl, s->pf_g1, s->pf_g2, n, F, Fp);
             HIP_TRY(hipGetLastError());
         }
-        LV_TRY(launch_gemm_sliced(st, s->pf_x, D, lw.w2, n, s->pf_xh, s->pf_xl, nullptr, true, parts, &pending));
+        LV_TRY(launch_gemm_sliced(st, s->pf_x, D, lw.w2, n, fh, fl, nullptr, true, parts, &pending));
     }
     if (pending) LV_TRY(launch_gemm_reduce(st, s->pf_x, D, parts, pending, D, n, true));
     if (with_head) {

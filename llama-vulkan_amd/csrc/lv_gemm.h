@@ -239,6 +239,11 @@ struct GemmArgs {
     // up (a matrix with few rows and a long K, like the down projection, fills the CUs that way)
     uint32_t slice_k;
     uint32_t nz;                        // matrices or slices in this launch
+    // gemm_kernel<true> only: w16[0] is a PAIR copy (expand_codes_kernel) of rows / 2 gate and rows / 2 up rows, and the
+    // result is not the products but ff = gate * up / (exp(-up) + 1) (matmul_silu_ff.comp:96) as the two fp16 halves the
+    // down projection's GEMM reads: tile order, n_pad x fKp
+    uint16_t *fh, *fl;
+    uint32_t fKp;
 };
 
 // out[n][ldo] (+)= p[0] + p[1] (+ p[2] + p[3]), the K slices of one product, each [n][rows]; always summed in this order
@@ -269,24 +274,32 @@ __global__ void gemm_reduce_kernel(GemmReduceArgs a)
 // The prompt copy of one matrix: codes as fp16 integers (q4_0: q - 8, q8_0: q) and scales as fp32, in the tile order
 // described at the top of this file.  One thread per (row of the padded matrix, block of the padded K); consecutive
 // threads take consecutive rows, so that every 16-byte chunk row they write is next to its neighbour's.
-template <int QT>
-__global__ __launch_bounds__(256) void expand_codes_kernel(uint16_t *__restrict__ dst, MatView m)
+// PAIR: the copy of the feed-forward's two input matrices as ONE matrix of 2 x rows whose 64-row groups (what one wave
+// of gemm_kernel multiplies) hold 32 rows of m followed by the same 32 rows of m2, so that a lane of that wave ends up
+// with both products of its (row, token) and can apply SwiGLU to them.  rows must be a multiple of 128 then.
+__host__ __device__ constexpr uint32_t gemm_pair_row(uint32_t copy_row) { return copy_row / 256 * 128 + (copy_row % 256) / 64 * 32 + copy_row % 32; }
+__host__ __device__ constexpr uint32_t gemm_pair_which(uint32_t copy_row) { return (copy_row % 64) / 32; }
+template <int QT, bool PAIR>
+__global__ __launch_bounds__(256) void expand_codes_kernel(uint16_t *__restrict__ dst, MatView m, MatView m2)
 {
-    const uint32_t Kp = gemm_k_padded(m.cols), rows_pad = gemm_rows_padded(m.rows), nbp = Kp / 32, nb = m.cols / 32;
+    const uint32_t rows_total = PAIR ? 2 * m.rows : m.rows;
+    const uint32_t Kp = gemm_k_padded(m.cols), rows_pad = gemm_rows_padded(rows_total), nbp = Kp / 32, nb = m.cols / 32;
     const uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const uint32_t r = (uint32_t)(t % kGemmRows);
     const uint64_t rest = t / kGemmRows;
     const uint32_t blk = (uint32_t)(rest % nbp), rt = (uint32_t)(rest / nbp);
     const uint32_t row = rt * kGemmRows + r;
     if (row >= rows_pad) return;
-    const bool real = row < m.rows && blk < nb;
+    const uint32_t src_row = PAIR ? gemm_pair_row(row) : row;
+    const MatView &src = (PAIR && gemm_pair_which(row)) ? m2 : m;
+    const bool real = row < rows_total && src_row < m.rows && blk < nb;
     _Float16 v[32];
     float d = 0.f;
     if (real) {
-        const uint64_t sb = (uint64_t)row * nb + blk;
-        d = mat_scale(m, sb);
+        const uint64_t sb = (uint64_t)src_row * nb + blk;
+        d = mat_scale(src, sb);
         if constexpr (QT == 4) {
-            const uint4 c = m.codes[sb];        // byte b: element b in the low nibble, element b + 16 in the high one
+            const uint4 c = src.codes[sb];        // byte b: element b in the low nibble, element b + 16 in the high one
             const uint32_t q[4] = {c.x, c.y, c.z, c.w};
 #pragma unroll
             for (int b = 0; b < 16; b++) {
@@ -295,7 +308,7 @@ __global__ __launch_bounds__(256) void expand_codes_kernel(uint16_t *__restrict_
                 v[b + 16] = (_Float16)((int)(byte >> 4) - 8);
             }
         } else {
-            const uint4 c0 = m.codes[sb * 2], c1 = m.codes[sb * 2 + 1];
+            const uint4 c0 = src.codes[sb * 2], c1 = src.codes[sb * 2 + 1];
             const uint32_t q[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
 #pragma unroll
             for (int b = 0; b < 32; b++) v[b] = (_Float16)(int)(int8_t)((q[b >> 2] >> (8 * (b & 3))) & 0xffu);
@@ -312,7 +325,7 @@ __global__ __launch_bounds__(256) void expand_codes_kernel(uint16_t *__restrict_
         for (int e = 0; e < 8; e++) pk.h[e] = v[8 * c + e];
         *reinterpret_cast<uint4 *>(dst + (((uint64_t)rt * nchunk + (uint64_t)blk * 4 + c) * kGemmRows + r) * 8) = pk.u;
     }
-    float *sc = reinterpret_cast<float *>(dst + gemm_copy_code_halfs(m.rows, m.cols));
+    float *sc = reinterpret_cast<float *>(dst + gemm_copy_code_halfs(rows_total, m.cols));
     sc[((uint64_t)rt * nbp + blk) * kGemmRows + r] = d;
 }
 
@@ -430,6 +443,7 @@ __device__ unsigned long long gemm_clock_words[3];
 // of stage s (which every wave has by then read into registers), and reads the next step's operands between its MFMAs.
 // The scale multiply-adds of a 32 x 32 tile follow its last MFMA five issue slots later, four after each MFMA, so that
 // neither the matrix pipe nor the vector pipe waits for the other.
+template <bool SILU>
 __global__ __launch_bounds__(512) void gemm_kernel(GemmArgs a)
 {
     constexpr int TN = kGemmTile, RM = kGemmRows, NST = kGemmStages;
@@ -574,7 +588,6 @@ __global__ __launch_bounds__(512) void gemm_kernel(GemmArgs a)
 
     // D[i][j]: i = token within the 32-tile, j = weight row; lane l holds j = l%32 and, in register r,
     // i = 8*(r/4) + 4*(l/32) + r%4
-    float *const out = a.outs[z];
     // the per-token scales of this lane's 32 tokens, fetched before the first store (the stores may alias them for all the
     // compiler knows, and a load behind every store costs the launch 6 us)
     float4 ts[2][4];
@@ -585,6 +598,39 @@ __global__ __launch_bounds__(512) void gemm_kernel(GemmArgs a)
             ts[ti][q] = make_float4(1.f, 1.f, 1.f, 1.f);
             if (a.xscale) ts[ti][q] = *reinterpret_cast<const float4 *>(a.xscale + tt * TN + wm * 64 + ti * 32 + 8 * q + 4 * lhi);   // n_pad entries: in range
         }
+    if constexpr (SILU) {
+        // acc[ti][0] = gate rows, acc[ti][1] = the same up rows: this lane's ff values of row rt * 128 + wn * 32 + l31 and its 32
+        // tokens.  They pass through LDS (per wave: [64 tokens][32 rows] halfs, high and low apart) to come out as 16-byte
+        // chunks of 8 consecutive rows of one token, consecutive lanes taking consecutive tokens: what a chunk row of the
+        // down projection's activation tile is.  Padding tokens give 0 * 0 / 2 = 0, as their rows of the tile must be.
+        constexpr int TS = 80;                      // bytes per token in the exchange: 64 + 16, so that 8 lanes' 16-byte reads miss each other's banks
+        __syncthreads();                            // every wave holds its last operands in registers: the stages are free
+        uint8_t *xb = lds + wave * (2 * 64 * TS);
+#pragma unroll
+        for (int ti = 0; ti < 2; ti++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int tok = ti * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
+                const float4 t4 = ts[ti][r / 4];
+                const float sc = (r % 4) == 0 ? t4.x : (r % 4) == 1 ? t4.y : (r % 4) == 2 ? t4.z : t4.w;
+                const float g = acc[ti][0][r] * sc, u = acc[ti][1][r] * sc;
+                const float f = g * u / (__expf(-u) + 1.f);
+                const uint16_t h = float_to_half_bits(f), l = float_to_half_bits(f - half_bits_to_float(h));
+                *reinterpret_cast<uint16_t *>(xb + tok * TS + l31 * 2) = h;
+                *reinterpret_cast<uint16_t *>(xb + 64 * TS + tok * TS + l31 * 2) = l;
+            }
+        __syncthreads();
+        const uint32_t n = tt * TN + wm * 64 + lane;                  // below n_pad: the token tiles cover the padded batch
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const uint4 hv = *reinterpret_cast<const uint4 *>(xb + lane * TS + c * 16), lv = *reinterpret_cast<const uint4 *>(xb + 64 * TS + lane * TS + c * 16);
+            const size_t o = gemm_x_offset(n, rt * 128 + wn * 32 + c * 8, a.fKp);
+            *reinterpret_cast<uint4 *>(a.fh + o) = hv;
+            *reinterpret_cast<uint4 *>(a.fl + o) = lv;
+        }
+        return;
+    }
+    float *const out = a.outs[z];
 #pragma unroll
     for (int ti = 0; ti < 2; ti++)
 #pragma unroll

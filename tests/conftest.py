@@ -43,6 +43,9 @@ def tiny_models(lva, tmp_path_factory):
         ("tiny_q4", lva.LV_Q4_0, 5, dict(vocab=512, dim=256, heads=4, layers=2, ff=704)),      # head size 64
         ("tiny_q8", lva.LV_Q8_0, 6, dict(vocab=512, dim=256, heads=2, layers=2, ff=704)),      # head size 128
         ("small_q4", lva.LV_Q4_0, 7, dict(vocab=1024, dim=512, heads=16, layers=3, ff=1376)),  # head size 32
+        # feed-forward widths that 128 divides: a prompt batch takes gate and up as one paired GEMM with SwiGLU in its epilogue
+        ("pair_q4", lva.LV_Q4_0, 8, dict(vocab=512, dim=256, heads=2, layers=2, ff=640)),
+        ("pair_q8", lva.LV_Q8_0, 9, dict(vocab=512, dim=512, heads=4, layers=2, ff=768)),
     ]:
         p = str(d / f"{name}.ggml")
         lva.write_model(p, wtype=wtype, seed=seed, **shape)

@@ -90,7 +90,7 @@ def test_gemm_special_inputs(lva, orc, ctx):
     ctx.matrix_free(m)
 
 
-@pytest.mark.parametrize("name,n_prompt", [("tiny_q4", 40), ("tiny_q8", 130), ("small_q4", 77)])
+@pytest.mark.parametrize("name,n_prompt", [("tiny_q4", 40), ("tiny_q8", 130), ("small_q4", 77), ("pair_q4", 150), ("pair_q8", 33)])
 def test_prompt_as_one_batch_matches_oracle(lva, orc, ctx, tiny_models, name, n_prompt):
     path = tiny_models[name]
     om = orc.Model(path)
