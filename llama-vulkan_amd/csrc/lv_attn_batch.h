@@ -31,6 +31,8 @@
 // which walk down the rows at one chunk, spread over the banks.
 #pragma once
 
+#include <type_traits>
+
 #include "lv_gemm.h"
 
 namespace lv {
@@ -172,7 +174,7 @@ __global__ __launch_bounds__(256) void attention_batch_kernel(AttnBatchArgs a)
     constexpr int STAGE = 4 * PLANE;            // kh, kl, v1, v2
     constexpr int NI = PLANE / 1024;            // direct loads (1 KB per wave instruction) per plane
     constexpr int XS = R + 4;                   // row stride of the result exchange in floats
-    static_assert(TQ * XS * 4 <= 2 * STAGE, "the result exchange reuses the tile buffers");
+    static_assert(2 * TQ * XS * 4 <= 2 * STAGE, "the result exchange reuses the tile buffers");
     extern __shared__ __attribute__((aligned(16))) uint8_t attn_lds[];
     __shared__ float den_s[2][2][32];           // [position tile][query tile][query row]
     // the last query tile walks the most cache tiles: it is dispatched first, so the short ones fill the tail
@@ -281,81 +283,82 @@ __global__ __launch_bounds__(256) void attention_batch_kernel(AttnBatchArgs a)
         }
         // register r of sc: position k0 + 32 pt + 8 (r / 4) + 4 hh + r % 4, query n32 of the wave's tile
         // ---- O += P V, sixteen positions (registers 8t .. 8t+7 of both lane halves) at a time --------------------------------
+        // a tile wholly below the diagonal (every query of the wave's 32 sees every position of its 32) needs no masks
+        const bool interior = k0 + 32 * pt + 31 <= pos0 + z0 + 32 * qt && z0 + 32 * qt + 31 < a.n && k0 + 32 * pt + 31 < a.backlog;
+        auto sums = [&](auto masked) {
 #pragma unroll
-        for (int tt = 0; tt < 2; tt++) {
-            uint32_t w1[4], w2[4], w3[4];
+            for (int tt = 0; tt < 2; tt++) {
+                uint32_t w1[4], w2[4], w3[4];
 #pragma unroll
-            for (int e = 0; e < 8; e += 2) {
-                uint32_t b1[2], b2[2], b3[2];
+                for (int e = 0; e < 8; e += 2) {
+                    uint32_t b1[2], b2[2], b3[2];
 #pragma unroll
-                for (int u = 0; u < 2; u++) {
-                    const int r = 8 * tt + e + u;
-                    const uint32_t p = k0 + 32 * pt + 8 * (r / 4) + 4 * hh + (r % 4);
-                    const bool ok = zok && p <= limit && p < a.backlog;
-                    const float e0 = ok ? __expf(sc[r] * scale) : 0.f;
-                    den += e0;
-                    b1[u] = __float_as_uint(e0) & 0xffff0000u;
-                    const float r1 = e0 - __uint_as_float(b1[u]);
-                    b2[u] = __float_as_uint(r1) & 0xffff0000u;
-                    b3[u] = __float_as_uint(r1 - __uint_as_float(b2[u]));   // eight bits at most are left
+                    for (int u = 0; u < 2; u++) {
+                        const int r = 8 * tt + e + u;
+                        float e0 = __expf(sc[r] * scale);
+                        if constexpr (decltype(masked)::value) {
+                            const uint32_t p = k0 + 32 * pt + 8 * (r / 4) + 4 * hh + (r % 4);
+                            const bool ok = zok && p <= limit && p < a.backlog;
+                            e0 = ok ? e0 : 0.f;
+                        }
+                        den += e0;
+                        b1[u] = __float_as_uint(e0) & 0xffff0000u;
+                        const float r1 = e0 - __uint_as_float(b1[u]);
+                        b2[u] = __float_as_uint(r1) & 0xffff0000u;
+                        b3[u] = __float_as_uint(r1 - __uint_as_float(b2[u]));   // eight bits at most are left
+                    }
+                    w1[e / 2] = (b1[0] >> 16) | b1[1];
+                    w2[e / 2] = (b2[0] >> 16) | b2[1];
+                    w3[e / 2] = (b3[0] >> 16) | (b3[1] & 0xffff0000u);
                 }
-                w1[e / 2] = (b1[0] >> 16) | b1[1];
-                w2[e / 2] = (b2[0] >> 16) | b2[1];
-                w3[e / 2] = (b3[0] >> 16) | (b3[1] & 0xffff0000u);
-            }
-            const lv_b8 p1 = __builtin_bit_cast(lv_b8, make_uint4(w1[0], w1[1], w1[2], w1[3]));
-            const lv_b8 p2 = __builtin_bit_cast(lv_b8, make_uint4(w2[0], w2[1], w2[2], w2[3]));
-            const lv_b8 p3 = __builtin_bit_cast(lv_b8, make_uint4(w3[0], w3[1], w3[2], w3[3]));
+                const lv_b8 p1 = __builtin_bit_cast(lv_b8, make_uint4(w1[0], w1[1], w1[2], w1[3]));
+                const lv_b8 p2 = __builtin_bit_cast(lv_b8, make_uint4(w2[0], w2[1], w2[2], w2[3]));
+                const lv_b8 p3 = __builtin_bit_cast(lv_b8, make_uint4(w3[0], w3[1], w3[2], w3[3]));
 #pragma unroll
-            for (int d = 0; d < DT; d++) {
-                const int dim = 32 * d + n32, c = (4 * pt + 2 * tt + hh) ^ (dim & 7);
-                const lv_b8 va = *reinterpret_cast<const lv_b8 *>(vb + dim * 128 + c * 16);
-                const lv_b8 vc = *reinterpret_cast<const lv_b8 *>(vb + PLANE + dim * 128 + c * 16);
-                acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(p3, va, acc[d], 0, 0, 0);
-                acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(p2, vc, acc[d], 0, 0, 0);
-                acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(p2, va, acc[d], 0, 0, 0);
-                acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(p1, vc, acc[d], 0, 0, 0);
-                acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(p1, va, acc[d], 0, 0, 0);
+                for (int d = 0; d < DT; d++) {
+                    const int dim = 32 * d + n32, c = (4 * pt + 2 * tt + hh) ^ (dim & 7);
+                    const lv_b8 va = *reinterpret_cast<const lv_b8 *>(vb + dim * 128 + c * 16);
+                    const lv_b8 vc = *reinterpret_cast<const lv_b8 *>(vb + PLANE + dim * 128 + c * 16);
+                    acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(p3, va, acc[d], 0, 0, 0);
+                    acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(p2, vc, acc[d], 0, 0, 0);
+                    acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(p2, va, acc[d], 0, 0, 0);
+                    acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(p1, vc, acc[d], 0, 0, 0);
+                    acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(p1, va, acc[d], 0, 0, 0);
+                }
             }
-        }
+        };
+        if (interior) sums(std::false_type{});
+        else sums(std::true_type{});
     }
 
     // ---- combine the two position tiles, divide, write -------------------------------------------------------------
-    // acc[d][r]: query row 8 (r / 4) + 4 hh + r % 4 of the wave's tile, dim 32 d + n32
+    // acc[d][r]: query row 8 (r / 4) + 4 hh + r % 4 of the wave's tile, dim 32 d + n32.  Both position tiles leave their sums in
+    // LDS ([position tile][query row of the workgroup][XS]); then a thread takes 8 dims of a row at a time: sum, divide, write.
     den += __shfl_xor(den, 32, kWave);                    // both lane halves: all positions this wave saw, query row n32
+    __syncthreads();                                      // every wave is done with the tile buffers
     if (hh == 0) den_s[pt][qt][n32] = den;
-    __syncthreads();                                      // also: every wave is done with the tile buffers
-    float *xch = reinterpret_cast<float *>(attn_lds);     // [query row of the workgroup][XS]
-    if (pt == 1) {
+    float *xch = reinterpret_cast<float *>(attn_lds) + pt * (TQ * XS);
 #pragma unroll
-        for (int d = 0; d < DT; d++)
+    for (int d = 0; d < DT; d++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) xch[(32 * qt + 8 * (r / 4) + 4 * hh + (r % 4)) * XS + 32 * d + n32] = acc[d][r];
-    }
+        for (int r = 0; r < 16; r++) xch[(32 * qt + 8 * (r / 4) + 4 * hh + (r % 4)) * XS + 32 * d + n32] = acc[d][r];
     __syncthreads();
-    if (pt == 0) {
-#pragma unroll
-        for (int d = 0; d < DT; d++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int i = 8 * (r / 4) + 4 * hh + (r % 4);
-                float *x = &xch[(32 * qt + i) * XS + 32 * d + n32];
-                *x = (acc[d][r] + *x) / (den_s[0][qt][i] + den_s[1][qt][i]);
-            }
-    }
-    __syncthreads();
+    const float *x0p = reinterpret_cast<const float *>(attn_lds), *x1p = x0p + TQ * XS;
     for (int g = t; g < TQ * (R / 8); g += 256) {
         const int row = g / (R / 8), c8 = g % (R / 8);
         const uint32_t z = z0 + row;
-        const float4 x0 = *reinterpret_cast<const float4 *>(&xch[row * XS + c8 * 8]), x1 = *reinterpret_cast<const float4 *>(&xch[row * XS + c8 * 8 + 4]);
         const bool live = z < a.n;
+        const float total = den_s[0][row >> 5][row & 31] + den_s[1][row >> 5][row & 31];
+        const float4 a0 = *reinterpret_cast<const float4 *>(&x0p[row * XS + c8 * 8]), a1 = *reinterpret_cast<const float4 *>(&x0p[row * XS + c8 * 8 + 4]);
+        const float4 b0 = *reinterpret_cast<const float4 *>(&x1p[row * XS + c8 * 8]), b1 = *reinterpret_cast<const float4 *>(&x1p[row * XS + c8 * 8 + 4]);
+        float f[8] = {(a0.x + b0.x) / total, (a0.y + b0.y) / total, (a0.z + b0.z) / total, (a0.w + b0.w) / total,
+                      (a1.x + b1.x) / total, (a1.y + b1.y) / total, (a1.z + b1.z) / total, (a1.w + b1.w) / total};
         if (a.out && live) {
             float *o = a.out + (size_t)z * D + (size_t)h * R + c8 * 8;
-            *reinterpret_cast<float4 *>(o) = x0;
-            *reinterpret_cast<float4 *>(o + 4) = x1;
+            *reinterpret_cast<float4 *>(o) = make_float4(f[0], f[1], f[2], f[3]);
+            *reinterpret_cast<float4 *>(o + 4) = make_float4(f[4], f[5], f[6], f[7]);
         }
         if (a.xh) {
-            float f[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
             if (!live) {
 #pragma unroll
                 for (int e = 0; e < 8; e++) f[e] = 0.f;

@@ -353,27 +353,40 @@ __global__ __launch_bounds__(256) void prefill_norm_kernel(PrefillNormArgs a)
     const bool live = row < a.n;
     const size_t ro = (size_t)(live ? row : 0) * dim;
     float v[PER][8], wv[PER][8];
+    // every load of the row first (x, up to four slices, the weights: nothing depends on anything), then the sums and the
+    // stores: a store between them would hold back the loads behind it, which may alias it for all the compiler knows
+    float4 x4[PER][2], p4[kGemmMaxMats][PER][2];
 #pragma unroll
     for (int j = 0; j < PER; j++) {
         const uint32_t i = threadIdx.x + j * 256;
-        const bool ok = live && i < n8;
-        const uint32_t ic = ok ? i : 0;
+        const uint32_t ic = (live && i < n8) ? i : 0;
 #pragma unroll
         for (int hf = 0; hf < 2; hf++) {
             const float4 w4 = reinterpret_cast<const float4 *>(a.w)[(i < n8 ? i : 0) * 2 + hf];
             wv[j][4 * hf] = w4.x; wv[j][4 * hf + 1] = w4.y; wv[j][4 * hf + 2] = w4.z; wv[j][4 * hf + 3] = w4.w;
-            float4 x4 = reinterpret_cast<const float4 *>(a.x + ro)[ic * 2 + hf];
+            x4[j][hf] = reinterpret_cast<const float4 *>(a.x + ro)[ic * 2 + hf];
+#pragma unroll
+            for (int q = 0; q < kGemmMaxMats; q++)
+                if (q < (int)a.nparts) p4[q][j][hf] = reinterpret_cast<const float4 *>(a.parts[q] + ro)[ic * 2 + hf];
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+        const uint32_t i = threadIdx.x + j * 256;
+        const bool ok = live && i < n8;
+#pragma unroll
+        for (int hf = 0; hf < 2; hf++) {
+            float4 x = x4[j][hf];
             if (a.nparts) {
-                float4 s4 = reinterpret_cast<const float4 *>(a.parts[0] + ro)[ic * 2 + hf];
-                for (uint32_t q = 1; q < a.nparts; q++) {
-                    const float4 p4 = reinterpret_cast<const float4 *>(a.parts[q] + ro)[ic * 2 + hf];
-                    s4.x += p4.x; s4.y += p4.y; s4.z += p4.z; s4.w += p4.w;
-                }
-                x4.x = s4.x + x4.x; x4.y = s4.y + x4.y; x4.z = s4.z + x4.z; x4.w = s4.w + x4.w;
-                if (ok) reinterpret_cast<float4 *>(a.x + ro)[ic * 2 + hf] = x4;
+                float4 s4 = p4[0][j][hf];
+#pragma unroll
+                for (int q = 1; q < kGemmMaxMats; q++)
+                    if (q < (int)a.nparts) { s4.x += p4[q][j][hf].x; s4.y += p4[q][j][hf].y; s4.z += p4[q][j][hf].z; s4.w += p4[q][j][hf].w; }
+                x.x = s4.x + x.x; x.y = s4.y + x.y; x.z = s4.z + x.z; x.w = s4.w + x.w;
+                if (ok) reinterpret_cast<float4 *>(a.x + ro)[i * 2 + hf] = x;
             }
-            if (!ok) x4 = make_float4(0.f, 0.f, 0.f, 0.f);
-            v[j][4 * hf] = x4.x; v[j][4 * hf + 1] = x4.y; v[j][4 * hf + 2] = x4.z; v[j][4 * hf + 3] = x4.w;
+            if (!ok) x = make_float4(0.f, 0.f, 0.f, 0.f);
+            v[j][4 * hf] = x.x; v[j][4 * hf + 1] = x.y; v[j][4 * hf + 2] = x.z; v[j][4 * hf + 3] = x.w;
         }
     }
     float s = 0.f;
