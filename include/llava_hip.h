@@ -192,12 +192,15 @@ int lv_kernel_normalize(lv_ctx *ctx, float *out, const float *x, const float *w,
 int lv_kernel_kv_append(lv_ctx *ctx, void *cache, const float *in, uint32_t pos, uint32_t dim, uint32_t batch,
                         uint32_t backlog);
 /* mhsa + softmax + kqv_matching fused (mhsa.comp:32-60, softmax.comp:26-44, kqv_matching.comp:27-42):
- * out[z][dim] = sum_{p <= pos+z} softmax_p( Q_z . Rot(-(pos+z-p) theta) K_p / sqrt(rot) ) V_p  per head */
+ * out[z][dim] = sum_{p <= pos+z} softmax_p( Q_z . Rot(-(pos+z-p) theta) K_p / sqrt(rot) ) V_p  per head.
+ * Up to 15 rows go through the one-query kernel of the decode path, 16 and more through the kernels of a prompt batch
+ * (matrix cores on exact 16-bit pieces of the fp32 operands); the two agree to about 1e-6 of the largest output. */
 int lv_kernel_attention(lv_ctx *ctx, float *out, const void *kcache, const void *vcache, const float *q,
                         uint32_t pos, uint32_t backlog, uint32_t heads, uint32_t rot, uint32_t batch);
 
 /* lv_kernel_attention for callers that cannot allocate device memory (code under HIP graph capture, serving loops and
- * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments, same result; the rotation
+ * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments, same result (the one-query
+ * kernel at every batch size); the rotation
  * table, the partial sums and the split counters live in a fixed 2 MiB work area that every device holds from library
  * load to process end, so the call allocates nothing and frees nothing.  Limits (LV_ERR_RANGE beyond them):
  * backlog * rot / 2 <= 131072, batch * heads * ceil(backlog / 64) * (rot + 1) <= 262144, batch * heads <= 256.
