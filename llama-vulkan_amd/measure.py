@@ -209,6 +209,109 @@ def prefill_case(ctx, case, name, wtype, report=emit):
     return r
 
 
+def board_power_watts():
+    """the board's power sensor (amdgpu hwmon, microwatts), or None where the driver does not show one"""
+    import glob
+    for f in glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input") + glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_average"):
+        try:
+            return int(open(f).read()) / 1e6
+        except (OSError, ValueError):
+            pass
+    return None
+
+
+def board_power_cap_watts():
+    import glob
+    for f in glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_cap"):
+        try:
+            return int(open(f).read()) / 1e6
+        except (OSError, ValueError):
+            pass
+    return None
+
+
+def prefill_power_case(ctx, case, name, wtype, seconds=4.0, report=emit):
+    """The 512-token prompt step repeated for `seconds` while a thread reads the board's power sensor every 10 ms:
+    the time per step and the sensor's readings from the idle board, over the run, and in its second half."""
+    import threading
+    import time
+    shape = SHAPES[name]
+    model = lva.Model(ctx, model_file(name, wtype, 3))
+    s = lva.Session(model, 512)
+    prompt = lva.synth_tokens(512, 3, shape["vocab"], seed=3)
+    idle = board_power_watts()
+    s.begin(prompt, 0)
+    s.wait()
+    samples, stop = [], threading.Event()
+
+    def sampler():
+        while not stop.is_set():
+            samples.append((time.monotonic(), board_power_watts()))
+            time.sleep(0.01)
+    th = threading.Thread(target=sampler)
+    th.start()
+    t0 = time.monotonic()
+    times = []
+    while time.monotonic() - t0 < seconds:
+        s.timer_start()
+        s.begin(prompt, 0)
+        times.append(s.timer_stop())
+    t1 = time.monotonic()
+    stop.set()
+    th.join()
+    w = [p for t, p in samples if p is not None and t0 <= t <= t1]
+    late = [p for t, p in samples if p is not None and (t0 + t1) / 2 <= t <= t1]
+    half = len(times) // 2
+    r = report(case=case, model=name, wtype="q4_0" if wtype == lva.LV_Q4_0 else "q8_0", tokens=512, steps=len(times),
+               ms_first=round(times[0], 2), ms_mean_first_half=round(sum(times[:half]) / max(1, half), 2),
+               ms_mean_second_half=round(sum(times[half:]) / max(1, len(times) - half), 2),
+               power_cap_W=board_power_cap_watts(), idle_W=idle, samples=len(w),
+               power_mean_W=round(sum(w) / len(w), 1) if w else None, power_max_W=max(w) if w else None,
+               power_mean_second_half_W=round(sum(late) / len(late), 1) if late else None)
+    s.close()
+    model.close()
+    return r
+
+
+def decode_power_case(ctx, case, seconds=3.0, report=emit):
+    """Greedy decode of the 7B q4_0 model at positions 448..511, the window repeated for `seconds`, with the board's power
+    sensor read every 10 ms: is the decode kernel anywhere near the board's power cap?"""
+    import threading
+    import time
+    shape = SHAPES["7b"]
+    model = lva.Model(ctx, model_file("7b", lva.LV_Q4_0, 0))
+    s = lva.Session(model, 512)
+    s.begin(lva.synth_tokens(440, 3, shape["vocab"], seed=0), 0)
+    tok = s.argmax()
+    for pos in range(440, 448):
+        s.begin([tok], pos)
+        tok = s.argmax()
+    samples, stop = [], threading.Event()
+
+    def sampler():
+        while not stop.is_set():
+            samples.append(board_power_watts())
+            time.sleep(0.01)
+    th = threading.Thread(target=sampler)
+    th.start()
+    t0 = time.monotonic()
+    steps = 0
+    while time.monotonic() - t0 < seconds:
+        for pos in range(448, 512):      # the same cache rows rewritten: a decode step's work does not depend on the token
+            s.begin([tok], pos)
+            tok = s.argmax()
+        steps += 64
+    dt = time.monotonic() - t0
+    stop.set()
+    th.join()
+    w = [p for p in samples if p is not None]
+    r = report(case=case, steps=steps, tok_s=round(steps / dt, 1), power_cap_W=board_power_cap_watts(), samples=len(w),
+               power_mean_W=round(sum(w) / len(w), 1) if w else None, power_max_W=max(w) if w else None)
+    s.close()
+    model.close()
+    return r
+
+
 def handover_case(name, wtype, seed, backlog, last):
     """Loads the timing build of the library (libllava_hip_timing.so, -DLV_MEGA_TIMING: workgroup 0 of the persistent kernel
     writes the 100 MHz wall clock at every phase boundary of layers 0..3) and prints, for the decode step at position
@@ -326,6 +429,10 @@ def main():
         decode_case(ctx, "decode-7b-graph", "7b", lva.LV_Q4_0, 0, 512, 440, 68, force_path=lva.PATH_GRAPH)
     if which in ("prefill-13b", "all"):
         prefill_case(ctx, "prefill-13b", "13b", lva.LV_Q8_0)
+    if which == "decode-7b-power":
+        decode_power_case(ctx, "decode-7b-power")
+    if which == "prefill-13b-power":
+        prefill_power_case(ctx, "prefill-13b-power", "13b", lva.LV_Q8_0)
     if which in ("prefill-13b-q4", "all"):
         prefill_case(ctx, "prefill-13b-q4", "13b", lva.LV_Q4_0)
     if which in ("prefill-7b", "all"):
