@@ -160,3 +160,43 @@ def test_second_batch_appends_behind_the_first(lva, orc, ctx, tiny_models):
     assert np.all(np.abs(got - want) <= 1e-2 + 1e-3 * np.abs(want))
     assert s.argmax() == orc.greedy(want)
     s.close(); model.close(); osess.close(); om.close()
+
+
+def test_prompt_batch_of_a_width_that_64_does_not_divide(lva, orc, ctx, tmp_path):
+    """dim 96 = 3 heads of 32: the GEMM pads K to 128, so the attention result goes through the split kernel (which writes
+    the zero columns) instead of being written as halves by the attention kernel; ff 160 cannot be paired either"""
+    path = str(tmp_path / "odd.ggml")
+    lva.write_model(path, wtype=lva.LV_Q8_0, seed=23, vocab=320, layers=2, dim=96, heads=3, ff=160)
+    om = orc.Model(path)
+    osess = orc.Session(om, 64)
+    model = lva.Model(ctx, path)
+    s = lva.Session(model, 64)
+    prompt = lva.synth_tokens(40, 3, 320, seed=24)
+    want = osess.eval(prompt)
+    s.begin(prompt, 0)
+    got = s.logits()
+    assert np.all(np.abs(got - want) <= 1e-2 + 1e-3 * np.abs(want)), float(np.max(np.abs(got - want)))
+    assert s.argmax() == orc.greedy(want)
+    s.close(); model.close(); osess.close(); om.close()
+
+
+def test_prompt_batch_in_a_cache_whose_length_64_does_not_divide(lva, ctx, tiny_models):
+    """a backlog of 100 rows: the attention planes are padded to 128 rows, the cache is not; the batch must agree with the
+    same tokens evaluated one by one (the oracle's tree sums want a power-of-two backlog, so it cannot referee here)"""
+    model = lva.Model(ctx, tiny_models["pair_q8"])
+    a, b = lva.Session(model, 100), lva.Session(model, 100)
+    prompt = lva.synth_tokens(90, 3, 512, seed=25)
+    a.begin(prompt[:50], 0)
+    a.wait()
+    a.begin(prompt[50:], 50)
+    for i, t in enumerate(prompt):
+        b.begin([int(t)], i)
+        b.wait()
+    la, lb = a.logits(), b.logits()
+    assert float(np.max(np.abs(la - lb))) <= 1e-4 * max(1.0, float(np.max(np.abs(lb))))
+    for layer in range(2):
+        for which in (0, 1):
+            ra = a.kv(layer, which, 90).view(np.float16).astype(np.float32)
+            rb = b.kv(layer, which, 90).view(np.float16).astype(np.float32)
+            assert np.max(np.abs(ra - rb)) <= 2e-3 * float(np.max(np.abs(rb)))
+    a.close(); b.close(); model.close()
