@@ -259,7 +259,9 @@ __global__ __launch_bounds__(256) void attention_batch_kernel(AttnBatchArgs a)
 
     for (uint32_t it = 0; it < steps; it++) {
         const uint32_t k0 = it * TK;
-        __syncthreads();      // this tile's loads have landed (the barrier waits for the loads in flight); the other buffer is consumed
+        // this wave's direct loads of the tile have landed; behind the barrier everyone's have, and the other buffer is consumed
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
         if (it + 1 < steps) issue((it + 1) & 1, k0 + TK);
         if (k0 + 32 * pt > wave_last) continue;       // every pair of this wave's 32 x 32 tile is masked
         const uint8_t *kb = attn_lds + (it & 1) * STAGE, *vb = kb + 2 * PLANE;
