@@ -812,6 +812,26 @@ static int dispatch_gemm(hipStream_t st, GemmArgs a, const lv_matrix &w, uint32_
     return LV_OK;
 }
 
+// q, k and v of a prompt batch (three matrices of one shape) as one launch: q as fp32 rows of `q`, k and v rounded to fp16
+// straight into rows *row_ptr + row_add .. of their caches (rows of `dim` halfs, `backlog` of them)
+static int launch_gemm_qkv(hipStream_t st, float *q, uint16_t *kcache, uint16_t *vcache, const lv_matrix &wq, const lv_matrix &wk, const lv_matrix &wv,
+                           uint32_t n, const uint16_t *xh, const uint16_t *xl, const float *xscale, const uint32_t *row_ptr, uint32_t row_add,
+                           uint32_t backlog)
+{
+    GemmArgs a{};
+    a.xh = xh; a.xl = xl; a.n = n; a.xscale = xscale; a.rows = wq.view.rows; a.K = wq.view.cols; a.nz = 3; a.ldo = wq.view.rows;
+    a.outs[0] = q; a.w16[0] = wq.h16; a.w16[1] = wk.h16; a.w16[2] = wv.h16;
+    a.half_out[1] = kcache; a.half_out[2] = vcache; a.row_ptr = row_ptr; a.row_add = row_add; a.row_limit = backlog;
+    for (int i = 0; i < 3; i++)
+        if (!a.w16[i]) return fail(LV_ERR_STATE, "gemm: the matrix has no prompt copy");
+    HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_rows16_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLdsBytes));
+    const uint32_t token_tiles = (n + kGemmTile - 1) / kGemmTile, row_tiles = (a.rows + kGemmRows - 1) / kGemmRows;
+    const dim3 grid((row_tiles * 3 + 7) / 8 * 8 * token_tiles);
+    gemm_rows16_kernel<<<grid, dim3(512), kGemmLdsBytes, st>>>(a);
+    HIP_TRY(hipGetLastError());
+    return LV_OK;
+}
+
 // fh, fl (tile order, n_pad x gemm_k_padded(F)) = the halves of SwiGLU(x W3^T, x W1^T) for the pair copy `pair16` of two F x K matrices
 static int launch_gemm_silu(hipStream_t st, uint16_t *fh, uint16_t *fl, const uint16_t *pair16, uint32_t F, uint32_t K, uint32_t n,
                             const uint16_t *xh, const uint16_t *xl, const float *xscale)
@@ -1770,7 +1790,11 @@ static int record_prefill(lv_session *s, uint32_t idx0, uint32_t n, bool with_he
         const float *xscale = nullptr;
         LV_TRY(launch_prefill_norm(st, s, lw.attn_norm, n, D, parts, pending, !qkv_same, &xscale));
         pending = 0;
-        if (qkv_same) {
+        const bool kv_in_cache = qkv_same && lw.wq.view.rows == D;     // the GEMM's epilogue is the cache append of the batch
+        if (kv_in_cache) {
+            LV_TRY(launch_gemm_qkv(st, s->pf_q, kv_ptr(s, li, 0), kv_ptr(s, li, 1), lw.wq, lw.wk, lw.wv, n, s->pf_xh, s->pf_xl, xscale, pos_ptr, idx0,
+                                   s->backlog));
+        } else if (qkv_same) {
             float *const outs[3] = {s->pf_q, s->pf_k, s->pf_v};
             const lv_matrix *const ws[3] = {&lw.wq, &lw.wk, &lw.wv};
             LV_TRY(launch_gemm_multi(st, outs, D, ws, 3, n, s->pf_xh, s->pf_xl, false, xscale));
@@ -1779,12 +1803,13 @@ static int record_prefill(lv_session *s, uint32_t idx0, uint32_t n, bool with_he
             LV_TRY(launch_gemm_presplit(st, s->pf_k, D, lw.wk, n, s->pf_xh, s->pf_xl, false, xscale));
             LV_TRY(launch_gemm_presplit(st, s->pf_v, D, lw.wv, n, s->pf_xh, s->pf_xl, false, xscale));
         }
-        // the batch's K and V rows go to the cache in the first of the attention kernels
+        // the batch's K and V rows are in the cache already, or go there in the first of the attention kernels
+        const float *kin = kv_in_cache ? nullptr : s->pf_k, *vin = kv_in_cache ? nullptr : s->pf_v;
         if (D % kGemmK == 0) {     // the attention kernel writes the halves the output projection reads
-            LV_TRY(launch_attention_batch(st, nullptr, s->pf_xh, s->pf_xl, D, s->pf_planes, kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->pf_k, s->pf_v, s->pf_q, s->trig_abs,
+            LV_TRY(launch_attention_batch(st, nullptr, s->pf_xh, s->pf_xl, D, s->pf_planes, kv_ptr(s, li, 0), kv_ptr(s, li, 1), kin, vin, s->pf_q, s->trig_abs,
                                           pos_ptr, idx0, n, s->backlog, hp.heads, hp.rot));
         } else {                   // a padded K: the split kernel writes the zero columns as well
-            LV_TRY(launch_attention_batch(st, s->pf_vo, nullptr, nullptr, 0, s->pf_planes, kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->pf_k, s->pf_v, s->pf_q, s->trig_abs,
+            LV_TRY(launch_attention_batch(st, s->pf_vo, nullptr, nullptr, 0, s->pf_planes, kv_ptr(s, li, 0), kv_ptr(s, li, 1), kin, vin, s->pf_q, s->trig_abs,
                                           pos_ptr, idx0, n, s->backlog, hp.heads, hp.rot));
             LV_TRY(launch_split(st, s->pf_xh, s->pf_xl, nullptr, s->pf_vo, n, D));
         }

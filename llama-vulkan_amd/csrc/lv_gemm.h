@@ -244,6 +244,12 @@ struct GemmArgs {
     // down projection's GEMM reads: tile order, n_pad x fKp
     uint16_t *fh, *fl;
     uint32_t fKp;
+    // gemm_rows16_kernel only: for a matrix z with half_out[z] set the result is stored as fp16 (round to nearest even, what
+    // copy_to_cache.comp:29-37 does to K and V) at half_out[z][(*row_ptr + row_add + token) * ldo + m], rows below row_limit:
+    // the k and v products of a prompt batch go straight into their cache rows
+    uint16_t *half_out[kGemmMaxMats];
+    const uint32_t *row_ptr;
+    uint32_t row_add, row_limit;
 };
 
 // out[n][ldo] (+)= p[0] + p[1] (+ p[2] + p[3]), the K slices of one product, each [n][rows]; always summed in this order
@@ -456,9 +462,11 @@ __device__ unsigned long long gemm_clock_words[3];
 // of stage s (which every wave has by then read into registers), and reads the next step's operands between its MFMAs.
 // The scale multiply-adds of a 32 x 32 tile follow its last MFMA five issue slots later, four after each MFMA, so that
 // neither the matrix pipe nor the vector pipe waits for the other.
-template <bool SILU>
-__global__ __launch_bounds__(512) void gemm_kernel(GemmArgs a)
+// MODE 0: plain products; 1: SwiGLU of a pair copy (GemmArgs::fh); 2: plain, or fp16 rows where GemmArgs::half_out says so
+template <int MODE>
+__device__ __forceinline__ void gemm_body(const GemmArgs &a)
 {
+    constexpr bool SILU = MODE == 1;
     constexpr int TN = kGemmTile, RM = kGemmRows, NST = kGemmStages;
     constexpr int LPS = 5;   // direct loads per thread per stage
     extern __shared__ __attribute__((aligned(16))) uint8_t gemm_lds[];
@@ -643,6 +651,37 @@ __global__ __launch_bounds__(512) void gemm_kernel(GemmArgs a)
         }
         return;
     }
+    if constexpr (MODE == 2) {
+        if (a.half_out[z]) {
+            // the wave's 64 tokens x 64 rows pass through LDS as halfs ([token][row], 128 + 16 bytes a token) and leave as 16-byte
+            // chunks of 8 consecutive rows, eight lanes on the 128 bytes of a token
+            constexpr int TS = 144;
+            __syncthreads();                            // every wave holds its last operands in registers: the stages are free
+            uint8_t *xb = lds + wave * (64 * TS);
+#pragma unroll
+            for (int ti = 0; ti < 2; ti++)
+#pragma unroll
+                for (int tj = 0; tj < 2; tj++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int tok = ti * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
+                        const float4 t4 = ts[ti][r / 4];
+                        const float sc = (r % 4) == 0 ? t4.x : (r % 4) == 1 ? t4.y : (r % 4) == 2 ? t4.z : t4.w;
+                        *reinterpret_cast<uint16_t *>(xb + tok * TS + (tj * 32 + l31) * 2) = float_to_half_bits(acc[ti][tj][r] * sc);
+                    }
+            __syncthreads();
+            const uint32_t row0 = (a.row_ptr ? *a.row_ptr : 0u) + a.row_add;
+            uint16_t *const dst = a.half_out[z];
+#pragma unroll
+            for (int it = 0; it < 8; it++) {
+                const int tok = it * 8 + (lane >> 3), c = lane & 7;
+                const uint32_t n = tt * TN + wm * 64 + tok, m = rt * RM + wn * 64 + c * 8;
+                const uint4 v = *reinterpret_cast<const uint4 *>(xb + tok * TS + c * 16);
+                if (n < a.n && m < a.rows && row0 + n < a.row_limit) *reinterpret_cast<uint4 *>(dst + (size_t)(row0 + n) * a.ldo + m) = v;
+            }
+            return;
+        }
+    }
     float *const out = a.outs[z];
 #pragma unroll
     for (int ti = 0; ti < 2; ti++)
@@ -661,6 +700,18 @@ __global__ __launch_bounds__(512) void gemm_kernel(GemmArgs a)
                 }
             }
         }
+}
+
+template <bool SILU>
+__global__ __launch_bounds__(512) void gemm_kernel(GemmArgs a)
+{
+    gemm_body<SILU ? 1 : 0>(a);
+}
+
+// q, k and v of a prompt batch in one launch: q as fp32 rows, k and v as fp16 rows of their caches (GemmArgs::half_out)
+__global__ __launch_bounds__(512) void gemm_rows16_kernel(GemmArgs a)
+{
+    gemm_body<2>(a);
 }
 
 }  // namespace lv
