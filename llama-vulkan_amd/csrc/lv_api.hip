@@ -832,17 +832,38 @@ static int launch_gemm_qkv(hipStream_t st, float *q, uint16_t *kcache, uint16_t 
     return LV_OK;
 }
 
-// fh, fl (tile order, n_pad x gemm_k_padded(F)) = the halves of SwiGLU(x W3^T, x W1^T) for the pair copy `pair16` of two F x K matrices
+// fh, fl (tile order, n_pad x gemm_k_padded(F)) = the halves of SwiGLU(x W3^T, x W1^T) for the pair copy `pair16` of two F x K matrices.
+// Rounds.  A round holds 32 workgroups per XCD, i.e. cap = (32 / token tiles) * 8 row tiles.  When the last round would be
+// less than half full (7B at 512 tokens: 86 row tiles, 64 a round, 22 left) its row tiles are cut in two along K instead
+// and run as ONE round of half the length: raw products of both halves into g1 / g2 (scratch, n_pad x F floats each), summed
+// and passed through SwiGLU by silu_pair_tail_kernel.
 static int launch_gemm_silu(hipStream_t st, uint16_t *fh, uint16_t *fl, const uint16_t *pair16, uint32_t F, uint32_t K, uint32_t n,
-                            const uint16_t *xh, const uint16_t *xl, const float *xscale)
+                            const uint16_t *xh, const uint16_t *xl, const float *xscale, float *g1, float *g2)
 {
+    const uint32_t token_tiles = (n + kGemmTile - 1) / kGemmTile, tiles = 2 * F / kGemmRows, k_steps = gemm_k_padded(K) / kGemmK;
+    const uint32_t cap = token_tiles <= 32 ? (32 / token_tiles) * 8 : 0;
+    uint32_t tail = cap ? tiles % cap : 0;
+    if (tiles < cap + tail || tail * 2 > cap || k_steps < 32 || k_steps % 2 || !g1 || !g2) tail = 0;
+    const uint32_t head = tiles - tail;
     GemmArgs a{};
     a.xh = xh; a.xl = xl; a.n = n; a.xscale = xscale; a.w16[0] = pair16; a.rows = 2 * F; a.K = K; a.nz = 1;
     a.fh = fh; a.fl = fl; a.fKp = gemm_k_padded(F);
+    a.tile0 = 0; a.tile_count = head;
     HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLdsBytes));
-    const uint32_t token_tiles = (n + kGemmTile - 1) / kGemmTile, row_tiles = a.rows / kGemmRows;
-    const dim3 grid((row_tiles + 7) / 8 * 8 * token_tiles);
-    gemm_kernel<true><<<grid, dim3(512), kGemmLdsBytes, st>>>(a);
+    gemm_kernel<true><<<dim3((head + 7) / 8 * 8 * token_tiles), dim3(512), kGemmLdsBytes, st>>>(a);
+    HIP_TRY(hipGetLastError());
+    if (!tail) return LV_OK;
+    GemmArgs b{};
+    b.xh = xh; b.xl = xl; b.n = n; b.xscale = xscale; b.rows = 2 * F; b.K = K; b.nz = 2;
+    b.w16[0] = b.w16[1] = pair16; b.outs[0] = g1; b.outs[1] = g2; b.ldo = tail * kGemmRows;
+    b.slice_k = k_steps / 2 * kGemmK; b.tile0 = head; b.tile_count = tail;
+    HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_kernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLdsBytes));
+    gemm_kernel<false><<<dim3((tail * 2 + 7) / 8 * 8 * token_tiles), dim3(512), kGemmLdsBytes, st>>>(b);
+    HIP_TRY(hipGetLastError());
+    SiluTailArgs t{};
+    t.fh = fh; t.fl = fl; t.parts[0] = g1; t.parts[1] = g2; t.nparts = 2; t.n = n; t.F = F; t.Fp = gemm_k_padded(F); t.f0 = head * (kGemmRows / 2);
+    t.tail_rows = tail * kGemmRows;
+    silu_pair_tail_kernel<<<dim3((F - t.f0) / 64, token_tiles * kGemmTile / 32), dim3(256), 0, st>>>(t);
     HIP_TRY(hipGetLastError());
     return LV_OK;
 }
@@ -1818,7 +1839,7 @@ static int record_prefill(lv_session *s, uint32_t idx0, uint32_t n, bool with_he
         pending = 0;
         const uint16_t *fh = s->pf_xh, *fl = s->pf_xl;     // where the down projection finds its activations
         if (lw.gate_up16) {        // SwiGLU in the GEMM's epilogue
-            LV_TRY(launch_gemm_silu(st, s->pf_fh, s->pf_fl, lw.gate_up16, F, D, n, s->pf_xh, s->pf_xl, xscale));
+            LV_TRY(launch_gemm_silu(st, s->pf_fh, s->pf_fl, lw.gate_up16, F, D, n, s->pf_xh, s->pf_xl, xscale, s->pf_g1, s->pf_g2));
             fh = s->pf_fh; fl = s->pf_fl;
         } else if (gate_same) {
             float *const outs[2] = {s->pf_g1, s->pf_g2};

@@ -224,6 +224,43 @@ __global__ __launch_bounds__(256) void silu_split_kernel(uint16_t *__restrict__ 
 }
 
 constexpr int kGemmMaxMats = 4;
+
+// SwiGLU for the feed-forward rows f0 .. F-1 whose gate and up products come from a K-sliced launch over the last row tiles
+// of a pair copy (expand_codes_kernel<.., true>): parts[s][token][tail_rows] hold slice s in the pair copy's row order
+// (32 gate rows, then the same 32 up rows), summed slice 0 first.  Output as silu_split_kernel's, at columns f0 .. of the
+// activation tile.  f0 and F are multiples of 128.  grid ((F - f0) / 64, n_pad / 32), 256 threads.
+struct SiluTailArgs {
+    uint16_t *fh, *fl;
+    const float *parts[kGemmMaxMats];
+    uint32_t nparts, n, F, Fp, f0, tail_rows;
+};
+__global__ __launch_bounds__(256) void silu_pair_tail_kernel(SiluTailArgs a)
+{
+    uint32_t token, k;
+    gemm_producer_coords(token, k);                 // k counts from f0
+    const uint32_t f = a.f0 + k;
+    if (f >= a.F) return;
+    float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (token < a.n) {
+        const uint32_t prow = k / 128 * 256 + (k % 128) / 32 * 64 + k % 32;     // the chunk's 8 gate rows; their up rows follow 32 further on
+        float g[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, u[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        for (uint32_t s = 0; s < a.nparts; s++) {
+            const float *p = a.parts[s] + (size_t)token * a.tail_rows + prow;
+            const float4 g0 = *reinterpret_cast<const float4 *>(p), g1 = *reinterpret_cast<const float4 *>(p + 4);
+            const float4 u0 = *reinterpret_cast<const float4 *>(p + 32), u1 = *reinterpret_cast<const float4 *>(p + 36);
+            g[0] += g0.x; g[1] += g0.y; g[2] += g0.z; g[3] += g0.w; g[4] += g1.x; g[5] += g1.y; g[6] += g1.z; g[7] += g1.w;
+            u[0] += u0.x; u[1] += u0.y; u[2] += u0.z; u[3] += u0.w; u[4] += u1.x; u[5] += u1.y; u[6] += u1.z; u[7] += u1.w;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) v[j] = g[j] * u[j] / (__expf(-u[j]) + 1.f);
+    }
+    uint4 h, l;
+    gemm_split8(h, l, v);
+    const size_t o = gemm_x_offset(token, f, a.Fp);
+    *reinterpret_cast<uint4 *>(a.fh + o) = h;
+    *reinterpret_cast<uint4 *>(a.fl + o) = l;
+}
+
 struct GemmArgs {
     // up to four matrices of one shape applied to the same activations in one launch: q, k and v of a layer together fill the CUs that each alone leaves idle
     float *outs[kGemmMaxMats];          // [n][ldo] each
@@ -250,6 +287,9 @@ struct GemmArgs {
     uint16_t *half_out[kGemmMaxMats];
     const uint32_t *row_ptr;
     uint32_t row_add, row_limit;
+    // a launch over part of the row tiles: tile_count of them (0: all) from tile0 on; fp32 results then go to column
+    // m - tile0 * 256 of their output rows
+    uint32_t tile0, tile_count;
 };
 
 // out[n][ldo] (+)= p[0] + p[1] (+ p[2] + p[3]), the K slices of one product, each [n][rows]; always summed in this order
@@ -474,12 +514,12 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a)
     const int tid = threadIdx.x, lane = tid & 63, l31 = lane & 31, lhi = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wn = wave & 3, wm = wave >> 2;
-    const uint32_t tok_tiles = (a.n + TN - 1) / TN, row_tiles = (a.rows + RM - 1) / RM;
+    const uint32_t tok_tiles = (a.n + TN - 1) / TN, row_tiles = a.tile_count ? a.tile_count : (a.rows + RM - 1) / RM;
     // unit = (matrix or slice, row tile); unit u runs on XCD u % 8, its token tiles in consecutive slots of that XCD
     const uint32_t L = blockIdx.x, xcd = L & 7, slot = L >> 3;
     const uint32_t unit = (slot / tok_tiles) * 8 + xcd, tt = slot % tok_tiles;
     if (unit >= row_tiles * a.nz) return;
-    const uint32_t z = unit / row_tiles, rt = unit % row_tiles;
+    const uint32_t z = unit / row_tiles, rt = unit % row_tiles + a.tile0;
     const uint32_t Kp = gemm_k_padded(a.K), nchunk = Kp / 8, nblk = Kp / 32;
     // this workgroup's K steps: step0 .. step0 + steps - 1, an even number (slices are multiples of 64, and so is Kp)
     const uint32_t step0 = a.slice_k ? z * (a.slice_k / kGemmStep) : 0;
@@ -694,7 +734,7 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a)
                 const float4 t4 = ts[ti][r / 4];
                 const float sc = (r % 4) == 0 ? t4.x : (r % 4) == 1 ? t4.y : (r % 4) == 2 ? t4.z : t4.w;
                 if (n < a.n && m < a.rows) {
-                    float *dst = out + (size_t)n * a.ldo + m;
+                    float *dst = out + (size_t)n * a.ldo + (m - a.tile0 * RM);
                     const float v = acc[ti][tj][r] * sc;
                     *dst = a.accumulate ? *dst + v : v;
                 }

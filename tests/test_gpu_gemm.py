@@ -200,3 +200,26 @@ def test_prompt_batch_in_a_cache_whose_length_64_does_not_divide(lva, ctx, tiny_
             rb = b.kv(layer, which, 90).view(np.float16).astype(np.float32)
             assert np.max(np.abs(ra - rb)) <= 2e-3 * float(np.max(np.abs(rb)))
     a.close(); b.close(); model.close()
+
+
+def test_prompt_batch_whose_last_round_of_gate_up_tiles_is_cut_along_k(lva, orc, ctx, tmp_path):
+    """ff 8448 = 66 row tiles of the paired gate/up copy at 4 token tiles: 64 fill a round, the last 2 are multiplied in two K
+    halves by a second launch and pass through SwiGLU in a kernel of their own; dim 2048 gives the 32 K steps that needs"""
+    path = str(tmp_path / "tail.ggml")
+    lva.write_model(path, wtype=lva.LV_Q4_0, seed=31, vocab=320, layers=1, dim=2048, heads=16, ff=8448)
+    om = orc.Model(path)
+    osess = orc.Session(om, 512)
+    model = lva.Model(ctx, path)
+    a, b = lva.Session(model, 512), lva.Session(model, 512)
+    prompt = lva.synth_tokens(390, 3, 320, seed=32)
+    want = osess.eval(prompt)
+    a.begin(prompt, 0)                       # 4 token tiles: the cut applies
+    got = a.logits()
+    assert np.all(np.abs(got - want) <= 1e-2 + 1e-3 * np.abs(want)), float(np.max(np.abs(got - want)))
+    assert a.argmax() == orc.greedy(want)
+    b.begin(prompt[:256], 0)                 # 2 token tiles each: one launch, no cut
+    b.wait()
+    b.begin(prompt[256:], 256)
+    lb = b.logits()
+    assert float(np.max(np.abs(got - lb))) <= 1e-4 * max(1.0, float(np.max(np.abs(lb))))
+    a.close(); b.close(); model.close(); osess.close(); om.close()
