@@ -119,6 +119,38 @@ def attention_cases(ctx, report=emit):
     return out_cases
 
 
+def attention_batch_cases(ctx, report=emit):
+    """The prompt form of the same chain (lv_kernel_attention with 16 rows or more: attention_prepare_kernel, then
+    attention_batch_kernel): n query rows at cache positions pos .. pos+n-1, 13B and 7B head counts.  Useful flops =
+    4 * head_size * sum over the rows of the positions each sees (scores and sums, a multiply-add = 2); the kernels execute 4 x
+    that (3 + 5 products of 16-bit operand pieces)."""
+    import numpy as np
+    out_cases = []
+    rot = 128
+    for heads, pos, n in ((40, 0, 512), (32, 0, 512), (40, 1536, 512), (40, 0, 128)):
+        dim, backlog = heads * rot, 2048
+        rng = np.random.default_rng(heads + pos)
+        host = (rng.standard_normal((backlog, dim)) * 0.5).astype(np.float16)
+        k, v = ctx.to_device(host), ctx.to_device(host)
+        q = ctx.to_device(lva.synth_normal(n, dim, seed=3))
+        out = ctx.zeros(n * dim * 4)
+        for _ in range(3):
+            lva.check(ctx.lib.lv_kernel_attention(ctx.h, out, k, v, q, pos, backlog, heads, rot, n))
+        ctx.sync()
+        iters = 50
+        ctx.timer_start()
+        for _ in range(iters):
+            lva.check(ctx.lib.lv_kernel_attention(ctx.h, out, k, v, q, pos, backlog, heads, rot, n))
+        us = ctx.timer_stop() * 1e3 / iters
+        pairs = sum(pos + z + 1 for z in range(n))
+        flops = 4.0 * rot * pairs * heads
+        out_cases.append(report(case="attention-batch", heads=heads, head_size=rot, first_position=pos, rows=n, us_both_kernels=round(us, 2),
+                                useful_TFLOPs=round(flops / us / 1e6, 1), executed_TFLOPs=round(4 * flops / us / 1e6, 1)))
+        for b in (k, v, q, out):
+            ctx.free(b)
+    return out_cases
+
+
 def copy_case(ctx):
     n = 1 << 30
     src, dst = ctx.zeros(n), ctx.zeros(n)
@@ -415,6 +447,8 @@ def main():
         gemv_cases(ctx)
     if which in ("attention", "all"):
         attention_cases(ctx)
+    if which == "attention-batch":
+        attention_batch_cases(ctx)
     if which == "gemm":
         gemm_cases(ctx)
     if which in ("decode-q8", "all"):
