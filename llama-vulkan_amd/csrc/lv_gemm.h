@@ -33,6 +33,7 @@ namespace lv {
 
 typedef _Float16 lv_h8 __attribute__((ext_vector_type(8)));
 typedef float lv_f16v __attribute__((ext_vector_type(16)));
+typedef float lv_f4v __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) void lv_lds_void;
 typedef const __attribute__((address_space(1))) void lv_glb_void;
 
@@ -511,7 +512,7 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a)
     constexpr int LPS = 5;   // direct loads per thread per stage
     extern __shared__ __attribute__((aligned(16))) uint8_t gemm_lds[];
     uint8_t *const lds = gemm_lds;
-    const int tid = threadIdx.x, lane = tid & 63, l31 = lane & 31, lhi = lane >> 5;
+    const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wn = wave & 3, wm = wave >> 2;
     const uint32_t tok_tiles = (a.n + TN - 1) / TN, row_tiles = a.tile_count ? a.tile_count : (a.rows + RM - 1) / RM;
@@ -544,41 +545,45 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a)
         if (p == 4) __builtin_amdgcn_global_load_lds((lv_glb_void *)(gs + sc * kGemmScBytes), (lv_lds_void *)(buf + kGemmWBytes + 2 * kGemmXBytes + (wave & 3) * 256), 4, 0, 0);
     };
 
-    lv_f16v acc[2][2];
+    // Accumulators: 4 x 4 tiles of 16 tokens x 16 rows (v_mfma_f32_16x16x32_f16: one instruction takes a whole quant block of
+    // K = 32).  Lane l of a tile holds weight row l % 16 and, in register r, token 4 * (l / 16) + r.
+    const int l15 = lane & 15, l4 = lane >> 4;
+    lv_f4v acc[4][4];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < 4; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
-    const lv_f16v zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < 4; j++) acc[i][j] = lv_f4v{0.f, 0.f, 0.f, 0.f};
+    const lv_f4v zero = {0.f, 0.f, 0.f, 0.f};
 
-    struct Frag { lv_h8 xh[2][2], xl[2][2], wc[2][2]; float d[2]; };
-    // one sixth of the operand reads of a stage (two 16-byte reads), the scales with the last
+    struct Frag { lv_h8 xh[4], xl[4], wc[4]; float d[4]; };
+    // one sixth of the operand reads of a stage (two 16-byte reads: lane l takes row l % 16 of a 16-row tile, k chunk l / 16),
+    // the scales with the last
     auto read_part = [&](Frag &f, const uint8_t *buf, int part) {
         const uint8_t *sW = buf, *sH = buf + kGemmWBytes, *sL = buf + kGemmWBytes + kGemmXBytes;
-        const int kk = part & 1, what = part >> 1;      // what: 0 weights, 1 low halves, 2 high halves
-        const int chunk = 2 * kk + lhi;
+        const int half = part & 1, what = part >> 1;      // what: 0 weights, 1 low halves, 2 high halves
 #pragma unroll
-        for (int t = 0; t < 2; t++) {
-            if (what == 0) f.wc[kk][t] = *reinterpret_cast<const lv_h8 *>(sW + (chunk * RM + wn * 64 + t * 32 + l31) * 16);
-            if (what == 1) f.xl[kk][t] = *reinterpret_cast<const lv_h8 *>(sL + (chunk * TN + wm * 64 + t * 32 + l31) * 16);
-            if (what == 2) f.xh[kk][t] = *reinterpret_cast<const lv_h8 *>(sH + (chunk * TN + wm * 64 + t * 32 + l31) * 16);
+        for (int u = 0; u < 2; u++) {
+            const int t = 2 * half + u;
+            if (what == 0) f.wc[t] = *reinterpret_cast<const lv_h8 *>(sW + (l4 * RM + wn * 64 + t * 16 + l15) * 16);
+            if (what == 1) f.xl[t] = *reinterpret_cast<const lv_h8 *>(sL + (l4 * TN + wm * 64 + t * 16 + l15) * 16);
+            if (what == 2) f.xh[t] = *reinterpret_cast<const lv_h8 *>(sH + (l4 * TN + wm * 64 + t * 16 + l15) * 16);
         }
         if (part == 5) {
             const float *sD = reinterpret_cast<const float *>(buf + kGemmWBytes + 2 * kGemmXBytes);
 #pragma unroll
-            for (int j = 0; j < 2; j++) f.d[j] = sD[wn * 64 + j * 32 + l31];
+            for (int j = 0; j < 4; j++) f.d[j] = sD[wn * 64 + j * 16 + l15];
         }
     };
-    lv_f16v c3 = zero;              // tile 3 of the step before and the last four values of its tile 2: their scaling into
-    float c2[4] = {0.f, 0.f, 0.f, 0.f}, dc[2] = {0.f, 0.f};   // the result is interleaved with this step's first MFMAs
+    // A step = 32 MFMA slots: tile t (token tile t / 4, row tile t % 4) takes two, low halves first (from zero), then high
+    // halves on top; tiles go in pairs (L0 L1 H0 H1 L2 L3 ...), so that no MFMA waits for the one before it.  The scale
+    // multiply-adds, two per slot, follow in tile order four slots behind: tile t's four in slots 4 + 2t and 5 + 2t, at least two
+    // slots after its second MFMA was issued.  Those of tiles 14 and 15 fall into the first four slots of the next step (cv, cd).
+    float cv[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, cd[2] = {0.f, 0.f};
     auto step = [&](uint32_t s, const Frag &cur, Frag &nxt) {
-        lv_f16v T[4];
+        lv_f4v T[16];
 #pragma unroll
-        for (int g = 0; g < 16; g++) {
-            const int t = g >> 2, m = g & 3, i = t >> 1, j = t & 1;
-            if (g == 8) {
+        for (int g = 0; g < 32; g++) {
+            if (g == 16) {
                 // stage s + 1 has landed for everyone, and everyone holds stage s in registers: from here on its buffer may
                 // take stage s + 4
                 asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NST - 2) * LPS) : "memory");
@@ -586,36 +591,34 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a)
                 asm volatile("" ::: "memory");
                 __builtin_amdgcn_sched_barrier(0);
             }
-            const lv_h8 &xa = m < 2 ? cur.xl[m & 1][i] : cur.xh[m & 1][i];
-            if (m == 0) T[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xa, cur.wc[0][j], zero, 0, 0, 0);
-            else T[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xa, cur.wc[m & 1][j], T[t], 0, 0, 0);
+            const int t = g >> 1, ti = t >> 2, tj = t & 3;
+            if ((g & 1) == 0) T[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(cur.xl[ti], cur.wc[tj], zero, 0, 0, 0);
+            else T[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(cur.xh[ti], cur.wc[tj], T[t], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
-            if (g == 0) {
 #pragma unroll
-                for (int r = 0; r < 4; r++) acc[1][0][12 + r] = fmaf(c2[r], dc[0], acc[1][0][12 + r]);
-            } else if (g <= 4) {
-#pragma unroll
-                for (int r = 4 * (g - 1); r < 4 * g; r++) acc[1][1][r] = fmaf(c3[r], dc[1], acc[1][1][r]);
-            } else {
-                const int q = g - 5, pt = q >> 2;
-#pragma unroll
-                for (int r = 4 * (q & 3); r < 4 * (q & 3) + 4; r++) acc[pt >> 1][pt & 1][r] = fmaf(T[pt][r], cur.d[pt & 1], acc[pt >> 1][pt & 1][r]);
+            for (int e = 0; e < 2; e++) {
+                if (g < 4) {
+                    const int idx = 2 * g + e;      // tiles 14 and 15 of the step before: token tile 3, row tiles 2 and 3
+                    acc[3][2 + (idx >> 2)][idx & 3] = fmaf(cv[idx], cd[idx >> 2], acc[3][2 + (idx >> 2)][idx & 3]);
+                } else {
+                    const int k = 2 * (g - 4) + e, q = k >> 2, r = k & 3;
+                    acc[q >> 2][q & 3][r] = fmaf(T[q][r], cur.d[q & 3], acc[q >> 2][q & 3][r]);
+                }
             }
-            if (g >= 8 && g < 14) read_part(nxt, lds + ((s + 1) % NST) * kGemmStageBytes, g - 8);
+            if (g >= 16 && g < 22) read_part(nxt, lds + ((s + 1) % NST) * kGemmStageBytes, g - 16);
             // the five loads of stage s + 4, one at a time between the MFMAs of this step's second half and the next step's
             // first: issued together right behind the barrier, the forty of a workgroup back up and hold the waves that
-            // issue them, MFMAs included (1520 instead of 1300 cycles a step)
-            if (g == 9) issue_one(s + NST, 0);
-            if (g == 12) issue_one(s + NST, 1);
-            if (g == 15) issue_one(s + NST, 2);
-            if (g == 2) issue_one(s + NST - 1, 3);
-            if (g == 5) issue_one(s + NST - 1, 4);
+            // issue them, MFMAs included
+            if (g == 18) issue_one(s + NST, 0);
+            if (g == 24) issue_one(s + NST, 1);
+            if (g == 30) issue_one(s + NST, 2);
+            if (g == 4) issue_one(s + NST - 1, 3);
+            if (g == 10) issue_one(s + NST - 1, 4);
             __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
-        for (int r = 0; r < 4; r++) c2[r] = T[2][12 + r];
-        c3 = T[3];
-        dc[0] = cur.d[0]; dc[1] = cur.d[1];
+        for (int r = 0; r < 4; r++) { cv[r] = T[14][r]; cv[4 + r] = T[15][r]; }
+        cd[0] = cur.d[2]; cd[1] = cur.d[3];
     };
 #ifdef LV_MEGA_TIMING
     const unsigned long long clk0 = clock64(), wall0 = wall_clock64();
@@ -635,9 +638,7 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a)
         step(s + 1, FB, FA);
     }
 #pragma unroll
-    for (int r = 0; r < 4; r++) acc[1][0][12 + r] = fmaf(c2[r], dc[0], acc[1][0][12 + r]);
-#pragma unroll
-    for (int r = 0; r < 16; r++) acc[1][1][r] = fmaf(c3[r], dc[1], acc[1][1][r]);
+    for (int idx = 0; idx < 8; idx++) acc[3][2 + (idx >> 2)][idx & 3] = fmaf(cv[idx], cd[idx >> 2], acc[3][2 + (idx >> 2)][idx & 3]);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // the repeats past the end have landed before the workgroup gives up its LDS
 #ifdef LV_MEGA_TIMING
     if (blockIdx.x == 0 && tid == 0) {
@@ -647,39 +648,39 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a)
     }
 #endif
 
-    // D[i][j]: i = token within the 32-tile, j = weight row; lane l holds j = l%32 and, in register r,
-    // i = 8*(r/4) + 4*(l/32) + r%4
-    // the per-token scales of this lane's 32 tokens, fetched before the first store (the stores may alias them for all the
+    // acc[ti][tj][r]: token tt * 128 + wm * 64 + ti * 16 + 4 * l4 + r, weight row rt * 256 + wn * 64 + tj * 16 + l15.
+    // The per-token scales of this lane's 16 tokens, fetched before the first store (the stores may alias them for all the
     // compiler knows, and a load behind every store costs the launch 6 us)
-    float4 ts[2][4];
+    float4 ts[4];
 #pragma unroll
-    for (int ti = 0; ti < 2; ti++)
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-            ts[ti][q] = make_float4(1.f, 1.f, 1.f, 1.f);
-            if (a.xscale) ts[ti][q] = *reinterpret_cast<const float4 *>(a.xscale + tt * TN + wm * 64 + ti * 32 + 8 * q + 4 * lhi);   // n_pad entries: in range
-        }
+    for (int ti = 0; ti < 4; ti++) {
+        ts[ti] = make_float4(1.f, 1.f, 1.f, 1.f);
+        if (a.xscale) ts[ti] = *reinterpret_cast<const float4 *>(a.xscale + tt * TN + wm * 64 + ti * 16 + 4 * l4);   // n_pad entries: in range
+    }
+    auto tscale = [&](int ti, int r) { return r == 0 ? ts[ti].x : r == 1 ? ts[ti].y : r == 2 ? ts[ti].z : ts[ti].w; };
     if constexpr (SILU) {
-        // acc[ti][0] = gate rows, acc[ti][1] = the same up rows: this lane's ff values of row rt * 128 + wn * 32 + l31 and its 32
-        // tokens.  They pass through LDS (per wave: [64 tokens][32 rows] halfs, high and low apart) to come out as 16-byte
-        // chunks of 8 consecutive rows of one token, consecutive lanes taking consecutive tokens: what a chunk row of the
-        // down projection's activation tile is.  Padding tokens give 0 * 0 / 2 = 0, as their rows of the tile must be.
+        // row tiles 0, 1 = gate rows, 2, 3 = the same up rows: this lane's ff values of rows rt * 128 + wn * 32 + tj * 16 + l15
+        // (tj = 0, 1) and its 16 tokens.  They pass through LDS (per wave: [64 tokens][32 rows] halfs, high and low apart) to
+        // come out as 16-byte chunks of 8 consecutive rows of one token, consecutive lanes taking consecutive tokens: what a
+        // chunk row of the down projection's activation tile is.  Padding tokens give 0 * 0 / 2 = 0, as their rows of the
+        // tile must be.
         constexpr int TS = 80;                      // bytes per token in the exchange: 64 + 16, so that 8 lanes' 16-byte reads miss each other's banks
         __syncthreads();                            // every wave holds its last operands in registers: the stages are free
         uint8_t *xb = lds + wave * (2 * 64 * TS);
 #pragma unroll
-        for (int ti = 0; ti < 2; ti++)
+        for (int ti = 0; ti < 4; ti++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int tok = ti * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
-                const float4 t4 = ts[ti][r / 4];
-                const float sc = (r % 4) == 0 ? t4.x : (r % 4) == 1 ? t4.y : (r % 4) == 2 ? t4.z : t4.w;
-                const float g = acc[ti][0][r] * sc, u = acc[ti][1][r] * sc;
-                const float f = g * u / (__expf(-u) + 1.f);
-                const uint16_t h = float_to_half_bits(f), l = float_to_half_bits(f - half_bits_to_float(h));
-                *reinterpret_cast<uint16_t *>(xb + tok * TS + l31 * 2) = h;
-                *reinterpret_cast<uint16_t *>(xb + 64 * TS + tok * TS + l31 * 2) = l;
-            }
+            for (int tj = 0; tj < 2; tj++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int tok = ti * 16 + 4 * l4 + r;
+                    const float sc = tscale(ti, r);
+                    const float g = acc[ti][tj][r] * sc, u = acc[ti][tj + 2][r] * sc;
+                    const float f = g * u / (__expf(-u) + 1.f);
+                    const uint16_t h = float_to_half_bits(f), l = float_to_half_bits(f - half_bits_to_float(h));
+                    *reinterpret_cast<uint16_t *>(xb + tok * TS + (tj * 16 + l15) * 2) = h;
+                    *reinterpret_cast<uint16_t *>(xb + 64 * TS + tok * TS + (tj * 16 + l15) * 2) = l;
+                }
         __syncthreads();
         const uint32_t n = tt * TN + wm * 64 + lane;                  // below n_pad: the token tiles cover the padded batch
 #pragma unroll
@@ -699,15 +700,13 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a)
             __syncthreads();                            // every wave holds its last operands in registers: the stages are free
             uint8_t *xb = lds + wave * (64 * TS);
 #pragma unroll
-            for (int ti = 0; ti < 2; ti++)
+            for (int ti = 0; ti < 4; ti++)
 #pragma unroll
-                for (int tj = 0; tj < 2; tj++)
+                for (int tj = 0; tj < 4; tj++)
 #pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        const int tok = ti * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
-                        const float4 t4 = ts[ti][r / 4];
-                        const float sc = (r % 4) == 0 ? t4.x : (r % 4) == 1 ? t4.y : (r % 4) == 2 ? t4.z : t4.w;
-                        *reinterpret_cast<uint16_t *>(xb + tok * TS + (tj * 32 + l31) * 2) = float_to_half_bits(acc[ti][tj][r] * sc);
+                    for (int r = 0; r < 4; r++) {
+                        const int tok = ti * 16 + 4 * l4 + r;
+                        *reinterpret_cast<uint16_t *>(xb + tok * TS + (tj * 16 + l15) * 2) = float_to_half_bits(acc[ti][tj][r] * tscale(ti, r));
                     }
             __syncthreads();
             const uint32_t row0 = (a.row_ptr ? *a.row_ptr : 0u) + a.row_add;
@@ -724,18 +723,16 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a)
     }
     float *const out = a.outs[z];
 #pragma unroll
-    for (int ti = 0; ti < 2; ti++)
+    for (int ti = 0; ti < 4; ti++)
 #pragma unroll
-        for (int tj = 0; tj < 2; tj++) {
-            const uint32_t m = rt * RM + wn * 64 + tj * 32 + l31;
+        for (int tj = 0; tj < 4; tj++) {
+            const uint32_t m = rt * RM + wn * 64 + tj * 16 + l15;
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const uint32_t n = tt * TN + wm * 64 + ti * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
-                const float4 t4 = ts[ti][r / 4];
-                const float sc = (r % 4) == 0 ? t4.x : (r % 4) == 1 ? t4.y : (r % 4) == 2 ? t4.z : t4.w;
+            for (int r = 0; r < 4; r++) {
+                const uint32_t n = tt * TN + wm * 64 + ti * 16 + 4 * l4 + r;
                 if (n < a.n && m < a.rows) {
                     float *dst = out + (size_t)n * a.ldo + (m - a.tile0 * RM);
-                    const float v = acc[ti][tj][r] * sc;
+                    const float v = acc[ti][tj][r] * tscale(ti, r);
                     *dst = a.accumulate ? *dst + v : v;
                 }
             }
