@@ -90,7 +90,7 @@ def lavapipe_status():
 
 def other_cases(lva, ctx):
     """The other configurations under the same clock, after the headline's timed region: isolated GEMVs at the 7B decode
-    shapes in both weight types, 7B q8_0 at positions 1920..2047, 13B q4_0 with a 32-token prompt and 256 steps (on the
+    shapes in both weight types, the 512-token GEMM at the 13B layer shapes, 7B q8_0 at positions 1920..2047, 13B q4_0 with a 32-token prompt and 256 steps (on the
     persistent kernel and on the hipGraph of the operator chain), the 7B q4_0 headline workload on the hipGraph path, and
     the 13B q8_0 512-token prompt.  Each entry carries tok_s or ms or us, and frac of the roofline that bounds it (HBM for
     decode and GEMV, matrix cores for the prompt)."""
@@ -108,6 +108,9 @@ def other_cases(lva, ctx):
         d = measure.decode_case(ctx, *args, report=q, **kw)
         cases.append({"name": name, "path": d["path"], "tok_s": d["tok_s"], "ms": d["ms_per_token"], "GBps": d["GBps"], "frac": d["frac_of_peak"],
                       "bound": "hbm"})
+    for g in measure.gemm_cases(ctx, report=q):
+        cases.append({"name": f"gemm {g['wtype']} {g['rows']}x{g['cols']}, {g['tokens']} tokens (one lv_kernel_gemm call)", "us": g["us"],
+                      "executed_TFLOPs": g["executed_TFLOPs"], "frac": g["executed_frac_of_peak"], "bound": "mfma"})
     p = measure.prefill_case(ctx, "prefill-13b", "13b", lva.LV_Q8_0, report=q)
     cases.append({"name": "13B q8_0 prompt of 512 tokens as one step", "tok_s": p["tok_s"], "ms": p["ms"], "executed_TFLOPs": p["executed_TFLOPs"],
                   "frac": p["frac_of_mfma_peak"], "bound": "mfma"})

@@ -181,7 +181,9 @@ int lv_kernel_dequant(lv_ctx *ctx, const lv_matrix *m, uint32_t row0, uint32_t n
 int lv_kernel_gemv(lv_ctx *ctx, float *out, const lv_matrix *w, const float *x, uint32_t batch, int accumulate);
 /* the same product for many rows at once on the matrix cores: the *_batch variants of the shaders the reference
  * switches to when several tokens are pending (llava_session.cpp:243-255, llava_pipeline.cpp batch_enabled).
- * out[batch][rows] (+)= x[batch][cols] * W^T.  Synchronous (it owns a temporary workspace). */
+ * out[batch][rows] (+)= x[batch][cols] * W^T.  The first call on a matrix makes its prompt copy (2 bytes a weight, kept
+ * until lv_matrix_destroy); the activation workspace belongs to the context and only grows.  Neither is allocated again
+ * by later calls of the same size, which are asynchronous like the other kernels. */
 int lv_kernel_gemm(lv_ctx *ctx, float *out, const lv_matrix *w, const float *x, uint32_t batch, int accumulate);
 /* matmul_silu_ff* (matmul_silu_ff.comp:49-97): out = (W3 x) * silu(W1 x) */
 int lv_kernel_gemv_silu(lv_ctx *ctx, float *out, const lv_matrix *w3, const lv_matrix *w1, const float *x,

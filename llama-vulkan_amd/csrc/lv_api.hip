@@ -73,6 +73,9 @@ struct lv_ctx {
     uint32_t trig_abs_rows = 0, trig_abs_rot = 0;
     uint16_t *attn_planes = nullptr;
     size_t attn_plane_halfs = 0;
+    // workspace of the stand-alone GEMM entry point (activation halves, row scales, K-slice partials); grows, never shrinks
+    uint16_t *gemm_ws = nullptr;
+    size_t gemm_ws_bytes = 0;
     hipEvent_t ev_start = nullptr, ev_stop = nullptr;
     struct AttnScratch *scratch = nullptr;   // this device's copy of the file-scope scratch array (lv_kernel_attention_static)
     // Persistent decode kernels of different sessions (one per thread, llava_context.h:47-49 has the same pools and
@@ -89,7 +92,8 @@ struct lv_matrix {
     MatView view{};
     uint32_t ftype = 0;
     uint64_t bytes = 0;
-    const uint16_t *h16 = nullptr;   // prompt copy (lv_gemm.h): codes as fp16 integers and fp32 scales in tile order; null until a batch needs it
+    mutable const uint16_t *h16 = nullptr;   // prompt copy (lv_gemm.h): codes as fp16 integers and fp32 scales in tile order; null until a batch needs it
+    mutable uint16_t *h16_owned = nullptr;   // that copy when lv_kernel_gemm made it for a matrix outside a model; freed with the matrix
 };
 
 struct LayerWeights {
@@ -249,6 +253,7 @@ extern "C" int lv_ctx_destroy(lv_ctx *c)
     (void)hipFree(c->attn_counters);
     (void)hipFree(c->trig_abs);
     (void)hipFree(c->attn_planes);
+    (void)hipFree(c->gemm_ws);
     if (c->ev_start) (void)hipEventDestroy(c->ev_start);
     if (c->ev_stop) (void)hipEventDestroy(c->ev_stop);
     if (c->mega_done) (void)hipEventDestroy(c->mega_done);
@@ -484,6 +489,11 @@ extern "C" int lv_matrix_upload(lv_ctx *c, const void *blocks, uint32_t ftype, u
 extern "C" int lv_matrix_destroy(lv_matrix *m)
 {
     if (!m) return LV_OK;
+    if (m->h16_owned) {
+        // launches that read the copy may still be queued on the context's stream
+        if (m->ctx) { (void)hipSetDevice(m->ctx->device); (void)hipStreamSynchronize(m->ctx->stream); }
+        (void)hipFree(m->h16_owned);
+    }
     if (m->owned) (void)hipFree(m->owned);
     delete m;
     return LV_OK;
@@ -964,29 +974,40 @@ extern "C" int lv_kernel_gemm(lv_ctx *c, float *out, const lv_matrix *w, const f
     HIP_TRY(hipSetDevice(c->device));
     const size_t n_pad = (batch + kGemmTile - 1) / kGemmTile * kGemmTile, halfs = n_pad * gemm_k_padded(w->view.cols);
     if (w->view.cols % 32) return fail(LV_ERR_ARG, "gemm: %u columns", w->view.cols);
-    // workspace: the matrix's prompt copy, the two fp16 halves of the activations and, where K is cut in slices, their
-    // partial results
+    // The matrix's prompt copy is made by the first call and stays with the matrix; the workspace (the two fp16 halves of
+    // the activations, their row scales and, where K is cut in slices, the partial results) stays with the context.
+    if (!w->h16) {
+        hipError_t e = hipMalloc(reinterpret_cast<void **>(&w->h16_owned), (size_t)prompt_copy_halfs(*w) * 2);
+        if (e != hipSuccess) { w->h16_owned = nullptr; return fail(LV_ERR_OOM, "lv_kernel_gemm: prompt copy of the matrix"); }
+        int rc = launch_expand(c->stream, w->h16_owned, *w);
+        if (rc != LV_OK) {
+            (void)hipStreamSynchronize(c->stream);
+            (void)hipFree(w->h16_owned);
+            w->h16_owned = nullptr;
+            return rc;
+        }
+        w->h16 = w->h16_owned;
+    }
     const uint32_t slices = gemm_slices_for(*w, batch, w->view.rows);
     const size_t part = slices > 1 ? (size_t)batch * w->view.rows : 0;
-    const size_t w_halfs = w->h16 ? 0 : (size_t)prompt_copy_halfs(*w);
-    uint16_t *ws = nullptr;
-    hipError_t e = hipMalloc(reinterpret_cast<void **>(&ws), (w_halfs + halfs * 2) * 2 + n_pad * 4 + part * slices * 4);
-    if (e != hipSuccess) return fail(LV_ERR_OOM, "lv_kernel_gemm: workspace");
-    uint16_t *xh = ws + w_halfs, *xl = xh + halfs;
+    const size_t need = halfs * 2 * 2 + n_pad * 4 + part * slices * 4;
+    if (need > c->gemm_ws_bytes) {
+        HIP_TRY(hipStreamSynchronize(c->stream));
+        (void)hipFree(c->gemm_ws);
+        c->gemm_ws = nullptr;
+        c->gemm_ws_bytes = 0;
+        if (hipMalloc(reinterpret_cast<void **>(&c->gemm_ws), need) != hipSuccess) {
+            c->gemm_ws = nullptr;
+            return fail(LV_ERR_OOM, "lv_kernel_gemm: workspace");
+        }
+        c->gemm_ws_bytes = need;
+    }
+    uint16_t *xh = c->gemm_ws, *xl = xh + halfs;
     float *xscale = reinterpret_cast<float *>(xl + halfs);
     float *p0 = xscale + n_pad;
     float *const parts[kGemmMaxMats] = {p0, p0 + part, p0 + 2 * part, p0 + 3 * part};
-    lv_matrix wm = *w;
-    int rc = LV_OK;
-    if (!wm.h16) {
-        rc = launch_expand(c->stream, ws, *w);
-        wm.h16 = ws;
-    }
-    if (rc == LV_OK) rc = launch_split(c->stream, xh, xl, xscale, x, batch, w->view.cols);
-    if (rc == LV_OK) rc = launch_gemm_sliced(c->stream, out, w->view.rows, wm, batch, xh, xl, xscale, accumulate != 0, slices > 1 ? parts : nullptr);
-    (void)hipStreamSynchronize(c->stream);
-    (void)hipFree(ws);
-    return rc;
+    LV_TRY(launch_split(c->stream, xh, xl, xscale, x, batch, w->view.cols));
+    return launch_gemm_sliced(c->stream, out, w->view.rows, *w, batch, xh, xl, xscale, accumulate != 0, slices > 1 ? parts : nullptr);
 }
 
 extern "C" int lv_kernel_normalize(lv_ctx *c, float *out, const float *x, const float *w, uint32_t dim, uint32_t batch)

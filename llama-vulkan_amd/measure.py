@@ -411,23 +411,33 @@ def gemm_clock_case():
     ctx.close()
 
 
-def gemm_cases(ctx):
-    """lv_kernel_gemm allocates its workspace and splits the activations in every call, so the time of a call is not the
-    kernel's: this case exists to put gemm_kernel launches of known shape under rocprofv3 (kernel trace, counters)"""
+def gemm_cases(ctx, report=emit):
+    """reference: the *_batch shaders on 512 pending tokens (llava_session.cpp:243-255).  One lv_kernel_gemm call = the split of
+    the activations into fp16 halves + gemm_kernel (+ the sum of the K slices where the grid would not fill the device), at
+    the 13B layer shapes; the matrix's prompt copy and the workspace exist after the first call.  flops = 2 * tokens *
+    rows * cols; every product is executed twice (two activation halves)."""
     n, wtype = 512, lva.LV_Q8_0
+    out_cases = []
     for rows, cols in ((5120, 5120), (13824, 5120), (5120, 13824)):
         m = ctx.matrix(lva.synth_quant(wtype, rows, cols, seed=1), wtype, rows, cols)
         x = ctx.to_device(lva.synth_normal(n, cols, seed=2))
         out = ctx.zeros(n * rows * 4)
-        reps = 6
-        t0 = time.perf_counter()
-        for _ in range(reps):
+        for _ in range(3):
             lva.check(ctx.lib.lv_kernel_gemm(ctx.h, out, m, x, n, 0))
         ctx.sync()
-        emit(case="gemm", wtype="q8_0", rows=rows, cols=cols, tokens=n, launches=reps, us_per_call_with_workspace=round((time.perf_counter() - t0) / reps * 1e6, 1))
+        reps = 20
+        ctx.timer_start()
+        for _ in range(reps):
+            lva.check(ctx.lib.lv_kernel_gemm(ctx.h, out, m, x, n, 0))
+        us = ctx.timer_stop() * 1e3 / reps
+        useful = 2.0 * n * rows * cols / us / 1e6
+        out_cases.append(report(case="gemm", wtype="q8_0", rows=rows, cols=cols, tokens=n, launches=reps, us=round(us, 1),
+                                useful_TFLOPs=round(useful, 1), executed_TFLOPs=round(2 * useful, 1),
+                                executed_frac_of_peak=round(2 * useful / MFMA_PEAK_TFLOPS, 4)))
         ctx.matrix_free(m)
         ctx.free(x)
         ctx.free(out)
+    return out_cases
 
 
 def main():

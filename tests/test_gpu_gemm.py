@@ -90,6 +90,33 @@ def test_gemm_special_inputs(lva, orc, ctx):
     ctx.matrix_free(m)
 
 
+def test_gemm_calls_in_a_row_keep_their_workspace(lva, orc, ctx):
+    """lv_kernel_gemm keeps a matrix's prompt copy with the matrix and the activation workspace with the context: calls of
+    different sizes and on different matrices queued without a wait between them must not disturb each other, and a matrix
+    may be destroyed right after its call"""
+    shapes = [(lva.LV_Q8_0, 512, 1024, 96), (lva.LV_Q4_0, 256, 4096, 130), (lva.LV_Q8_0, 512, 1024, 17), (lva.LV_Q4_0, 4096, 4096, 512)]
+    mats, keep = {}, []
+    for i, (ftype, rows, cols, batch) in enumerate(shapes):
+        key = (ftype, rows, cols)
+        if key not in mats:
+            blocks = lva.synth_quant(ftype, rows, cols, seed=90 + i)
+            mats[key] = (blocks, ctx.matrix(blocks, ftype, rows, cols))
+        blocks, m = mats[key]
+        x = lva.synth_normal(batch, cols, seed=95 + i)
+        dx, dout = ctx.to_device(x), ctx.alloc(batch * rows * 4)
+        lva.check(ctx.lib.lv_kernel_gemm(ctx.h, dout, m, dx, batch, 0))     # queued; nothing waits here
+        keep.append((blocks, ftype, rows, cols, batch, x, dx, dout))
+    for blocks, m in mats.values():
+        ctx.matrix_free(m)
+    for blocks, ftype, rows, cols, batch, x, dx, dout in keep:
+        got = ctx.to_host(dout, (batch, rows), np.float32)
+        want = orc.gemv(blocks, ftype, rows, cols, x)
+        bound = 1e-5 * _abs_dot_bound(orc, blocks, ftype, rows, cols, x) + 1e-7
+        assert float(np.max(np.abs(got.astype(np.float64) - want) / bound)) <= 1.0, (rows, cols, batch)
+        ctx.free(dx)
+        ctx.free(dout)
+
+
 @pytest.mark.parametrize("name,n_prompt", [("tiny_q4", 40), ("tiny_q8", 130), ("small_q4", 77), ("pair_q4", 150), ("pair_q8", 33)])
 def test_prompt_as_one_batch_matches_oracle(lva, orc, ctx, tiny_models, name, n_prompt):
     path = tiny_models[name]
