@@ -128,8 +128,10 @@ int lv_kv_read(lv_session *s, uint32_t layer, int which, uint32_t n_tokens, void
 int lv_kv_write(lv_session *s, uint32_t layer, int which, uint32_t n_tokens, const void *src);
 
 /* ---- record mode: replaces the per-layer trace buffers of llava_layer_session_data.cpp:79-86 and their
- *      routing in llava_layer.cpp:43-51.  When enabled, every step keeps, per layer and for the last row:
- *      LV_TRACE_* below.  lv_trace_read copies one of them (count floats) to the host. */
+ *      routing in llava_layer.cpp:43-51.  When enabled, every step keeps, per layer and for every row of the step (the
+ *      reference's buffers are batch_size rows long, llava_layer_session_data.cpp:80-85), the LV_TRACE_* below; the
+ *      next step replaces them.  Memory: layers x rows x (5 x max(dim, ff) + backlog x heads) floats, grown to the
+ *      longest step recorded so far. */
 enum {
     LV_TRACE_NORM_IN = 0,        /* normalized_input_logit  [dim] */
     LV_TRACE_POST_ATTN = 1,      /* post_attn_logit         [dim] */
@@ -141,6 +143,12 @@ enum {
     LV_TRACE_COUNT = 6
 };
 int lv_trace_enable(lv_session *s, int enable);
+/* rows of the last recorded step (0 before the first) */
+int lv_trace_rows(lv_session *s, uint32_t *rows);
+/* rows [row0, row0 + n_rows) of one buffer of the last recorded step to the host, row after row with nothing between
+ * them: the memory layout of the reference's buffer (z_id * dim, z_id * BACKLOG * HEAD_COUNT: mhsa.comp:58) */
+int lv_trace_read_rows(lv_session *s, uint32_t layer, int which, uint32_t row0, uint32_t n_rows, float *dst);
+/* the last row of the last recorded step (count = the floats of one row) */
 int lv_trace_read(lv_session *s, uint32_t layer, int which, float *dst, uint32_t count);
 
 /* ---- device memory helpers for callers of the lv_kernel_* entry points (tests, microbenchmarks) -------- */

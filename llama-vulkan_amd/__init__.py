@@ -101,6 +101,8 @@ _HIP_SIGS = {
     "lv_kv_write": [_VP, _U32, _I, _U32, _VP],
     "lv_trace_enable": [_VP, _I],
     "lv_trace_read": [_VP, _U32, _I, _VP, _U32],
+    "lv_trace_rows": [_VP, C.POINTER(_U32)],
+    "lv_trace_read_rows": [_VP, _U32, _I, _U32, _U32, _VP],
     "lv_dev_alloc": [_VP, _U64, C.POINTER(_VP)],
     "lv_dev_free": [_VP, _VP],
     "lv_dev_upload": [_VP, _VP, _VP, _U64],
@@ -410,4 +412,23 @@ class Session:
             n = rows.value * self.model.header["heads"]
         out = np.empty(n, dtype=np.float32)
         check(self.lib.lv_trace_read(self.h, layer, which, _ptr(out), n))
+        return out
+
+    def trace_rows(self):
+        """rows the last recorded step left in the trace buffers"""
+        rows = C.c_uint32()
+        check(self.lib.lv_trace_rows(self.h, C.byref(rows)))
+        return rows.value
+
+    def trace_all(self, layer, which, row0=0, n_rows=None):
+        """rows [row0, row0 + n_rows) of one trace buffer of the last recorded step, shape (n_rows, floats per row)"""
+        n = self.model.header["ff"] if which == TRACE_FF else self.model.header["dim"]
+        if which == TRACE_ATTN:
+            rows = C.c_uint32()
+            check(self.lib.lv_session_backlog(self.h, C.byref(rows)))
+            n = rows.value * self.model.header["heads"]
+        if n_rows is None:
+            n_rows = self.trace_rows() - row0
+        out = np.empty((n_rows, n), dtype=np.float32)
+        check(self.lib.lv_trace_read_rows(self.h, layer, which, row0, n_rows, _ptr(out)))
         return out

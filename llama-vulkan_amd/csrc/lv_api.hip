@@ -189,8 +189,11 @@ struct lv_session {
     bool in_flight = false;
     bool have_logits = false;
     bool trace = false;
-    float *trace_buf = nullptr;  // [layers][LV_TRACE_ATTN][max(dim, ff)]: the five vector buffers
-    float *trace_attn = nullptr; // [layers][backlog][heads]: LV_TRACE_ATTN; follows the backlog
+    // record mode keeps every row of a step, as the reference's batch-sized buffers do (llava_layer_session_data.cpp:79-86)
+    float *trace_buf = nullptr;  // [layers][LV_TRACE_ATTN][trace_cap][max(dim, ff)]: the five vector buffers
+    float *trace_attn = nullptr; // [layers][trace_cap][backlog][heads]: LV_TRACE_ATTN; follows the backlog
+    uint32_t trace_cap = 0;      // rows the two buffers have room for
+    uint32_t trace_n = 0;        // rows the last recorded step wrote
     hipEvent_t ev_start = nullptr, ev_stop = nullptr;
 };
 
@@ -1465,18 +1468,46 @@ extern "C" int lv_session_create(lv_model *m, lv_session **out)
     return LV_OK;
 }
 
-// record mode's attention weights: one [backlog][heads] buffer per layer, zero until a traced step fills it
+// record mode's attention weights: one [backlog][heads] buffer per layer and row of a step, zero until a traced step fills it
 static int make_trace_attn(lv_session *s, uint32_t backlog)
 {
     const lv_hparams &hp = s->model->hp;
-    const size_t bytes = (size_t)hp.layers * backlog * hp.heads * 4;
+    const size_t bytes = (size_t)hp.layers * s->trace_cap * backlog * hp.heads * 4;
     if (bytes == 0) return LV_OK;
     hipError_t e = hipMalloc(reinterpret_cast<void **>(&s->trace_attn), bytes);
     if (e != hipSuccess) {
         (void)hipGetLastError();
-        return fail(e == hipErrorOutOfMemory ? LV_ERR_OOM : LV_ERR_HIP, "record mode: attention weights of %u rows: %s", backlog, hipGetErrorString(e));
+        s->trace_attn = nullptr;
+        return fail(e == hipErrorOutOfMemory ? LV_ERR_OOM : LV_ERR_HIP, "record mode: attention weights of %u steps rows x %u cache rows: %s", s->trace_cap, backlog,
+                    hipGetErrorString(e));
     }
     return zero_async(s->trace_attn, bytes, s->stream);
+}
+
+// room for the trace buffers of a step of `rows` tokens (the reference re-creates its buffers when the batch size
+// changes, llava_layer_session_data.cpp:60-61; here they only grow).  What an earlier step left is dropped on growth.
+static int trace_reserve(lv_session *s, uint32_t rows)
+{
+    if (rows <= s->trace_cap) return LV_OK;
+    const lv_hparams &hp = s->model->hp;
+    const size_t slot = hp.dim > hp.ff ? hp.dim : hp.ff;
+    HIP_TRY(hipStreamSynchronize(s->stream));
+    (void)hipFree(s->trace_buf);
+    (void)hipFree(s->trace_attn);
+    s->trace_buf = nullptr;
+    s->trace_attn = nullptr;
+    s->trace_cap = 0;
+    s->trace_n = 0;
+    const size_t bytes = (size_t)hp.layers * LV_TRACE_ATTN * rows * slot * 4;
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&s->trace_buf), bytes);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        s->trace_buf = nullptr;
+        return fail(e == hipErrorOutOfMemory ? LV_ERR_OOM : LV_ERR_HIP, "record mode: buffers for a step of %u rows: %s", rows, hipGetErrorString(e));
+    }
+    s->trace_cap = rows;
+    LV_TRY(zero_async(s->trace_buf, bytes, s->stream));
+    return make_trace_attn(s, s->backlog);
 }
 
 extern "C" int lv_session_reserve(lv_session *s, uint32_t backlog)
@@ -1618,12 +1649,23 @@ static int launch_mega(lv_session *s, uint32_t pos, uint32_t token, bool *refuse
 // -----------------------------------------------------------------------------------------------------------
 // the step
 // -----------------------------------------------------------------------------------------------------------
-static int trace_copy(lv_session *s, uint32_t layer, int which, const float *src, size_t count)
+static float *trace_slot(const lv_session *s, uint32_t layer, int which, uint32_t row)
 {
-    if (!s->trace) return LV_OK;
     const lv_hparams &hp = s->model->hp;
     const size_t slot = hp.dim > hp.ff ? hp.dim : hp.ff;
-    float *dst = s->trace_buf + ((size_t)layer * LV_TRACE_ATTN + which) * slot;
+    return s->trace_buf + (((size_t)layer * LV_TRACE_ATTN + which) * s->trace_cap + row) * slot;
+}
+
+static float *trace_attn_slot(const lv_session *s, uint32_t layer, uint32_t row)
+{
+    return s->trace_attn + ((size_t)layer * s->trace_cap + row) * s->backlog * s->model->hp.heads;
+}
+
+// row = the token's index in its step
+static int trace_copy(lv_session *s, uint32_t layer, int which, uint32_t row, const float *src, size_t count)
+{
+    if (!s->trace) return LV_OK;
+    float *dst = trace_slot(s, layer, which, row);
     HIP_TRY(hipMemcpyAsync(dst, src, count * 4, hipMemcpyDeviceToDevice, s->stream));
     return LV_OK;
 }
@@ -1663,7 +1705,7 @@ static int record_token(lv_session *s, uint32_t idx, bool with_head)
         } else {
             normalize_kernel<<<dim3(1), dim3(256), 0, st>>>(s->xn, s->x, lw.attn_norm, D);
             HIP_TRY(hipGetLastError());
-            LV_TRY(trace_copy(s, li, LV_TRACE_NORM_IN, s->xn, D));
+            LV_TRY(trace_copy(s, li, LV_TRACE_NORM_IN, idx, s->xn, D));
             LV_TRY(launch_gemv3(st, outs, mats, s->xn));
             kv_append2_kernel<<<dim3(kv_grid.x, kv_grid.y, 2), dim3(256), 0, st>>>(kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->k, s->v, pos_ptr, idx, D, s->backlog);
             HIP_TRY(hipGetLastError());
@@ -1671,23 +1713,23 @@ static int record_token(lv_session *s, uint32_t idx, bool with_head)
         LV_TRY(launch_attention(st, s->vo, kv_ptr(s, li, 0), kv_ptr(s, li, 1), s->q, s->trig, s->attn_part, s->attn_counters,
                                 pos_ptr, idx, s->backlog, hp.heads, hp.rot, 1));
         if (s->trace) {
-            attn_weights_kernel<<<dim3(hp.heads), dim3(256), 0, st>>>(s->trace_attn + (size_t)li * s->backlog * hp.heads, kv_ptr(s, li, 0), s->q,
+            attn_weights_kernel<<<dim3(hp.heads), dim3(256), 0, st>>>(trace_attn_slot(s, li, idx), kv_ptr(s, li, 0), s->q,
                                                                        s->trig, pos_ptr, idx, hp.heads, hp.rot, s->backlog);
             HIP_TRY(hipGetLastError());
         }
         LV_TRY(launch_gemv(st, s->x, lw.wo, nullptr, s->vo, 1, kGemvAdd));
-        LV_TRY(trace_copy(s, li, LV_TRACE_POST_ATTN, s->x, D));
+        LV_TRY(trace_copy(s, li, LV_TRACE_POST_ATTN, idx, s->x, D));
         if (fused) {
             LV_TRY(launch_gemv(st, s->ff, lw.w3, &lw.w1, s->x, 1, kGemvSilu, lw.ffn_norm));
         } else {
             normalize_kernel<<<dim3(1), dim3(256), 0, st>>>(s->xn, s->x, lw.ffn_norm, D);
             HIP_TRY(hipGetLastError());
-            LV_TRY(trace_copy(s, li, LV_TRACE_POST_ATTN_NORM, s->xn, D));
+            LV_TRY(trace_copy(s, li, LV_TRACE_POST_ATTN_NORM, idx, s->xn, D));
             LV_TRY(launch_gemv(st, s->ff, lw.w3, &lw.w1, s->xn, 1, kGemvSilu));
         }
-        LV_TRY(trace_copy(s, li, LV_TRACE_FF, s->ff, F));
+        LV_TRY(trace_copy(s, li, LV_TRACE_FF, idx, s->ff, F));
         LV_TRY(launch_gemv(st, s->x, lw.w2, nullptr, s->ff, 1, kGemvAdd));
-        LV_TRY(trace_copy(s, li, LV_TRACE_OUT, s->x, D));
+        LV_TRY(trace_copy(s, li, LV_TRACE_OUT, idx, s->x, D));
     }
     if (with_head) {
         if (!s->trace && gemv_streams(m->output.view, 1)) {
@@ -1904,6 +1946,10 @@ extern "C" int lv_step_begin(lv_session *s, const uint32_t *tokens, uint32_t n, 
 
     s->have_logits = false;
     s->pick_in_status = false;
+    if (s->trace) {
+        LV_TRY(trace_reserve(s, n));
+        s->trace_n = n;
+    }
 
     int path = LV_PATH_AUTO;
     (void)lv_session_path(s, &path);
@@ -2069,15 +2115,43 @@ extern "C" int lv_trace_enable(lv_session *s, int enable)
 {
     if (!s) return fail(LV_ERR_ARG, "lv_trace_enable: session is null");
     if (s->in_flight) return fail(LV_ERR_STATE, "lv_trace_enable: a step is in flight");
-    const lv_hparams &hp = s->model->hp;
     if (enable && !s->trace_buf) {
-        const size_t slot = hp.dim > hp.ff ? hp.dim : hp.ff;
         HIP_TRY(hipSetDevice(s->model->ctx->device));
-        HIP_TRY(hipMalloc(reinterpret_cast<void **>(&s->trace_buf), (size_t)hp.layers * LV_TRACE_ATTN * slot * 4));
-        LV_TRY(make_trace_attn(s, s->backlog));
+        LV_TRY(trace_reserve(s, 1));
         HIP_TRY(hipStreamSynchronize(s->stream));
     }
     s->trace = enable != 0;
+    return LV_OK;
+}
+
+extern "C" int lv_trace_rows(lv_session *s, uint32_t *rows)
+{
+    if (!s || !rows) return fail(LV_ERR_ARG, "lv_trace_rows: null argument");
+    if (!s->trace || !s->trace_buf) return fail(LV_ERR_STATE, "lv_trace_rows: record mode is off");
+    *rows = s->trace_n;
+    return LV_OK;
+}
+
+extern "C" int lv_trace_read_rows(lv_session *s, uint32_t layer, int which, uint32_t row0, uint32_t n_rows, float *dst)
+{
+    if (!s || (n_rows && !dst)) return fail(LV_ERR_ARG, "lv_trace_read_rows: null argument");
+    if (!s->trace || !s->trace_buf) return fail(LV_ERR_STATE, "lv_trace_read_rows: record mode is off");
+    const lv_hparams &hp = s->model->hp;
+    if (layer >= hp.layers || which < 0 || which >= LV_TRACE_COUNT) return fail(LV_ERR_RANGE, "lv_trace_read_rows: layer %u / buffer %d", layer, which);
+    if (row0 > s->trace_n || n_rows > s->trace_n - row0)
+        return fail(LV_ERR_RANGE, "lv_trace_read_rows: rows %u..%u of a step of %u", row0, row0 + n_rows, s->trace_n);
+    if (n_rows == 0) return LV_OK;
+    HIP_TRY(hipSetDevice(s->model->ctx->device));
+    if (which == LV_TRACE_ATTN) {
+        if (!s->trace_attn) return fail(LV_ERR_STATE, "lv_trace_read_rows: no attention weights (the cache has no rows)");
+        // rows of one layer lie one after the other
+        HIP_TRY(hipMemcpyAsync(dst, trace_attn_slot(s, layer, row0), (size_t)n_rows * s->backlog * hp.heads * 4, hipMemcpyDeviceToHost, s->stream));
+    } else {
+        const size_t slot = hp.dim > hp.ff ? hp.dim : hp.ff, have = which == LV_TRACE_FF ? hp.ff : hp.dim;
+        HIP_TRY(hipMemcpy2DAsync(dst, have * 4, trace_slot(s, layer, which, row0), slot * 4, have * 4, n_rows, hipMemcpyDeviceToHost, s->stream));
+    }
+    HIP_TRY(hipStreamSynchronize(s->stream));
+    s->in_flight = false;
     return LV_OK;
 }
 
@@ -2088,13 +2162,13 @@ extern "C" int lv_trace_read(lv_session *s, uint32_t layer, int which, float *ds
     const lv_hparams &hp = s->model->hp;
     if (layer >= hp.layers || which < 0 || which >= LV_TRACE_COUNT) return fail(LV_ERR_RANGE, "lv_trace_read: layer %u / buffer %d", layer, which);
     const uint32_t have = which == LV_TRACE_FF ? hp.ff : which == LV_TRACE_ATTN ? s->backlog * hp.heads : hp.dim;
-    if (count != have) return fail(LV_ERR_ARG, "lv_trace_read: buffer %d holds %u floats, %u asked", which, have, count);
-    const size_t slot = hp.dim > hp.ff ? hp.dim : hp.ff;
-    const float *src = which == LV_TRACE_ATTN ? s->trace_attn + (size_t)layer * have : s->trace_buf + ((size_t)layer * LV_TRACE_ATTN + which) * slot;
-    HIP_TRY(hipMemcpyAsync(dst, src, (size_t)count * 4, hipMemcpyDeviceToHost, s->stream));
-    HIP_TRY(hipStreamSynchronize(s->stream));
-    s->in_flight = false;
-    return LV_OK;
+    if (count != have) return fail(LV_ERR_ARG, "lv_trace_read: buffer %d holds %u floats a row, %u asked", which, have, count);
+    if (s->trace_n == 0) {
+        // nothing recorded yet: the buffers' initial zeros, as before any step
+        memset(dst, 0, (size_t)count * 4);
+        return LV_OK;
+    }
+    return lv_trace_read_rows(s, layer, which, s->trace_n - 1, 1, dst);
 }
 
 #ifdef LV_MEGA_TIMING

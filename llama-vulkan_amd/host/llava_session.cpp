@@ -73,13 +73,22 @@ void llava_layer_session_data::restore_kv_cache(const u8 *src, u32 token_count)
 void llava_layer_session_data::dump_tracing_layers(int out_fd, const std::string &name)
 {
     const u32 dim = session->model->get_header().dim, ff = session->model->get_ff_size(), heads = session->model->get_header().n_heads;
+    // the rows of the last recorded step; before the first one the reference has no trace buffers at all
+    // (llava_layer_session_data.cpp:79) and writes nothing
+    u32 rows = 0;
+    if (lv_trace_rows(session->device_session, &rows) != LV_OK) {
+        std::cerr << "dump_tracing_layers: " << lv_last_error() << std::endl;
+        return;
+    }
+    if (rows == 0) return;
     for (const TraceSlot &slot : kTraceSlots) {
-        // shape as the reference's buffers have it: (values per row, rows); attn_result is (backlog, heads x rows)
+        // shape as the reference's buffers have it: (values per row, rows); attn_result is (backlog, heads x rows).  In
+        // memory both are one row of the step after the other.
         const u32 shape0 = slot.shape == TraceShape::ff ? ff : slot.shape == TraceShape::attn ? session->backlog_size : dim;
-        const u32 shape1 = slot.shape == TraceShape::attn ? heads : 1u;      // the last row of the step
-        const u32 count = shape0 * shape1;
+        const u32 shape1 = slot.shape == TraceShape::attn ? heads * rows : rows;
+        const std::size_t count = static_cast<std::size_t>(shape0) * shape1;
         std::vector<float> values(count);
-        if (lv_trace_read(session->device_session, layer, slot.which, values.data(), count) != LV_OK) {
+        if (lv_trace_read_rows(session->device_session, layer, slot.which, 0, rows, values.data()) != LV_OK) {
             std::cerr << "dump_tracing_layers: " << lv_last_error() << std::endl;
             return;
         }

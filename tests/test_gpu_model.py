@@ -129,9 +129,26 @@ def test_trace_buffers_match_oracle(lva, orc, ctx, tiny_models):
         assert got.shape == want.shape == (128, om.hp["heads"])
         assert np.all(got[5:] == 0.0) and np.all(want[5:] == 0.0)
         assert np.max(np.abs(got - want)) <= 1e-5 and np.allclose(got.sum(axis=0), 1.0, atol=1e-5)
+    # every row of the step is kept (llava_layer_session_data.cpp:80-85): row z is what a step of the first z + 1 tokens leaves
+    assert s.trace_rows() == 5
+    for z in range(5):
+        oz = orc.Session(om, 128)
+        oz.eval(prompt[:z + 1])
+        for layer in range(2):
+            for which in range(6):
+                got, want = s.trace_all(layer, which, z, 1)[0], oz.trace(layer, which)
+                assert got.shape == want.shape
+                assert np.max(np.abs(got - want)) <= 1e-4 * max(1.0, np.max(np.abs(want))), (z, layer, which)
+            a = s.trace_all(layer, lva.TRACE_ATTN, z, 1)[0].reshape(128, -1)
+            assert np.all(a[z + 1:] == 0.0) and np.allclose(a.sum(axis=0), 1.0, atol=1e-5)
+        oz.close()
+    assert np.array_equal(s.trace_all(1, lva.TRACE_FF)[4], s.trace(1, lva.TRACE_FF))
+    with pytest.raises(lva.LvError):
+        s.trace_all(0, lva.TRACE_OUT, 3, 3)                   # rows 3..5 of a step of five
     # one more token: the weights now cover six rows; a larger backlog keeps the layout [backlog][heads]
     tok = orc.greedy(osess.eval([7]))
     s.begin([7], 5); s.wait()
+    assert s.trace_rows() == 1
     s.reserve(256)
     assert np.all(s.trace(0, lva.TRACE_ATTN) == 0.0)          # a fresh buffer of the new size
     s.begin([tok], 6); s.wait()

@@ -260,8 +260,17 @@ def test_save_frame_needs_tracing_and_writes_named_buffers(hl, orc, loaded, tmp_
     assert s.save_frame(frame) == hl.RC_OK
     raw = open(frame, "rb").read()
     om = orc.Model(path)
-    o = orc.Session(om, 128)
-    o.eval(np.array(s.tokens(), dtype=np.uint32))
+    toks = np.array(s.tokens(), dtype=np.uint32)
+    n = len(toks)
+    assert n > 1
+    # the frame holds every row of the step, as the reference's batch-sized buffers do (llava_layer_session_data.cpp:80-85);
+    # the oracle keeps the buffers of the last row it evaluated, so row z comes from a session fed the first z + 1 tokens
+    per_row = []
+    for z in range(n):
+        o = orc.Session(om, 128)
+        o.eval(toks[:z + 1])
+        per_row.append({(layer, w): o.trace(layer, w).copy() for layer in range(2) for w in range(6)})
+        o.close()
     which = {"normalized_input_logit": 0, "post_attn_logit": 1, "post_attn_norm_logit": 2, "ff_result": 3, "output_logit": 4, "attn_result": 5}
     cur, seen = 0, []
     while cur < len(raw):
@@ -272,13 +281,24 @@ def test_save_frame_needs_tracing_and_writes_named_buffers(hl, orc, loaded, tmp_
         vals = np.frombuffer(raw, dtype=np.float32, count=count * rows, offset=cur + head)
         cur += head + 4 * count * rows
         _, layer, slot = name.split(".")
-        # attn_result is (backlog, heads) as in llava_layer_session_data.cpp:80; the vectors are (length, 1 row)
-        assert ftype == 0 and (count, rows) == ((128, om.hp["heads"]) if slot == "attn_result" else (count, 1))
-        want = o.trace(int(layer), which[slot])
-        assert vals.shape == want.shape and np.max(np.abs(vals - want)) <= 1e-4 * max(1.0, np.max(np.abs(want))), name
+        # attn_result is (backlog, heads x rows) as in llava_layer_session_data.cpp:80; the vectors are (length, rows); in
+        # memory both are one row of the step after the other (mhsa.comp:58, z_id * BACKLOG * HEAD_COUNT)
+        assert ftype == 0 and (count, rows) == ((128, om.hp["heads"] * n) if slot == "attn_result" else (count, n))
+        vals = vals.reshape(n, -1)
+        for z in range(n):
+            want = per_row[z][(int(layer), which[slot])]
+            assert vals[z].shape == want.shape and np.max(np.abs(vals[z] - want)) <= 1e-4 * max(1.0, np.max(np.abs(want))), (name, z)
         seen.append(name)
     assert cur == len(raw) and len(seen) == 2 * 6 and seen[:2] == ["layer.0.attn_result", "layer.0.ff_result"]
-    o.close(); om.close()
+    heads = om.hp["heads"]
+    om.close()
+    # the next step is one token long, and so is its frame
+    assert s.push_token(5)
+    s.predict(True)
+    assert s.save_frame(frame) == hl.RC_OK
+    raw = open(frame, "rb").read()
+    count, rows, ftype = struct.unpack_from("<3I", raw, 0)
+    assert (count, rows) == (128, heads)
     assert s.set_options(0) == hl.RC_OK and not s.is_tracing()
     s.close()
 
