@@ -977,6 +977,8 @@ extern "C" int lv_kernel_gemm(lv_ctx *c, float *out, const lv_matrix *w, const f
     HIP_TRY(hipSetDevice(c->device));
     const size_t n_pad = (batch + kGemmTile - 1) / kGemmTile * kGemmTile, halfs = n_pad * gemm_k_padded(w->view.cols);
     if (w->view.cols % 32) return fail(LV_ERR_ARG, "gemm: %u columns", w->view.cols);
+    // the copy made below is freed by lv_matrix_destroy after a wait for the matrix's own context
+    if (!w->h16 && w->ctx != c) return fail(LV_ERR_ARG, "lv_kernel_gemm: the matrix belongs to another context");
     // The matrix's prompt copy is made by the first call and stays with the matrix; the workspace (the two fp16 halves of
     // the activations, their row scales and, where K is cut in slices, the partial results) stays with the context.
     if (!w->h16) {
