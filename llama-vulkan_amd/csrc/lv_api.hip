@@ -133,6 +133,10 @@ using Mega7Bq4 = MegaShape<4096, 11008, 32, 8, 4, 8>;
 using Mega7Bq8 = MegaShape<4096, 11008, 32, 8, 8, 4>;
 using Mega13Bq4 = MegaShape<5120, 13824, 40, 7, 4, 8>;
 using Mega13Bq8 = MegaShape<5120, 13824, 40, 7, 8, 4>;
+// the same for version-1 files (fp32 block scales; the reference loads q4_0 of that version only, llava_buffer.cpp:66-71)
+using Mega7Bq4v1 = MegaShape<4096, 11008, 32, 8, 4, 8, 1>;
+using Mega13Bq4v1 = MegaShape<5120, 13824, 40, 7, 4, 8, 1>;
+constexpr int kMegaKinds = 6;
 
 template <class Fn>
 static int mega_dispatch(int kind, Fn &&fn)
@@ -142,6 +146,8 @@ static int mega_dispatch(int kind, Fn &&fn)
     case 2: return fn(Mega7Bq8{});
     case 3: return fn(Mega13Bq4{});
     case 4: return fn(Mega13Bq8{});
+    case 5: return fn(Mega7Bq4v1{});
+    case 6: return fn(Mega13Bq4v1{});
     default: return fail(LV_ERR_STATE, "no persistent kernel for this model");
     }
 }
@@ -1157,7 +1163,7 @@ static const lv_tensor_desc *find_desc(const lv_tensor_desc *t, uint32_t n, cons
 }
 
 // Persistent-kernel form of the weights: a second copy laid out as per-wave tile streams (lv_mega.h).
-// Built when the model has a compiled shape class, all matrices are q4_0 and the embeddings fp32.
+// Built when the model has a compiled shape class and all matrices have one type and one kind of scale plane.
 template <class S>
 static int build_mega_stream(lv_model *m)
 {
@@ -1199,15 +1205,18 @@ static int build_mega(lv_model *m)
 {
     const lv_hparams &hp = m->hp;
     const uint32_t ft = m->output.ftype;
-    bool uniform = (ft == LV_Q4_0 || ft == LV_Q8_0) && m->output.view.scales != nullptr;   // the tile stream carries fp16 scales
+    // one weight type and one kind of scale plane (fp16, or the fp32 one of a version-1 file) throughout
+    const bool sf32 = m->output.view.scales_f32 != nullptr;
+    bool uniform = ft == LV_Q4_0 || ft == LV_Q8_0;
     for (const LayerWeights &lw : m->layers)
-        for (const lv_matrix *x : {&lw.wq, &lw.wk, &lw.wv, &lw.wo, &lw.w1, &lw.w2, &lw.w3}) uniform = uniform && x->ftype == ft;
+        for (const lv_matrix *x : {&lw.wq, &lw.wk, &lw.wv, &lw.wo, &lw.w1, &lw.w2, &lw.w3})
+            uniform = uniform && x->ftype == ft && (x->view.scales_f32 != nullptr) == sf32;
     if (!uniform || (int)m->ctx->props.multiProcessorCount < kMegaWGs) return LV_OK;
-    for (int kind = 1; kind <= 4; kind++) {
+    for (int kind = 1; kind <= kMegaKinds; kind++) {
         bool fits = false;
         (void)mega_dispatch(kind, [&](auto shape) -> int {
             using S = decltype(shape);
-            fits = hp.dim == (uint32_t)S::D && hp.ff == (uint32_t)S::F && hp.heads == (uint32_t)S::H && ft == (S::QT == 4 ? LV_Q4_0 : LV_Q8_0) &&
+            fits = hp.dim == (uint32_t)S::D && hp.ff == (uint32_t)S::F && hp.heads == (uint32_t)S::H && ft == (S::QT == 4 ? LV_Q4_0 : LV_Q8_0) && S::SF32 == sf32 &&
                    (hp.vocab + kMegaWGs - 1) / kMegaWGs <= (uint32_t)(S::HEAD * S::NRD);
             return LV_OK;
         });

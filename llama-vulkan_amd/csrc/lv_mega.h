@@ -67,12 +67,14 @@ constexpr int cdiv(int a, int b) { return (a + b - 1) / b; }
 constexpr int round_up(int a, int b) { return cdiv(a, b) * b; }
 
 // Static shape of one model class.  NW = wavefronts per workgroup.
-template <int D_, int F_, int H_, int NW_, int QT_, int DEPTH_ = 0>
+// SF32_: the tiles carry fp32 block scales (a version-1 file, llava_buffer.cpp:193-224) instead of fp16 ones.
+template <int D_, int F_, int H_, int NW_, int QT_, int DEPTH_ = 0, int SF32_ = 0>
 struct MegaShape {
     static constexpr int D = D_, F = F_, H = H_, NW = NW_, R = 128;
     static constexpr int QT = QT_;                               // 4: q4_0, 8: q8_0
     static constexpr int CODE = QT == 4 ? 16 : 32;               // bytes of codes per block
-    static constexpr int TILE = 64 * CODE + 128;                 // bytes per tile: 64 blocks of codes, 64 fp16 scales
+    static constexpr bool SF32 = SF32_ != 0;
+    static constexpr int TILE = 64 * CODE + (SF32 ? 256 : 128);  // bytes per tile: 64 blocks of codes, 64 fp16 (or fp32) scales
     static constexpr int DEPTH = DEPTH_ ? DEPTH_ : (QT == 4 ? 4 : 2);   // tiles in flight per wave
     static constexpr int NBD = D / 32, NBF = F / 32;            // blocks per row
     static constexpr int NSD = cdiv(NBD, 64), NSF = cdiv(NBF, 64);  // column slabs
@@ -134,7 +136,8 @@ struct MegaArgs {
 
 struct MegaTile {
     uint4 c, c2;   // c2: second half of the codes of a q8_0 block (unused for q4_0)
-    uint16_t d;
+    uint16_t d;    // fp16 scale bits
+    uint32_t d32;  // fp32 scale bits (shapes with SF32; the other member is unused then, and this one otherwise)
 };
 
 template <class S>
@@ -142,15 +145,19 @@ __device__ __forceinline__ void load_tile(MegaTile &t, const uint8_t *p, int lan
 {
     t.c = *reinterpret_cast<const uint4 *>(p + lane * S::CODE);
     if constexpr (S::QT == 8) t.c2 = *reinterpret_cast<const uint4 *>(p + lane * S::CODE + 16);
-    t.d = *reinterpret_cast<const uint16_t *>(p + 64 * S::CODE + lane * 2);
+    if constexpr (S::SF32) t.d32 = *reinterpret_cast<const uint32_t *>(p + 64 * S::CODE + lane * 4);
+    else t.d = *reinterpret_cast<const uint16_t *>(p + 64 * S::CODE + lane * 2);
 }
 
 // one block column of one row: sum over 32 weights of w * x, from the raw codes
 template <class S>
 __device__ __forceinline__ float tile_dot(const MegaTile &t, const float (&xr)[32], float xsum)
 {
-    if constexpr (S::QT == 4) return (q4_block_dot(t.c, xr) - 8.f * xsum) * half_bits_to_float(t.d);
-    else return (q8_block_dot(t.c, t.c2, xr) - 128.f * xsum) * half_bits_to_float(t.d);
+    float d;
+    if constexpr (S::SF32) d = __uint_as_float(t.d32);
+    else d = half_bits_to_float(t.d);
+    if constexpr (S::QT == 4) return (q4_block_dot(t.c, xr) - 8.f * xsum) * d;
+    else return (q8_block_dot(t.c, t.c2, xr) - 128.f * xsum) * d;
 }
 
 // ---- polling helpers ----------------------------------------------------------------------------------------
@@ -750,6 +757,7 @@ __global__ void mega_pack_kernel(uint8_t *dst /* start of the phase region */, M
     uint8_t *out = dst + tile * S::TILE;
     uint4 codes = make_uint4(0, 0, 0, 0), codes2 = codes;
     uint16_t scale = 0;
+    float scale32 = 0.f;
     const int blk = slab * 64 + lane;
     bool ok = rset < nr && blk < nb;
     const MatView *mv = nullptr;
@@ -779,11 +787,13 @@ __global__ void mega_pack_kernel(uint8_t *dst /* start of the phase region */, M
             codes = mv->codes[2 * sb];
             codes2 = mv->codes[2 * sb + 1];
         }
-        scale = mv->scales[sb];
+        if constexpr (S::SF32) scale32 = mv->scales_f32[sb];
+        else scale = mv->scales[sb];
     }
     *reinterpret_cast<uint4 *>(out + lane * S::CODE) = codes;
     if constexpr (S::QT == 8) *reinterpret_cast<uint4 *>(out + lane * S::CODE + 16) = codes2;
-    *reinterpret_cast<uint16_t *>(out + 64 * S::CODE + lane * 2) = scale;
+    if constexpr (S::SF32) *reinterpret_cast<float *>(out + 64 * S::CODE + lane * 4) = scale32;
+    else *reinterpret_cast<uint16_t *>(out + 64 * S::CODE + lane * 2) = scale;
 }
 
 }  // namespace lv

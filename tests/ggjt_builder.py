@@ -98,8 +98,11 @@ def blocks_to_v1(blocks, ftype):
     return out.reshape(-1)
 
 
-def convert_to_v1(src, dst):
-    """Rewrites a version-3 GGJT file as version 1, tensor by tensor, keeping names, shapes and vocabulary."""
+def convert_to_v1(src, dst, jitter_seed=None):
+    """Rewrites a version-3 GGJT file as version 1, tensor by tensor, keeping names, shapes and vocabulary.  With
+    jitter_seed every block scale is moved by up to 1 %, so that it needs the 24 bits of the fp32 a version-1 block holds
+    (a converted scale alone is an fp16 value)."""
+    rng = np.random.default_rng(jitter_seed) if jitter_seed is not None else None
     data = np.fromfile(src, dtype=np.uint8)
     hdr = np.frombuffer(data[:36].tobytes(), dtype=np.uint32).copy()
     assert hdr[0] == MAGIC and hdr[1] == 3
@@ -119,7 +122,17 @@ def convert_to_v1(src, dst):
         cur = (cur + head_len + 31) & ~31
         size = payload_bytes(ft, n, 3)
         payload = data[cur:cur + size]
-        out += (blocks_to_v1(payload, ft) if ft in (Q4_0, Q8_0) else payload).tobytes()
+        if ft in (Q4_0, Q8_0):
+            v1 = blocks_to_v1(payload, ft)
+            if rng is not None:
+                b = v1.reshape(-1, 20 if ft == Q4_0 else 36)
+                scale = b[:, :4].copy().view(np.float32).reshape(-1)
+                scale *= (1.0 + rng.uniform(-0.01, 0.01, scale.shape)).astype(np.float32)
+                b[:, :4] = scale.view(np.uint8).reshape(-1, 4)
+                v1 = b.reshape(-1)
+            out += v1.tobytes()
+        else:
+            out += payload.tobytes()
         cur += size
     with open(dst, "wb") as f:
         f.write(out)

@@ -135,22 +135,32 @@ def v1_models(lva, tiny_models, tmp_path_factory):
     out["wide_q4"] = str(d / "wide_v1.ggml")
     gb.convert_to_v1(src, out["wide_q4"])
     out["wide_q4_v3"] = src
+    # the same with scales no fp16 holds: what the persistent kernel's fp32-scale tiles are for
+    out["wide_q4_jit"] = str(d / "wide_v1_jit.ggml")
+    gb.convert_to_v1(src, out["wide_q4_jit"], jitter_seed=5)
     return out
 
 
-@pytest.mark.parametrize("name", ["tiny_q4", "tiny_q8", "wide_q4"])
-@pytest.mark.parametrize("graph", [True, False])
-def test_v1_model_greedy_decode_matches_oracle(lva, orc, ctx, v1_models, name, graph):
+@pytest.mark.parametrize("name,mode", [("tiny_q4", "graph"), ("tiny_q4", "operator"), ("tiny_q8", "graph"), ("tiny_q8", "operator"),
+                                       ("wide_q4", "graph"), ("wide_q4", "operator"), ("wide_q4", "persistent"),
+                                       ("wide_q4_jit", "persistent"), ("wide_q4_jit", "graph")])
+def test_v1_model_greedy_decode_matches_oracle(lva, orc, ctx, v1_models, name, mode):
     path = v1_models[name]
     om = orc.Model(path)
     assert om.hp["file_version"] == 1
     osess = orc.Session(om, 128)
     model = lva.Model(ctx, path)
     sess = lva.Session(model, 128)
-    # the persistent kernel reads fp16 scale planes only: a version-1 model runs the operator chain
-    assert sess.path() == lva.PATH_GRAPH
-    assert ctx.lib.lv_session_set_path(sess.h, lva.PATH_PERSISTENT) == -1
-    sess.use_graph(graph)
+    if name.startswith("wide"):
+        # 7B layer widths, q4_0: the persistent kernel has a shape class whose tiles carry the fp32 scales of this version
+        assert sess.path() == lva.PATH_PERSISTENT
+        if mode != "persistent":
+            sess.set_path(lva.PATH_GRAPH if mode == "graph" else lva.PATH_KERNELS)
+    else:
+        assert mode != "persistent" and sess.path() == lva.PATH_GRAPH
+        assert ctx.lib.lv_session_set_path(sess.h, lva.PATH_PERSISTENT) == -1
+    if mode != "persistent":
+        sess.use_graph(mode == "graph")
     vocab = om.hp["vocab"]
     prompt = lva.synth_tokens(8, 3, vocab, seed=0)
     want = osess.eval(prompt)
@@ -166,6 +176,7 @@ def test_v1_model_greedy_decode_matches_oracle(lva, orc, ctx, v1_models, name, g
         got = sess.logits()
         _check_logits(got, want)
         pos += 1
+    assert sess.path() == {"persistent": lva.PATH_PERSISTENT, "graph": lva.PATH_GRAPH, "operator": lva.PATH_KERNELS}[mode]
     sess.close(); model.close(); osess.close(); om.close()
 
 
