@@ -115,6 +115,9 @@ def test_trace_buffers_match_oracle(lva, orc, ctx, tiny_models):
     model = lva.Model(ctx, path)
     s = lva.Session(model, 128)
     s.trace_enable(True)
+    # nothing recorded yet: no rows; the last-row read gives the buffers' initial zeros
+    assert s.trace_rows() == 0 and s.trace_all(0, lva.TRACE_OUT).shape == (0, om.hp["dim"])
+    assert np.all(s.trace(0, lva.TRACE_OUT) == 0.0) and np.all(s.trace(1, lva.TRACE_ATTN) == 0.0)
     prompt = lva.synth_tokens(5, 3, 512, seed=6)
     osess.eval(prompt)
     s.begin(prompt, 0)
