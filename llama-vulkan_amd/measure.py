@@ -5,6 +5,7 @@
     python llama-vulkan_amd/measure.py attention     the one-token attention kernel by itself (7B heads) over 512 and 2048 cache rows
     python llama-vulkan_amd/measure.py decode-q8     7B q8_0, cache positions 1920..2047 (128 greedy steps)
     python llama-vulkan_amd/measure.py decode-q8-graph    the same on the hipGraph of the operator chain (attention_kernel over 2048 rows)
+    python llama-vulkan_amd/measure.py gemv-13b      the same GEMVs at the 13B layer shapes
     python llama-vulkan_amd/measure.py decode-13b    13B q4_0, 32-token prompt + 256 greedy steps (persistent kernel)
     python llama-vulkan_amd/measure.py decode-13b-graph   the same on the hipGraph of the operator chain
     python llama-vulkan_amd/measure.py decode-7b-graph    7B q4_0, positions 444..511 on the hipGraph of the operator chain
@@ -44,11 +45,15 @@ def block_bytes(ftype):
     return 18 if ftype == lva.LV_Q4_0 else 34
 
 
-def gemv_cases(ctx, report=emit):
+GEMV_SHAPES_7B = ((4096, 4096, "store"), (11008, 4096, "silu"), (4096, 11008, "add"), (32000, 4096, "store"))
+GEMV_SHAPES_13B = ((5120, 5120, "store"), (13824, 5120, "silu"), (5120, 13824, "add"), (32000, 5120, "store"))
+
+
+def gemv_cases(ctx, report=emit, shapes=GEMV_SHAPES_7B):
     """reference: matmul.glsl / matmul_q8.glsl / matmul_silu_ff.comp at the three layer shapes and the output matrix"""
     out_cases = []
     for ftype, tname in ((lva.LV_Q4_0, "q4_0"), (lva.LV_Q8_0, "q8_0")):
-        for rows, cols, mode in ((4096, 4096, "store"), (11008, 4096, "silu"), (4096, 11008, "add"), (32000, 4096, "store")):
+        for rows, cols, mode in shapes:
             nbytes = rows * cols // 32 * block_bytes(ftype) * (2 if mode == "silu" else 1) + 4 * cols + 4 * rows * (2 if mode == "add" else 1)
             # enough distinct matrices that the working set exceeds the 256 MB last-level cache
             nmat = max(2, min(12, int(1.5e9 // nbytes)))
@@ -455,6 +460,8 @@ def main():
         copy_case(ctx)
     if which in ("gemv", "all"):
         gemv_cases(ctx)
+    if which == "gemv-13b":
+        gemv_cases(ctx, shapes=GEMV_SHAPES_13B)
     if which in ("attention", "all"):
         attention_cases(ctx)
     if which == "attention-batch":
