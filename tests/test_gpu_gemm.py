@@ -117,6 +117,21 @@ def test_gemm_calls_in_a_row_keep_their_workspace(lva, orc, ctx):
         ctx.free(dout)
 
 
+def test_gemm_refuses_a_matrix_of_another_context(lva, ctx):
+    """the prompt copy lv_kernel_gemm makes is freed with the matrix after a wait for the matrix's context: a launch queued
+    on another context's stream could outlive it, so that call is refused"""
+    other = lva.Context(0)
+    blocks = lva.synth_quant(lva.LV_Q8_0, 128, 128, seed=3)
+    m = ctx.matrix(blocks, lva.LV_Q8_0, 128, 128)
+    dx, dout = other.to_device(lva.synth_normal(16, 128, seed=4)), other.alloc(16 * 128 * 4)
+    with pytest.raises(lva.LvError) as err:
+        lva.check(other.lib.lv_kernel_gemm(other.h, dout, m, dx, 16, 0))
+    assert err.value.code == -1 and "another context" in str(err.value)       # LV_ERR_ARG
+    other.free(dx); other.free(dout)
+    ctx.matrix_free(m)
+    other.close()
+
+
 @pytest.mark.parametrize("name,n_prompt", [("tiny_q4", 40), ("tiny_q8", 130), ("small_q4", 77), ("pair_q4", 150), ("pair_q8", 33)])
 def test_prompt_as_one_batch_matches_oracle(lva, orc, ctx, tiny_models, name, n_prompt):
     path = tiny_models[name]
