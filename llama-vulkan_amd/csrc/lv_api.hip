@@ -134,8 +134,8 @@ using Mega7Bq8 = MegaShape<4096, 11008, 32, 8, 8, 4>;
 using Mega13Bq4 = MegaShape<5120, 13824, 40, 7, 4, 8>;
 using Mega13Bq8 = MegaShape<5120, 13824, 40, 7, 8, 4>;
 // the same for version-1 files (fp32 block scales; the reference loads q4_0 of that version only, llava_buffer.cpp:66-71)
-using Mega7Bq4v1 = MegaShape<4096, 11008, 32, 8, 4, 8, 1>;
-using Mega13Bq4v1 = MegaShape<5120, 13824, 40, 7, 4, 8, 1>;
+using Mega7Bq4v1 = MegaShapeV1<4096, 11008, 32, 8, 4, 8>;
+using Mega13Bq4v1 = MegaShapeV1<5120, 13824, 40, 7, 4, 8>;
 constexpr int kMegaKinds = 6;
 
 template <class Fn>

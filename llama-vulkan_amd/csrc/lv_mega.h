@@ -68,12 +68,12 @@ constexpr int round_up(int a, int b) { return cdiv(a, b) * b; }
 
 // Static shape of one model class.  NW = wavefronts per workgroup.
 // SF32_: the tiles carry fp32 block scales (a version-1 file, llava_buffer.cpp:193-224) instead of fp16 ones.
-template <int D_, int F_, int H_, int NW_, int QT_, int DEPTH_ = 0, int SF32_ = 0>
-struct MegaShape {
+template <int D_, int F_, int H_, int NW_, int QT_, int DEPTH_, bool SF32_>
+struct MegaShapeBase {
     static constexpr int D = D_, F = F_, H = H_, NW = NW_, R = 128;
     static constexpr int QT = QT_;                               // 4: q4_0, 8: q8_0
     static constexpr int CODE = QT == 4 ? 16 : 32;               // bytes of codes per block
-    static constexpr bool SF32 = SF32_ != 0;
+    static constexpr bool SF32 = SF32_;
     static constexpr int TILE = 64 * CODE + (SF32 ? 256 : 128);  // bytes per tile: 64 blocks of codes, 64 fp16 (or fp32) scales
     static constexpr int DEPTH = DEPTH_ ? DEPTH_ : (QT == 4 ? 4 : 2);   // tiles in flight per wave
     static constexpr int NBD = D / 32, NBF = F / 32;            // blocks per row
@@ -98,6 +98,11 @@ struct MegaShape {
     static constexpr size_t LAYER_BYTES = PHASE_A_BYTES + PHASE_C_BYTES + PHASE_D_BYTES + PHASE_E_BYTES;
     static constexpr size_t HEAD_BYTES = (size_t)kMegaWGs * NW * HEAD * TILE;
 };
+// the shape classes the kernel is instantiated for: fp16 block scales (file version 3), fp32 ones (version 1)
+template <int D_, int F_, int H_, int NW_, int QT_, int DEPTH_ = 0>
+struct MegaShape : MegaShapeBase<D_, F_, H_, NW_, QT_, DEPTH_, false> {};
+template <int D_, int F_, int H_, int NW_, int QT_, int DEPTH_ = 0>
+struct MegaShapeV1 : MegaShapeBase<D_, F_, H_, NW_, QT_, DEPTH_, true> {};
 
 struct MegaArgs {
     const uint8_t *wstream;    // [layers] x LAYER_BYTES, then HEAD_BYTES, then one all-zero tile
