@@ -83,6 +83,7 @@ struct lv_ctx {
     // for each other.  A launch on another session's stream first waits for the event the last launch recorded.
     std::mutex mega_mutex;
     hipEvent_t mega_done = nullptr;
+    int xcd_local = -1;                   // 1: workgroup b of a 256-workgroup launch runs on XCD b % 8 (probed once); 0: not; -1: not probed
     const void *mega_last = nullptr;      // session whose launch mega_done belongs to
 };
 
@@ -192,6 +193,7 @@ struct lv_session {
     bool mega_step = false;               // the step in flight ran the persistent kernel
     int mega_failures = 0;                // steps of the persistent kernel in a row that ended with an expired wait
     bool mega_off = false;                // the persistent kernel is no longer used by this session (refused launch, or two such steps)
+    bool xcd_local_off = false;           // a launch found a workgroup on another XCD than the probe had: device-scope hand-overs from then on
     bool in_flight = false;
     bool have_logits = false;
     bool trace = false;
@@ -1201,6 +1203,26 @@ static int build_mega_stream(lv_model *m)
     return LV_OK;
 }
 
+// Does this device place workgroup b of a launch on XCD b % 8?  The persistent kernel then keeps the hand-overs between the
+// workgroups of a head inside that XCD's L2 (lv_mega.h: ld_xcd).  One small launch; the kernel checks again for itself.
+static int probe_xcd_placement(lv_ctx *c)
+{
+    if (c->xcd_local >= 0) return LV_OK;
+    uint32_t *dev = nullptr;
+    std::vector<uint32_t> host(kMegaWGs, 0xffu);
+    HIP_TRY(hipMalloc(reinterpret_cast<void **>(&dev), kMegaWGs * 4));
+    xcd_probe_kernel<<<dim3(kMegaWGs), dim3(64), 0, c->stream>>>(dev);
+    hipError_t e = hipGetLastError();
+    if (e == hipSuccess) e = hipMemcpyAsync(host.data(), dev, kMegaWGs * 4, hipMemcpyDeviceToHost, c->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
+    (void)hipFree(dev);
+    HIP_TRY(e);
+    bool ok = true;
+    for (int b = 0; b < kMegaWGs; b++) ok = ok && host[b] == (uint32_t)(b & 7);
+    c->xcd_local = ok ? 1 : 0;
+    return LV_OK;
+}
+
 static int build_mega(lv_model *m)
 {
     const lv_hparams &hp = m->hp;
@@ -1221,6 +1243,7 @@ static int build_mega(lv_model *m)
             return LV_OK;
         });
         if (!fits) continue;
+        LV_TRY(probe_xcd_placement(m->ctx));
         LV_TRY(mega_dispatch(kind, [&](auto shape) { return build_mega_stream<decltype(shape)>(m); }));
         if (m->tok_ftype != LV_F32) {
             // llava_buffer.cpp:339-401 dequantises the token's row on the host at every step; here the whole table is
@@ -1630,6 +1653,7 @@ static int launch_mega(lv_session *s, uint32_t pos, uint32_t token, bool *refuse
     a.status = s->status_host;
     a.layers = m->hp.layers; a.vocab = m->hp.vocab; a.backlog = s->backlog; a.pos = pos; a.token = token;
     a.spin_limit = s->wait_limit ? s->wait_limit : kSpinLimit;
+    a.xcd_local = m->ctx->xcd_local == 1 && !s->xcd_local_off;
     s->xchg_turn++;
     void *params[] = {&a};
     lv_ctx *c = m->ctx;
@@ -2034,7 +2058,12 @@ extern "C" int lv_step_wait(lv_session *s)
     const bool mega_step = s->mega_step;
     s->mega_step = false;
     if (s->status_host && *s->status_host) {
+        const bool misplaced = *s->status_host == 2u;
         *s->status_host = 0;
+        if (misplaced) {
+            s->xcd_local_off = true;
+            return fail(LV_ERR_HIP, "persistent decode kernel: a workgroup ran on another XCD than expected; this session now hands over at device scope");
+        }
         if (++s->mega_failures >= 2) {
             s->mega_off = true;
             return fail(LV_ERR_HIP, "persistent decode kernel: a hand-over wait expired in two steps in a row; this session now takes the %s path",

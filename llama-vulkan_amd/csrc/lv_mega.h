@@ -54,6 +54,41 @@ __device__ __forceinline__ void st_dev(float *p, float v)
     __hip_atomic_store(reinterpret_cast<uint32_t *>(p), __float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// Hand-overs inside one XCD.  The workgroups of a launch go to the XCDs in turn (workgroup b runs on XCD b % 8), and the
+// CUs of an XCD share its L2.  A plain store is written through the CU's cache into that L2, and a non-temporal load
+// does not stop at the CU's cache, so a value stored by one workgroup is seen by another one of the same XCD after one
+// L2 round trip: 0.5 us for a flag bounced between two such workgroups, against 1.1 us with the device-scope pair above,
+// whose store has to reach memory (measured; a load with only sc0 set keeps hitting the CU's own cache and never sees
+// the store).  Across XCDs only the device-scope pair works.
+__device__ __forceinline__ uint32_t ld_xcd(const uint32_t *p) { return __builtin_nontemporal_load(p); }
+
+// Where a workgroup stands in the attention phase: XCD b % 8 holds H / 8 heads, for each of them the CPH workgroups that
+// take a chunk of the cache each; chunk 0 also combines the chunks.  The same XCD computes the query, key and value rows
+// of its heads in phase A, so these two hand-overs stay inside the XCD.
+template <class S>
+struct MegaPlace {
+    int xcd, slot, h, c;
+    bool attends;
+    __device__ __forceinline__ explicit MegaPlace(int b)
+    {
+        static_assert(S::H % 8 == 0 && (S::H / 8) * S::CPH <= kMegaWGs / 8, "heads must split over eight XCDs");
+        xcd = b & 7; slot = b >> 3;
+        const int hl = slot / S::CPH;
+        c = slot % S::CPH;
+        attends = hl < S::H / 8;
+        h = hl * 8 + xcd;
+    }
+};
+// row t of workgroup b in phase A: which of q, k, v (0..2) and which of its D rows
+template <class S>
+__host__ __device__ __forceinline__ void mega_qkv_row(int b, int t, int &which, int &row)
+{
+    const int lr = (b >> 3) * S::ROWS_A + t;            // among the 3 R H / 8 rows of the XCD's heads
+    const int hl = lr / (3 * S::R), within = lr % (3 * S::R);
+    which = within / S::R;
+    row = (hl * 8 + (b & 7)) * S::R + within % S::R;
+}
+
 // Workgroup barrier that orders LDS traffic only: global loads of the weight queue stay in flight across it
 // (__syncthreads would wait for vmcnt(0) and drain the queue at every phase step).
 __device__ __forceinline__ void lds_barrier()
@@ -116,6 +151,8 @@ struct MegaArgs {
     uint32_t *status;          // host-visible; [0] set non-zero when a poll loop expired, [kStatusToken] = greedy pick
     uint32_t layers, vocab, backlog, pos, token;
     uint32_t spin_limit;       // polls per hand-over before the step is given up (kSpinLimit; tests of the failure path lower it)
+    uint32_t xcd_local;        // non-zero: workgroup b is known to run on XCD b % 8, so the hand-overs between the workgroups of
+                               // a head go through that XCD's L2 (ld_xcd); zero: device scope everywhere
 };
 
 // Optional phase timestamps (built only with -DLV_MEGA_TIMING): workgroup 0 records the 100 MHz wall clock at
@@ -167,7 +204,7 @@ __device__ __forceinline__ float tile_dot(const MegaTile &t, const float (&xr)[3
 
 // ---- polling helpers ----------------------------------------------------------------------------------------
 // N values strided by `stride` elements starting at p; spins until none of them is the not-ready pattern.
-template <int N, int SLEEP = 0>
+template <int N, int SLEEP = 0, bool XCD = false>
 __device__ __forceinline__ void poll_values(float (&v)[N], const float *p, int stride, const bool (&want)[N], uint32_t *status,
                                             uint32_t spin_limit, int group_stride = 0 /* when non-zero: element j lives at p[(j/8)*8*group_stride + j%8] */)
 {
@@ -176,11 +213,12 @@ __device__ __forceinline__ void poll_values(float (&v)[N], const float *p, int s
     if constexpr (SLEEP > 0) __builtin_amdgcn_s_sleep(SLEEP);
     do {
         pending = false;
+        if constexpr (XCD) asm volatile("" ::: "memory");      // the loads below are ordinary ones: every turn has to issue them again
 #pragma unroll
         for (int j = 0; j < N; j++) {
             uint32_t u = 0;
             const size_t off = group_stride ? (size_t)(j / 8) * 8 * group_stride + (j % 8) : (size_t)j * stride;
-            if (want[j]) u = ld_dev(reinterpret_cast<const uint32_t *>(p) + off);
+            if (want[j]) u = XCD ? ld_xcd(reinterpret_cast<const uint32_t *>(p) + off) : ld_dev(reinterpret_cast<const uint32_t *>(p) + off);
             v[j] = __uint_as_float(u);
             pending |= (u == kNotReady);
         }
@@ -398,6 +436,14 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
     const int st = threadIdx.x;
     uint32_t *status = a.status;
     const uint32_t spin_limit = a.spin_limit;
+    const MegaPlace<S> place(b);
+    const bool xcd_local = a.xcd_local != 0;
+    if (xcd_local && threadIdx.x == 0) {
+        // the hand-overs through an XCD's L2 rest on this placement; a launch that does not have it gives the step up
+        uint32_t xcc;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+        if ((int)(xcc & 0xf) != place.xcd) *status = 2u;
+    }
 
     // ---- start the weight stream ------------------------------------------------------------------------------
     MegaTile q[S::DEPTH];
@@ -433,22 +479,25 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
         lds_barrier();
         if (threadIdx.x < S::ROWS_A) {
             const float v = red_row<S::NSD>(red, threadIdx.x) * inv_a;
-            const int g = b * S::ROWS_A + threadIdx.x, which = g / D, col = g % D;
-            if (which == 0) {
-                st_dev(xc + S::OFF_QKV + col, v);
-            } else {
+            int which, col;
+            mega_qkv_row<S>(b, threadIdx.x, which, col);
+            float out = v;
+            if (which != 0) {
                 // copy_to_cache.comp:35: the cache keeps fp16; attention of this very step reads the rounded value too
                 const uint16_t hbits = float_to_half_bits(v);
                 (which == 1 ? kc : vc)[(size_t)pos * D + col] = hbits;
-                st_dev(xc + S::OFF_QKV + which * D + col, half_bits_to_float(hbits));
+                out = half_bits_to_float(hbits);
             }
+            // read by the chunk workgroups of the row's head, which run on this XCD
+            if (xcd_local) xc[S::OFF_QKV + which * D + col] = out;
+            else st_dev(xc + S::OFF_QKV + which * D + col, out);
         }
 
         // ================= B: attention chunk (head h, chunk c) ================================================
         MEGA_STAMP(2);
         {
-            const int h = b / S::CPH, c = b % S::CPH;
-            if (h < H) {
+            const int h = place.h, c = place.c;
+            if (place.attends) {
                 const uint32_t n_valid = pos + 1;
                 uint32_t chunk = (n_valid + S::CPH - 1) / S::CPH;
                 chunk = (chunk + 3) & ~3u;
@@ -490,7 +539,8 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
                 if (w < 3 && (w == 0 || holds_new)) {
                     float pv[2];
                     const bool want2[2] = {true, true};
-                    poll_values<2, 0>(pv, xc + S::OFF_QKV + w * D + h * R + lane * 2, 1, want2, status, spin_limit);
+                    if (xcd_local) poll_values<2, 0, true>(pv, xc + S::OFF_QKV + w * D + h * R + lane * 2, 1, want2, status, spin_limit);
+                    else poll_values<2, 0>(pv, xc + S::OFF_QKV + w * D + h * R + lane * 2, 1, want2, status, spin_limit);
                     l.qkv[w * R + lane * 2] = pv[0];
                     l.qkv[w * R + lane * 2 + 1] = pv[1];
                 }
@@ -574,27 +624,27 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
                     float t = 0.f;
 #pragma unroll
                     for (int i = 0; i < NW; i++) t += l.attn_red[i * (R + 1) + st];
-                    st_dev(xc + S::OFF_PART + (h * S::CPH + c) * S::PART + st, t);
+                    // read by chunk 0 of this head, on this XCD
+                    if (xcd_local) xc[S::OFF_PART + (h * S::CPH + c) * S::PART + st] = t;
+                    else st_dev(xc + S::OFF_PART + (h * S::CPH + c) * S::PART + st, t);
                 }
             }
         }
 
         // ================= B': combine the chunks of head b (one wait for numerators and denominators) ==========
         MEGA_STAMP(4);
-        if (b < H && st < R) {
+        if (place.attends && place.c == 0 && st < R) {
             float nd[2 * S::CPH];
-            bool want[2 * S::CPH];
-#pragma unroll
-            for (int c = 0; c < 2 * S::CPH; c++) want[c] = true;
-            const float *hp = xc + S::OFF_PART + (size_t)b * S::CPH * S::PART;
+            const uint32_t *hp = reinterpret_cast<const uint32_t *>(xc + S::OFF_PART + (size_t)place.h * S::CPH * S::PART);
             uint32_t spins = 0;
             bool pending;
             do {
                 pending = false;
+                if (xcd_local) asm volatile("" ::: "memory");      // ordinary loads: every turn has to issue them again
 #pragma unroll
                 for (int c = 0; c < S::CPH; c++) {
-                    const uint32_t un = ld_dev(reinterpret_cast<const uint32_t *>(hp + c * S::PART + st));
-                    const uint32_t ud = ld_dev(reinterpret_cast<const uint32_t *>(hp + c * S::PART + R));
+                    const uint32_t un = xcd_local ? ld_xcd(hp + c * S::PART + st) : ld_dev(hp + c * S::PART + st);
+                    const uint32_t ud = xcd_local ? ld_xcd(hp + c * S::PART + R) : ld_dev(hp + c * S::PART + R);
                     nd[c] = __uint_as_float(un);
                     nd[S::CPH + c] = __uint_as_float(ud);
                     pending |= (un == kNotReady) | (ud == kNotReady);
@@ -604,7 +654,7 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
             float n = 0.f, d = 0.f;
 #pragma unroll
             for (int c = 0; c < S::CPH; c++) { n += nd[c]; d += nd[S::CPH + c]; }
-            st_dev(xc + S::OFF_O + b * R + st, n / d);
+            st_dev(xc + S::OFF_O + place.h * R + st, n / d);       // every workgroup of the device reads this one
         }
 
         // ================= C: x += Wo o ============================================================================
@@ -779,7 +829,12 @@ __global__ void mega_pack_kernel(uint8_t *dst /* start of the phase region */, M
             const int j = rset * tiles + i;
             ok = j < rows;
             const int g = b * rows + j;
-            if (phase == 0) { mv = &src.m[g / S::D]; row = g % S::D; }
+            if (phase == 0) {
+                int which = 0, r = 0;
+                if (ok) mega_qkv_row<S>(b, j, which, r);
+                mv = &src.m[which];
+                row = r;
+            }
             else if (phase == 2) { mv = &src.m[g & 1]; row = g >> 1; }
             else { mv = &src.m[0]; row = g; }
         }
@@ -799,6 +854,16 @@ __global__ void mega_pack_kernel(uint8_t *dst /* start of the phase region */, M
     if constexpr (S::QT == 8) *reinterpret_cast<uint4 *>(out + lane * S::CODE + 16) = codes2;
     if constexpr (S::SF32) *reinterpret_cast<float *>(out + 64 * S::CODE + lane * 4) = scale32;
     else *reinterpret_cast<uint16_t *>(out + 64 * S::CODE + lane * 2) = scale;
+}
+
+// Which XCD each workgroup of a 256-workgroup launch runs on (MegaArgs::xcd_local is set only when it is b % 8).
+__global__ void xcd_probe_kernel(uint32_t *out)
+{
+    if (threadIdx.x == 0) {
+        uint32_t xcc;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+        out[blockIdx.x] = xcc & 0xf;
+    }
 }
 
 }  // namespace lv
