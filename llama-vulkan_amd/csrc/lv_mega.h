@@ -114,6 +114,9 @@ struct MegaShapeBase {
     static constexpr int NBD = D / 32, NBF = F / 32;            // blocks per row
     static constexpr int NSD = cdiv(NBD, 64), NSF = cdiv(NBF, 64);  // column slabs
     static constexpr int NRD = NW / NSD, NRF = NW / NSF;        // row sets (waves sharing a slab split the rows)
+    // phase E: every wave of the workgroup owns exactly one column slab; each then fetches its own part of the input vector
+    // (acquire_own_slab).  Where waves are left over (7B: six slabs, eight waves) the common fetch by all threads is as fast.
+    static constexpr bool OWN_SLAB_E = NRF == 1 && NSF == NW;
     static constexpr int ROWS_A = 3 * D / kMegaWGs, ROWS_C = D / kMegaWGs, ROWS_D = 2 * F / kMegaWGs, ROWS_E = D / kMegaWGs;
     static constexpr int TA = cdiv(ROWS_A, NRD), TC = cdiv(ROWS_C, NRD), TD = cdiv(ROWS_D, NRD), TE = cdiv(ROWS_E, NRF);
     static constexpr int SEQ_A = 0, SEQ_C = TA, SEQ_D = TA + TC, SEQ_E = TA + TC + TD;
@@ -421,6 +424,43 @@ __device__ __forceinline__ float acquire_vector(float *xs, const float *src, con
     return inv;
 }
 
+// Phase E, where every working wave owns one column slab (S::NRF == 1): a wave fetches the 2048 floats of its own slab and
+// nothing else, 16 bytes a lane and load, at device scope; it starts on its tiles when the producers of that slab have
+// stored, without a workgroup barrier, and the workgroup no longer moves the whole F-float vector with every thread.
+// The slab passes through the wave's own part of LDS to reach the block-per-lane order of load_slab.
+typedef uint32_t mega_u4v __attribute__((ext_vector_type(4)));
+template <class S, int SLEEP>
+__device__ __forceinline__ void acquire_own_slab(float (&xr)[32], float &xsum, float *xs, const float *src, int slab, int lane, bool active,
+                                                 bool lane_has, uint32_t *status, uint32_t spin_limit)
+{
+    static_assert(S::NRF == 1 && S::F % 4 == 0, "one wave per slab");
+    if (active) {
+        // loads past the end of the vector return zero (the last slab is not full)
+        const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(src), 0, S::F * 4, 0x00020000);
+        const int base = slab * 2048;
+        mega_u4v v[8];
+        uint32_t spins = 0;
+        bool pending;
+        if constexpr (SLEEP > 0) __builtin_amdgcn_s_sleep(SLEEP);
+        do {
+            pending = false;
+            asm volatile("" ::: "memory");      // every turn issues the loads again
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                v[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (base + (j * 64 + lane) * 4) * 4, 0, 16 /* sc1: device scope */);
+                pending |= (v[j].x == kNotReady) | (v[j].y == kNotReady) | (v[j].z == kNotReady) | (v[j].w == kNotReady);
+            }
+        } while (pending && ++spins < spin_limit);
+        if (pending) *status = 1u;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int idx = base + (j * 64 + lane) * 4;
+            if (idx < S::F) *reinterpret_cast<mega_u4v *>(xs + xs_index(idx)) = v[j];
+        }
+    }
+    load_slab(xr, xsum, xs, slab * 64 + lane, active && lane_has);
+}
+
 template <class S>
 __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
 {
@@ -685,9 +725,14 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
 
         // ================= E: x += W2 ff ===========================================================================
         MEGA_STAMP(9);
-        acquire_vector<F, NW, false, kPollDelay>(xs, xc + S::OFF_FF, nullptr, scratch, status, spin_limit);
-        MEGA_STAMP(10);
-        load_slab(xr, xsum, xs, mw.sF * 64 + lane, mw.laneF);
+        if constexpr (S::OWN_SLAB_E) {
+            acquire_own_slab<S, kPollDelay>(xr, xsum, xs, xc + S::OFF_FF, mw.sF, lane, mw.actF, mw.laneF, status, spin_limit);
+            MEGA_STAMP(10);
+        } else {
+            acquire_vector<F, NW, false, kPollDelay>(xs, xc + S::OFF_FF, nullptr, scratch, status, spin_limit);
+            MEGA_STAMP(10);
+            load_slab(xr, xsum, xs, mw.sF * 64 + lane, mw.laneF);
+        }
         gemv_phase<S, S::SEQ_E, S::TE, S::NSF>(q, mw, layer, xr, xsum, mw.sF, mw.rF, mw.actF, S::ROWS_E, red);
         // padding slots of the layer's sequence carry no tile, but the slot S::DEPTH ahead of them does
 #pragma unroll
