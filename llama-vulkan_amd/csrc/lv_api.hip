@@ -83,7 +83,6 @@ struct lv_ctx {
     // for each other.  A launch on another session's stream first waits for the event the last launch recorded.
     std::mutex mega_mutex;
     hipEvent_t mega_done = nullptr;
-    int xcd_local = -1;                   // 1: workgroup b of a 256-workgroup launch runs on XCD b % 8 (probed once); 0: not; -1: not probed
     const void *mega_last = nullptr;      // session whose launch mega_done belongs to
 };
 
@@ -96,6 +95,40 @@ struct lv_matrix {
     mutable const uint16_t *h16 = nullptr;   // prompt copy (lv_gemm.h): codes as fp16 integers and fp32 scales in tile order; null until a batch needs it
     mutable uint16_t *h16_owned = nullptr;   // that copy when lv_kernel_gemm made it for a matrix outside a model; freed with the matrix
 };
+
+// Uncached device memory (hipDeviceMallocUncached) for the persistent kernel's device-wide hand-over vectors.  Such memory
+// is never given back to the runtime once a kernel has read it (allocations made after such a free have been seen to hold
+// wrong values); a session that ends leaves its buffers here for the next one of the same size.
+struct UncachedBlock { int device; size_t bytes; void *ptr; };
+static std::mutex g_uncached_mutex;
+static std::vector<UncachedBlock> g_uncached_free;
+
+static int uncached_take(int device, void **out, size_t bytes)
+{
+    {
+        std::lock_guard<std::mutex> lock(g_uncached_mutex);
+        for (size_t i = 0; i < g_uncached_free.size(); i++)
+            if (g_uncached_free[i].device == device && g_uncached_free[i].bytes == bytes) {
+                *out = g_uncached_free[i].ptr;
+                g_uncached_free.erase(g_uncached_free.begin() + (long)i);
+                return LV_OK;
+            }
+    }
+    hipError_t e = hipExtMallocWithFlags(out, bytes, hipDeviceMallocUncached);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        *out = nullptr;
+        return fail(e == hipErrorOutOfMemory ? LV_ERR_OOM : LV_ERR_HIP, "uncached hand-over buffer of %llu bytes: %s", (unsigned long long)bytes, hipGetErrorString(e));
+    }
+    return LV_OK;
+}
+
+static void uncached_give(int device, void *ptr, size_t bytes)
+{
+    if (!ptr) return;
+    std::lock_guard<std::mutex> lock(g_uncached_mutex);
+    g_uncached_free.push_back({device, bytes, ptr});
+}
 
 struct LayerWeights {
     lv_matrix wq, wk, wv, wo, w1, w2, w3;
@@ -185,7 +218,9 @@ struct lv_session {
     // operand planes of the batched attention (one layer's worth, rewritten per layer): four of attn_plane_halfs() each
     uint16_t *pf_planes = nullptr;
     size_t pf_plane_halfs = 0;
-    float *xchg[2] = {nullptr, nullptr};  // hand-over buffer sets of the persistent kernel
+    float *xchg[2] = {nullptr, nullptr};  // hand-over buffer sets of the persistent kernel: uncached memory (uncached_take / uncached_give) ...
+    size_t xchg_bytes = 0;
+    float *xl[2] = {nullptr, nullptr};    // ... and the part of them that stays inside an XCD, ordinary memory
     uint32_t xchg_turn = 0;
     uint32_t *status_host = nullptr;      // pinned, written by the persistent kernel: [0] a poll expired, [kStatusToken] greedy pick
     uint32_t wait_limit = 0;              // polls per hand-over of the persistent kernel; 0 = default
@@ -193,7 +228,6 @@ struct lv_session {
     bool mega_step = false;               // the step in flight ran the persistent kernel
     int mega_failures = 0;                // steps of the persistent kernel in a row that ended with an expired wait
     bool mega_off = false;                // the persistent kernel is no longer used by this session (refused launch, or two such steps)
-    bool xcd_local_off = false;           // a launch found a workgroup on another XCD than the probe had: device-scope hand-overs from then on
     bool in_flight = false;
     bool have_logits = false;
     bool trace = false;
@@ -1203,26 +1237,6 @@ static int build_mega_stream(lv_model *m)
     return LV_OK;
 }
 
-// Does this device place workgroup b of a launch on XCD b % 8?  The persistent kernel then keeps the hand-overs between the
-// workgroups of a head inside that XCD's L2 (lv_mega.h: ld_xcd).  One small launch; the kernel checks again for itself.
-static int probe_xcd_placement(lv_ctx *c)
-{
-    if (c->xcd_local >= 0) return LV_OK;
-    uint32_t *dev = nullptr;
-    std::vector<uint32_t> host(kMegaWGs, 0xffu);
-    HIP_TRY(hipMalloc(reinterpret_cast<void **>(&dev), kMegaWGs * 4));
-    xcd_probe_kernel<<<dim3(kMegaWGs), dim3(64), 0, c->stream>>>(dev);
-    hipError_t e = hipGetLastError();
-    if (e == hipSuccess) e = hipMemcpyAsync(host.data(), dev, kMegaWGs * 4, hipMemcpyDeviceToHost, c->stream);
-    if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
-    (void)hipFree(dev);
-    HIP_TRY(e);
-    bool ok = true;
-    for (int b = 0; b < kMegaWGs; b++) ok = ok && host[b] == (uint32_t)(b & 7);
-    c->xcd_local = ok ? 1 : 0;
-    return LV_OK;
-}
-
 static int build_mega(lv_model *m)
 {
     const lv_hparams &hp = m->hp;
@@ -1243,7 +1257,6 @@ static int build_mega(lv_model *m)
             return LV_OK;
         });
         if (!fits) continue;
-        LV_TRY(probe_xcd_placement(m->ctx));
         LV_TRY(mega_dispatch(kind, [&](auto shape) { return build_mega_stream<decltype(shape)>(m); }));
         if (m->tok_ftype != LV_F32) {
             // llava_buffer.cpp:339-401 dequantises the token's row on the host at every step; here the whole table is
@@ -1439,8 +1452,10 @@ extern "C" int lv_session_destroy(lv_session *s)
                    s->cfg, s->argmax_dev, s->trace_buf, s->trace_attn, s->pf_x, s->pf_xn, s->pf_q, s->pf_k, s->pf_v, s->pf_vo, s->pf_g1, s->pf_g2,
                    s->pf_xh, s->pf_xl, s->pf_xs, s->pf_planes, s->pf_fh, s->pf_fl};
     for (void *p : dev) (void)hipFree(p);
-    (void)hipFree(s->xchg[0]);
-    (void)hipFree(s->xchg[1]);
+    for (int i = 0; i < 2; i++) {
+        uncached_give(s->model->ctx->device, s->xchg[i], s->xchg_bytes);
+        (void)hipFree(s->xl[i]);
+    }
     if (s->status_host) (void)hipHostFree(s->status_host);
     if (s->cfg_host) (void)hipHostFree(s->cfg_host);
     if (s->argmax_host) (void)hipHostFree(s->argmax_host);
@@ -1469,14 +1484,18 @@ static int session_alloc(lv_session *s)
     HIP_TRY(hipHostMalloc(reinterpret_cast<void **>(&s->cfg_host), (1 + kMaxStepTokens) * 4, hipHostMallocDefault));
     HIP_TRY(hipHostMalloc(reinterpret_cast<void **>(&s->argmax_host), 4, hipHostMallocDefault));
     if (s->model->mega_kind) {
-        size_t bytes = 0;
+        size_t bytes = 0, local_bytes = 0;
         LV_TRY(mega_dispatch(s->model->mega_kind, [&](auto shape) -> int {
             bytes = ((size_t)hp.layers * decltype(shape)::XCHG_LAYER + decltype(shape)::XCHG_TAIL) * 4;
+            local_bytes = (size_t)hp.layers * decltype(shape)::LOCAL_LAYER * 4;
             return LV_OK;
         }));
+        s->xchg_bytes = bytes;
         for (int i = 0; i < 2; i++) {
-            HIP_TRY(hipMalloc(reinterpret_cast<void **>(&s->xchg[i]), bytes));
+            LV_TRY(uncached_take(s->model->ctx->device, reinterpret_cast<void **>(&s->xchg[i]), bytes));
             HIP_TRY(hipMemsetAsync(s->xchg[i], 0xff, bytes, s->stream));
+            HIP_TRY(hipMalloc(reinterpret_cast<void **>(&s->xl[i]), local_bytes));
+            HIP_TRY(hipMemsetAsync(s->xl[i], 0xff, local_bytes, s->stream));
         }
         HIP_TRY(hipHostMalloc(reinterpret_cast<void **>(&s->status_host), 4096, hipHostMallocDefault));
         memset(s->status_host, 0, 4096);
@@ -1649,11 +1668,13 @@ static int launch_mega(lv_session *s, uint32_t pos, uint32_t token, bool *refuse
     a.trig = s->trig;
     a.xchg = s->xchg[s->xchg_turn & 1];
     a.xchg_rearm = s->xchg[(s->xchg_turn + 1) & 1];
+    a.xl = s->xl[s->xchg_turn & 1];
+    a.xl_rearm = s->xl[(s->xchg_turn + 1) & 1];
     a.logits = s->logits;
     a.status = s->status_host;
     a.layers = m->hp.layers; a.vocab = m->hp.vocab; a.backlog = s->backlog; a.pos = pos; a.token = token;
     a.spin_limit = s->wait_limit ? s->wait_limit : kSpinLimit;
-    a.xcd_local = m->ctx->xcd_local == 1 && !s->xcd_local_off;
+    a.xcd_local = 1;
     s->xchg_turn++;
     void *params[] = {&a};
     lv_ctx *c = m->ctx;
@@ -2058,12 +2079,7 @@ extern "C" int lv_step_wait(lv_session *s)
     const bool mega_step = s->mega_step;
     s->mega_step = false;
     if (s->status_host && *s->status_host) {
-        const bool misplaced = *s->status_host == 2u;
         *s->status_host = 0;
-        if (misplaced) {
-            s->xcd_local_off = true;
-            return fail(LV_ERR_HIP, "persistent decode kernel: a workgroup ran on another XCD than expected; this session now hands over at device scope");
-        }
         if (++s->mega_failures >= 2) {
             s->mega_off = true;
             return fail(LV_ERR_HIP, "persistent decode kernel: a hand-over wait expired in two steps in a row; this session now takes the %s path",

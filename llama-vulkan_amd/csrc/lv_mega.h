@@ -54,15 +54,16 @@ __device__ __forceinline__ void st_dev(float *p, float v)
     __hip_atomic_store(reinterpret_cast<uint32_t *>(p), __float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Hand-overs inside one XCD.  The workgroups of a launch go to the XCDs in turn (workgroup b runs on XCD b % 8), and the
-// CUs of an XCD share its L2.  A plain store is written through the CU's cache into that L2, and a non-temporal load
+// Hand-overs inside one XCD.  The workgroups of a launch go to the XCDs in turn (workgroups b and b + 8 run on the same
+// XCD; which one workgroup 0 gets depends on what was dispatched before, and launches of other streams dispatched in
+// between break the pattern, so every launch looks: see the kernel's first layer), and the CUs of an XCD share its L2.  A plain store is written through the CU's cache into that L2, and a non-temporal load
 // does not stop at the CU's cache, so a value stored by one workgroup is seen by another one of the same XCD after one
 // L2 round trip: 0.5 us for a flag bounced between two such workgroups, against 1.1 us with the device-scope pair above,
 // whose store has to reach memory (measured; a load with only sc0 set keeps hitting the CU's own cache and never sees
 // the store).  Across XCDs only the device-scope pair works.
 __device__ __forceinline__ uint32_t ld_xcd(const uint32_t *p) { return __builtin_nontemporal_load(p); }
 
-// Where a workgroup stands in the attention phase: XCD b % 8 holds H / 8 heads, for each of them the CPH workgroups that
+// Where a workgroup stands in the attention phase: the 32 workgroups with one value of b % 8 hold H / 8 heads, for each of them the CPH workgroups that
 // take a chunk of the cache each; chunk 0 also combines the chunks.  The same XCD computes the query, key and value rows
 // of its heads in phase A, so these two hand-overs stay inside the XCD.
 template <class S>
@@ -125,9 +126,12 @@ struct MegaShapeBase {
     static constexpr int CPH = kMegaWGs / H;                    // position chunks per head
     static constexpr int PART = R + 4;                          // floats per partial (128 numerators, denominator, pad)
     // floats of one layer's hand-over buffers
-    static constexpr int OFF_QKV = 0, OFF_PART = 3 * D, OFF_O = OFF_PART + H * CPH * PART, OFF_X1 = OFF_O + D,
-                         OFF_FF = OFF_X1 + D, OFF_X2 = OFF_FF + F, XCHG_LAYER = OFF_X2 + D;
-    static constexpr int XCHG_TAIL = 2 * kMegaWGs;              // after the layers: every workgroup's best logit (value, index)
+    // two buffers: what stays inside an XCD (q, k, v, the chunks' partial sums) and what every workgroup reads
+    static constexpr int OFF_QKV = 0, OFF_PART = 3 * D, LOCAL_LAYER = OFF_PART + H * CPH * PART;
+    static constexpr int OFF_O = 0, OFF_X1 = OFF_O + D, OFF_FF = OFF_X1 + D, OFF_X2 = OFF_FF + F, XCHG_LAYER = OFF_X2 + D;
+    static_assert(LOCAL_LAYER % 4 == 0 && XCHG_LAYER % 4 == 0, "re-armed sixteen bytes at a time");
+    // after the layers: every workgroup's best logit (value, index), then the XCD every workgroup found itself on
+    static constexpr int XCHG_TAIL = 3 * kMegaWGs, OFF_XCC = 2 * kMegaWGs;
     static_assert((3 * D) % kMegaWGs == 0 && (2 * F) % kMegaWGs == 0 && D % kMegaWGs == 0, "rows must split over 256 workgroups");
     static_assert(H * R == D && CPH >= 1 && NRD >= 1 && NRF >= 1, "shape");
     // bytes of the weight stream of one layer
@@ -148,14 +152,17 @@ struct MegaArgs {
     const float *tok_f32;      // embedding table [vocab][D] (fp32)
     uint16_t *kv;              // [layers][2][backlog][D] fp16
     const float2 *trig;        // [backlog][64]
-    float *xchg;               // this token's hand-over buffers: [layers] x XCHG_LAYER + XCHG_TAIL floats, all kNotReady
+    float *xchg;               // this token's hand-over buffers for the vectors every workgroup reads: [layers] x XCHG_LAYER +
+                               // XCHG_TAIL floats, all kNotReady.  Uncached device memory: a flag bounced between two XCDs takes
+                               // 0.80 us per round trip there against 1.24 us in ordinary memory (measured)
     float *xchg_rearm;         // the other set, re-armed to kNotReady during this token
+    float *xl, *xl_rearm;      // the same for what stays inside an XCD: [layers] x LOCAL_LAYER floats of ordinary memory (ld_xcd)
     float *logits;             // [vocab]
     uint32_t *status;          // host-visible; [0] set non-zero when a poll loop expired, [kStatusToken] = greedy pick
     uint32_t layers, vocab, backlog, pos, token;
     uint32_t spin_limit;       // polls per hand-over before the step is given up (kSpinLimit; tests of the failure path lower it)
-    uint32_t xcd_local;        // non-zero: workgroup b is known to run on XCD b % 8, so the hand-overs between the workgroups of
-                               // a head go through that XCD's L2 (ld_xcd); zero: device scope everywhere
+    uint32_t xcd_local;        // non-zero: the hand-overs between the workgroups of a head may go through their XCD's L2 (ld_xcd)
+                               // where the launch placed all of them on one XCD; zero: device scope everywhere
 };
 
 // Optional phase timestamps (built only with -DLV_MEGA_TIMING): workgroup 0 records the 100 MHz wall clock at
@@ -375,6 +382,7 @@ struct MegaLds {
     float scratch[2 * S::NW];        // two halves: the waves' sums of x, then of x^2 (later: best logit and its index)
     float attn_red[S::NW * (S::R + 1)];
     float qkv[3 * S::R];             // query of the workgroup's head, K and V row of the newest position
+    float same_xcd;                  // non-zero: the 32 workgroups this one shares heads with all run on its XCD
 };
 
 // Brings the N-float vector at `src` (being produced by other workgroups) into LDS.  With NORM the vector is to be
@@ -477,13 +485,15 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
     uint32_t *status = a.status;
     const uint32_t spin_limit = a.spin_limit;
     const MegaPlace<S> place(b);
-    const bool xcd_local = a.xcd_local != 0;
-    if (xcd_local && threadIdx.x == 0) {
-        // the hand-overs through an XCD's L2 rest on this placement; a launch that does not have it gives the step up
-        uint32_t xcc;
-        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-        if ((int)(xcc & 0xf) != place.xcd) *status = 2u;
-    }
+    // Every workgroup says which XCD it runs on; before its first hand-over inside a head a workgroup reads what the 32
+    // workgroups it shares heads with have said (below, layer 0) and takes the path through the XCD's L2 only if all of
+    // them are where it is.  All 32 read the same words, so they decide alike.
+    uint32_t my_xcc;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(my_xcc));
+    my_xcc &= 0xfu;
+    float *const xcc_table = a.xchg + (size_t)a.layers * S::XCHG_LAYER + S::OFF_XCC;
+    if (threadIdx.x == 0) st_dev(xcc_table + b, __uint_as_float(my_xcc));
+    bool xcd_local = false;
 
     // ---- start the weight stream ------------------------------------------------------------------------------
     MegaTile q[S::DEPTH];
@@ -492,10 +502,12 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
 
     // ---- re-arm the other buffer set for the next token ---------------------------------------------------------
     {
-        const size_t n4 = ((size_t)a.layers * S::XCHG_LAYER + S::XCHG_TAIL) / 4;
-        uint4 *dst = reinterpret_cast<uint4 *>(a.xchg_rearm);
+        const size_t n4 = ((size_t)a.layers * S::XCHG_LAYER + S::XCHG_TAIL) / 4, m4 = (size_t)a.layers * S::LOCAL_LAYER / 4;
+        uint4 *dst = reinterpret_cast<uint4 *>(a.xchg_rearm), *dl = reinterpret_cast<uint4 *>(a.xl_rearm);
         for (size_t i = (size_t)b * T + threadIdx.x; i < n4; i += (size_t)kMegaWGs * T)
             dst[i] = make_uint4(kNotReady, kNotReady, kNotReady, kNotReady);
+        for (size_t i = (size_t)b * T + threadIdx.x; i < m4; i += (size_t)kMegaWGs * T)
+            dl[i] = make_uint4(kNotReady, kNotReady, kNotReady, kNotReady);
     }
 
     const uint32_t pos = a.pos;
@@ -506,7 +518,7 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
     float xsum;
 
     for (uint32_t layer = 0; layer < a.layers; layer++) {
-        float *xc = a.xchg + (size_t)layer * S::XCHG_LAYER;
+        float *xc = a.xchg + (size_t)layer * S::XCHG_LAYER, *xlc = a.xl + (size_t)layer * S::LOCAL_LAYER;
         const float *norm_w = a.norms + (size_t)layer * 2 * D;
         uint16_t *kc = a.kv + (size_t)layer * 2 * a.backlog * D, *vc = kc + (size_t)a.backlog * D;
 
@@ -516,7 +528,21 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
         MEGA_STAMP(1);
         load_slab(xr, xsum, xs, mw.sD * 64 + lane, mw.laneD);
         gemv_phase<S, S::SEQ_A, S::TA, S::NSD>(q, mw, layer, xr, xsum, mw.sD, mw.rD, mw.actD, S::ROWS_A, red);
+        if (layer == 0 && a.xcd_local && w == 0) {
+            // lane j asks for workgroup (b % 8) + 8 j; the words were stored when the kernel started
+            float got[1];
+            const bool want1[1] = {lane < kMegaWGs / 8};
+            poll_values<1, 0>(got, xcc_table + (b & 7) + 8 * (lane & 31), 1, want1, status, spin_limit);
+            const bool same = !want1[0] || __float_as_uint(got[0]) == my_xcc;
+            if (lane == 0) l.same_xcd = __builtin_amdgcn_ballot_w64(!same) == 0 ? 1.f : 0.f;
+        }
         lds_barrier();
+        if (layer == 0) {
+            xcd_local = a.xcd_local && l.same_xcd != 0.f;
+#ifdef LV_MEGA_TIMING
+            if (blockIdx.x == LV_MEGA_TIMING_WG && threadIdx.x == 0) status[3] = xcd_local ? 1u : 0u;
+#endif
+        }
         if (threadIdx.x < S::ROWS_A) {
             const float v = red_row<S::NSD>(red, threadIdx.x) * inv_a;
             int which, col;
@@ -529,8 +555,8 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
                 out = half_bits_to_float(hbits);
             }
             // read by the chunk workgroups of the row's head, which run on this XCD
-            if (xcd_local) xc[S::OFF_QKV + which * D + col] = out;
-            else st_dev(xc + S::OFF_QKV + which * D + col, out);
+            if (xcd_local) xlc[S::OFF_QKV + which * D + col] = out;
+            else st_dev(xlc + S::OFF_QKV + which * D + col, out);
         }
 
         // ================= B: attention chunk (head h, chunk c) ================================================
@@ -579,8 +605,8 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
                 if (w < 3 && (w == 0 || holds_new)) {
                     float pv[2];
                     const bool want2[2] = {true, true};
-                    if (xcd_local) poll_values<2, 0, true>(pv, xc + S::OFF_QKV + w * D + h * R + lane * 2, 1, want2, status, spin_limit);
-                    else poll_values<2, 0>(pv, xc + S::OFF_QKV + w * D + h * R + lane * 2, 1, want2, status, spin_limit);
+                    if (xcd_local) poll_values<2, 0, true>(pv, xlc + S::OFF_QKV + w * D + h * R + lane * 2, 1, want2, status, spin_limit);
+                    else poll_values<2, 0>(pv, xlc + S::OFF_QKV + w * D + h * R + lane * 2, 1, want2, status, spin_limit);
                     l.qkv[w * R + lane * 2] = pv[0];
                     l.qkv[w * R + lane * 2 + 1] = pv[1];
                 }
@@ -665,8 +691,8 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
 #pragma unroll
                     for (int i = 0; i < NW; i++) t += l.attn_red[i * (R + 1) + st];
                     // read by chunk 0 of this head, on this XCD
-                    if (xcd_local) xc[S::OFF_PART + (h * S::CPH + c) * S::PART + st] = t;
-                    else st_dev(xc + S::OFF_PART + (h * S::CPH + c) * S::PART + st, t);
+                    if (xcd_local) xlc[S::OFF_PART + (h * S::CPH + c) * S::PART + st] = t;
+                    else st_dev(xlc + S::OFF_PART + (h * S::CPH + c) * S::PART + st, t);
                 }
             }
         }
@@ -675,7 +701,7 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
         MEGA_STAMP(4);
         if (place.attends && place.c == 0 && st < R) {
             float nd[2 * S::CPH];
-            const uint32_t *hp = reinterpret_cast<const uint32_t *>(xc + S::OFF_PART + (size_t)place.h * S::CPH * S::PART);
+            const uint32_t *hp = reinterpret_cast<const uint32_t *>(xlc + S::OFF_PART + (size_t)place.h * S::CPH * S::PART);
             uint32_t spins = 0;
             bool pending;
             do {
@@ -899,16 +925,6 @@ __global__ void mega_pack_kernel(uint8_t *dst /* start of the phase region */, M
     if constexpr (S::QT == 8) *reinterpret_cast<uint4 *>(out + lane * S::CODE + 16) = codes2;
     if constexpr (S::SF32) *reinterpret_cast<float *>(out + 64 * S::CODE + lane * 4) = scale32;
     else *reinterpret_cast<uint16_t *>(out + 64 * S::CODE + lane * 2) = scale;
-}
-
-// Which XCD each workgroup of a 256-workgroup launch runs on (MegaArgs::xcd_local is set only when it is b % 8).
-__global__ void xcd_probe_kernel(uint32_t *out)
-{
-    if (threadIdx.x == 0) {
-        uint32_t xcc;
-        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-        out[blockIdx.x] = xcc & 0xf;
-    }
 }
 
 }  // namespace lv
