@@ -121,6 +121,13 @@ int lv_session_path(const lv_session *s, int *path);
  * that failure path set 1.  The step can simply be issued again afterwards; after two such steps in a row it runs in
  * the graph path (see lv_session_set_path). */
 int lv_session_set_wait_limit(lv_session *s, uint32_t polls);
+/* The persistent kernel hands a head's query, key and value rows and its partial sums over inside one XCD (through that
+ * XCD's L2 instead of memory) whenever a launch has placed the workgroups that share heads on one XCD; it looks at every
+ * launch and falls back to device scope by itself.  enable = 0 keeps every launch at device scope (for comparison and
+ * diagnosis; results are bit-identical either way).  lv_session_xcd_handover tells what the session's last persistent
+ * step did (0 before one).  No counterpart in the reference, which has one queue and no such choice. */
+int lv_session_set_xcd_handover(lv_session *s, int enable);
+int lv_session_xcd_handover(lv_session *s, int *used);
 
 /* ---- cache dump / restore: replaces llava_layer_session_data::dump_kv_cache / restore_kv_cache
  *      (llava_layer_session_data.cpp:165-181).  which: 0 = K, 1 = V.  n_tokens rows of `dim` fp16 values. */

@@ -92,6 +92,8 @@ _HIP_SIGS = {
     "lv_session_use_graph": [_VP, _I],
     "lv_session_set_path": [_VP, _I],
     "lv_session_set_wait_limit": [_VP, C.c_uint32],
+    "lv_session_set_xcd_handover": [_VP, _I],
+    "lv_session_xcd_handover": [_VP, C.POINTER(_I)],
     "lv_session_path": [_VP, C.POINTER(_I)],
     "lv_step_begin": [_VP, _VP, _U32, _U32],
     "lv_step_wait": [_VP],
@@ -361,6 +363,15 @@ class Session:
 
     def set_wait_limit(self, polls):
         check(self.lib.lv_session_set_wait_limit(self.h, int(polls)))
+
+    def set_xcd_handover(self, on):
+        check(self.lib.lv_session_set_xcd_handover(self.h, int(on)))
+
+    def xcd_handover(self):
+        """did the last persistent step keep the hand-overs inside a head inside one XCD?"""
+        used = C.c_int()
+        check(self.lib.lv_session_xcd_handover(self.h, C.byref(used)))
+        return bool(used.value)
 
     def path(self):
         p = C.c_int()

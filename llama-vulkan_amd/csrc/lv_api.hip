@@ -224,6 +224,7 @@ struct lv_session {
     uint32_t xchg_turn = 0;
     uint32_t *status_host = nullptr;      // pinned, written by the persistent kernel: [0] a poll expired, [kStatusToken] greedy pick
     uint32_t wait_limit = 0;              // polls per hand-over of the persistent kernel; 0 = default
+    bool xcd_handover = true;             // the persistent kernel may keep a head's hand-overs inside its XCD (lv_session_set_xcd_handover)
     bool pick_in_status = false;          // the last step ran the persistent kernel, whose greedy pick is in status_host
     bool mega_step = false;               // the step in flight ran the persistent kernel
     int mega_failures = 0;                // steps of the persistent kernel in a row that ended with an expired wait
@@ -1674,7 +1675,7 @@ static int launch_mega(lv_session *s, uint32_t pos, uint32_t token, bool *refuse
     a.status = s->status_host;
     a.layers = m->hp.layers; a.vocab = m->hp.vocab; a.backlog = s->backlog; a.pos = pos; a.token = token;
     a.spin_limit = s->wait_limit ? s->wait_limit : kSpinLimit;
-    a.xcd_local = 1;
+    a.xcd_local = s->xcd_handover ? 1u : 0u;
     s->xchg_turn++;
     void *params[] = {&a};
     lv_ctx *c = m->ctx;
@@ -2113,6 +2114,21 @@ extern "C" int lv_argmax(lv_session *s, uint32_t *token)
     HIP_TRY(hipMemcpyAsync(s->argmax_host, s->argmax_dev, 4, hipMemcpyDeviceToHost, s->stream));
     LV_TRY(lv_step_wait(s));
     *token = *s->argmax_host;
+    return LV_OK;
+}
+
+extern "C" int lv_session_set_xcd_handover(lv_session *s, int enable)
+{
+    if (!s) return fail(LV_ERR_ARG, "lv_session_set_xcd_handover: session is null");
+    s->xcd_handover = enable != 0;
+    return LV_OK;
+}
+
+extern "C" int lv_session_xcd_handover(lv_session *s, int *used)
+{
+    if (!s || !used) return fail(LV_ERR_ARG, "lv_session_xcd_handover: null argument");
+    if (s->in_flight) return fail(LV_ERR_STATE, "lv_session_xcd_handover: a step is in flight");
+    *used = s->status_host && s->status_host[kStatusXcd] ? 1 : 0;
     return LV_OK;
 }
 

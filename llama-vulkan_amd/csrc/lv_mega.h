@@ -39,6 +39,7 @@ constexpr int kMegaVocabRows = 125;     // output-matrix rows per workgroup the 
 // hand-over ran out still ends within seconds.
 constexpr uint32_t kSpinLimit = 1u << 14;
 constexpr int kStatusToken = 2;         // word of the status block that receives the index of the largest logit
+constexpr int kStatusXcd = 3;           // word that tells whether workgroup 0 handed over inside its XCD in the last launch
 // A consumer reaches a hand-over about when its producers store: a load issued at once samples memory before the
 // stores are visible (0.6 us) yet comes back only after the prefetched tiles ahead of it on the CU's return path
 // (1-2 us), and the second try pays that again.  Sleeping this many 64-clock units first makes the first try
@@ -539,9 +540,7 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
         lds_barrier();
         if (layer == 0) {
             xcd_local = a.xcd_local && l.same_xcd != 0.f;
-#ifdef LV_MEGA_TIMING
-            if (blockIdx.x == LV_MEGA_TIMING_WG && threadIdx.x == 0) status[3] = xcd_local ? 1u : 0u;
-#endif
+            if (b == 0 && threadIdx.x == 0) status[kStatusXcd] = xcd_local ? 1u : 0u;      // what workgroup 0's 32 decided
         }
         if (threadIdx.x < S::ROWS_A) {
             const float v = red_row<S::NSD>(red, threadIdx.x) * inv_a;

@@ -383,7 +383,7 @@ def handover_case(name, wtype, seed, backlog, last):
     emit(case=name, wtype="q4_0" if wtype == lva.LV_Q4_0 else "q8_0", position=last, kernel_ms=round(float(np.mean(ms)), 4),
          layer_us=round(float(acc.sum()), 2), phases_us={n: round(float(v), 2) for n, v in zip(names, acc)},
          handover_us=round(float(acc[[0, 2, 4, 5, 7, 9]].sum()), 2), work_us=round(float(acc[[1, 3, 6, 8, 10]].sum()), 2),
-         head_handovers_inside_xcd=bool(words[3]))
+         head_handovers_inside_xcd=s.xcd_handover())
     s.close()
     model.close()
     ctx.close()

@@ -255,6 +255,27 @@ def test_persistent_kernel_is_deterministic_and_rearms(lva, ctx, wide_model):
     a.close(); b.close(); model.close()
 
 
+def test_persistent_kernel_hands_over_alike_inside_an_xcd_and_at_device_scope(lva, ctx, wide_model):
+    """a head's q, k, v rows and partial sums travel through the XCD's L2 where the launch allows it, through memory otherwise:
+    only the transport differs, so the logits are the same bits; with the switch off no launch may take the short way"""
+    model = lva.Model(ctx, wide_model)
+    a, b = lva.Session(model, 128), lva.Session(model, 128)
+    assert not a.xcd_handover()                          # no persistent step yet
+    b.set_xcd_handover(False)
+    toks = lva.synth_tokens(12, 3, 2048, seed=4)
+    inside = 0
+    for i, t in enumerate(toks):
+        a.begin([t], i)
+        la = a.logits()
+        inside += a.xcd_handover()
+        b.begin([t], i)
+        lb = b.logits()
+        assert not b.xcd_handover()
+        assert np.array_equal(la, lb), i
+    print("steps that handed over inside an XCD:", inside, "of", len(toks))
+    a.close(); b.close(); model.close()
+
+
 def test_persistent_kernel_refused_for_other_shapes(lva, ctx, tiny_models):
     model = lva.Model(ctx, tiny_models["tiny_q4"])
     s = lva.Session(model, 128)
