@@ -20,6 +20,9 @@
 // store; consumers poll the data itself with device-scope loads.  No flag, no fence, no wait for store
 // acknowledgement.  Two buffer sets alternate between tokens; each token re-arms the other set.
 // Every poll loop is bounded: on expiry the kernel raises *status and carries on to its end.
+// The vectors every workgroup reads (o, x1, ff, x2) lie in uncached device memory, where such a hand-over between
+// XCDs is a third shorter; q, k, v and the partial sums go from a head's producers to that head's own workgroups
+// only, which a launch normally places on one XCD: those two hand-overs then go through the XCD's L2 (ld_xcd).
 //
 // Weight stream: for each (layer, phase, workgroup, wave) the tiles that wave will consume, in order.
 // A tile is one matrix row restricted to the wave's 64-block column slab: 64 x 16 B (q4_0) or 64 x 32 B
