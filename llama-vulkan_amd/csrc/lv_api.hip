@@ -2253,6 +2253,82 @@ extern "C" int lv_debug_gemm_clock(unsigned long long *dst)
     return LV_OK;
 }
 
+// Timing builds only: a counter bounced `rounds` times between workgroups wg_a and wg_b of a 256-workgroup launch, thread 0 of
+// each polling the other's word: what one hand-over of the persistent kernel costs at the least, by kind of memory
+// (0 ordinary, 1 uncached, 2 fine-grained) and by cache policy of the polling load (0 plain, 1 sc0, 2 sc1 = device scope,
+// 3 non-temporal) and of the store (0 plain, 2 sc1).  Every wait is bounded; a pair that never sees the other's store
+// reports expired = 1 (a load that keeps hitting its CU's cache).  out: {100 MHz ticks, expired, XCC id of a, XCC id of b}.
+template <int LD> __device__ __forceinline__ uint32_t flag_load(const uint32_t *p)
+{
+    uint32_t v;
+    if constexpr (LD == 0) asm volatile("global_load_dword %0, %1, off\n s_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
+    else if constexpr (LD == 1) asm volatile("global_load_dword %0, %1, off sc0\n s_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
+    else if constexpr (LD == 2) asm volatile("global_load_dword %0, %1, off sc1\n s_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
+    else asm volatile("global_load_dword %0, %1, off nt\n s_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
+template <int ST> __device__ __forceinline__ void flag_store(uint32_t *p, uint32_t v)
+{
+    if constexpr (ST == 0) asm volatile("global_store_dword %0, %1, off\n s_waitcnt vmcnt(0)" ::"v"(p), "v"(v) : "memory");
+    else asm volatile("global_store_dword %0, %1, off sc1\n s_waitcnt vmcnt(0)" ::"v"(p), "v"(v) : "memory");
+}
+template <int LD, int ST>
+__global__ void flag_roundtrip_kernel(uint32_t *flag /* two words 256 bytes apart */, int a, int b, int rounds, uint32_t limit, uint32_t *out)
+{
+    if (threadIdx.x != 0) return;
+    const int me = (int)blockIdx.x == a ? 0 : (int)blockIdx.x == b ? 1 : -1;
+    if (me < 0) return;
+    uint32_t xcc;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+    out[2 + me] = xcc & 0xfu;
+    uint32_t *mine = flag + 64 * me, *other = flag + 64 * (1 - me);
+    bool expired = false;
+    const uint64_t t0 = wall_clock64();
+    for (int r = 1; r <= rounds && !expired; r++) {
+        if (me == 0) flag_store<ST>(mine, (uint32_t)r);
+        uint32_t n = 0;
+        while (flag_load<LD>(other) < (uint32_t)r)
+            if (++n > limit) { expired = true; break; }
+        if (me == 1 && !expired) flag_store<ST>(mine, (uint32_t)r);
+    }
+    if (me == 0) out[0] = (uint32_t)(wall_clock64() - t0);
+    if (expired) out[1] = 1u;
+}
+
+extern "C" int lv_debug_flag_roundtrip(lv_ctx *c, int memory, int load_policy, int store_policy, int wg_a, int wg_b, int rounds, uint32_t *out4)
+{
+    if (!c || !out4 || memory < 0 || memory > 2 || wg_a < 0 || wg_b < 0 || wg_a >= 256 || wg_b >= 256 || wg_a == wg_b || rounds < 1) return LV_ERR_ARG;
+    HIP_TRY(hipSetDevice(c->device));
+    // the flag words are never freed: memory allocated after freeing an uncached buffer has held wrong values on this platform
+    static uint32_t *flags[3] = {nullptr, nullptr, nullptr};
+    static uint32_t *out = nullptr;
+    if (!flags[memory]) {
+        if (memory == 0) HIP_TRY(hipMalloc(reinterpret_cast<void **>(&flags[0]), 1024));
+        else HIP_TRY(hipExtMallocWithFlags(reinterpret_cast<void **>(&flags[memory]), 1024, memory == 1 ? hipDeviceMallocUncached : hipDeviceMallocFinegrained));
+    }
+    if (!out) HIP_TRY(hipMalloc(reinterpret_cast<void **>(&out), 16));
+    HIP_TRY(hipMemsetAsync(flags[memory], 0, 1024, c->stream));
+    HIP_TRY(hipMemsetAsync(out, 0, 16, c->stream));
+    const dim3 grid(256), block(64);
+    const uint32_t limit = 20000u;
+#define LV_FLAG_CASE(LD, ST) flag_roundtrip_kernel<LD, ST><<<grid, block, 0, c->stream>>>(flags[memory], wg_a, wg_b, rounds, limit, out)
+    const int key = load_policy * 4 + store_policy;
+    switch (key) {
+    case 0: LV_FLAG_CASE(0, 0); break;
+    case 4: LV_FLAG_CASE(1, 0); break;
+    case 8: LV_FLAG_CASE(2, 0); break;
+    case 10: LV_FLAG_CASE(2, 2); break;
+    case 12: LV_FLAG_CASE(3, 0); break;
+    case 14: LV_FLAG_CASE(3, 2); break;
+    default: return LV_ERR_ARG;
+    }
+#undef LV_FLAG_CASE
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipMemcpyAsync(out4, out, 16, hipMemcpyDeviceToHost, c->stream));
+    HIP_TRY(hipStreamSynchronize(c->stream));
+    return LV_OK;
+}
+
 // debugging aid of timing builds only: the persistent kernel's phase timestamps
 extern "C" int lv_debug_status_words(lv_session *s, uint32_t *dst, uint32_t n)
 {

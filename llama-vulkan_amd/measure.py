@@ -15,6 +15,7 @@
     python llama-vulkan_amd/measure.py gemm          isolated 512-token GEMMs at the 13B shapes, q8_0 (for kernel traces and counters)
     python llama-vulkan_amd/measure.py handover      phases of the persistent kernel inside a layer (7B q4_0, position 511; timing build)
     python llama-vulkan_amd/measure.py handover-q8   the same for 7B q8_0 at position 2047
+    python llama-vulkan_amd/measure.py flag-roundtrip  a flag bounced between two workgroups by memory kind and cache policy: the floor of a hand-over (timing build)
     python llama-vulkan_amd/measure.py gemm-clock    shader clock and cycles per K step of gemm_kernel during the 13B q8_0 prompt (timing build)
     python llama-vulkan_amd/measure.py copy          1 GiB device-to-device copy: achievable bandwidth, counter calibration
     python llama-vulkan_amd/measure.py all
@@ -389,6 +390,28 @@ def handover_case(name, wtype, seed, backlog, last):
     ctx.close()
 
 
+def flag_roundtrip_case():
+    """What a hand-over costs at the least (timing build): a counter bounced 2000 times between two workgroups of a
+    256-workgroup launch, on one XCD (workgroups 0 and 8) and on two (0 and 9), for the three kinds of device memory and the
+    cache policies of the polling load and of the store.  Every wait is bounded; "never" = the load kept hitting its CU's cache."""
+    import ctypes as C
+    import numpy as np
+    lva._libs["libllava_hip.so"] = C.CDLL(os.path.join(HERE, "libllava_hip_timing.so"), mode=C.RTLD_GLOBAL)
+    ctx = lva.Context(0)
+    ctx.lib.lv_debug_flag_roundtrip.argtypes = [C.c_void_p] + [C.c_int] * 6 + [C.c_void_p]
+    rounds = 2000
+    mem_names = ["ordinary", "uncached", "fine-grained"]
+    pol = [("plain", 0, "plain", 0), ("sc0", 1, "plain", 0), ("non-temporal", 3, "plain", 0), ("non-temporal", 3, "sc1", 2), ("sc1", 2, "plain", 0), ("sc1", 2, "sc1", 2)]
+    for mem in range(3):
+        for other in (8, 9):
+            for lname, ld, sname, st in pol:
+                out = np.zeros(4, dtype=np.uint32)
+                lva.check(ctx.lib.lv_debug_flag_roundtrip(ctx.h, mem, ld, st, 0, other, rounds, out.ctypes.data_as(C.c_void_p)))
+                emit(case="flag-roundtrip", memory=mem_names[mem], load=lname, store=sname, workgroups=[0, other], xcc=[int(out[2]), int(out[3])],
+                     us_per_round_trip=None if out[1] else round(float(out[0]) / 100.0 / rounds, 3), seen="never" if out[1] else "yes")
+    ctx.close()
+
+
 def gemm_clock_case():
     """Loads the timing build and evaluates the 13B q8_0 512-token prompt eight times; after each pass reads what workgroup 0
     of the last gemm_kernel launch (the last layer's down projection: a K slice of 4608 = 144 steps) measured around its K
@@ -450,6 +473,8 @@ def main():
     which = sys.argv[1] if len(sys.argv) > 1 else "all"
     if which == "gemm-clock":
         return gemm_clock_case()
+    if which == "flag-roundtrip":
+        return flag_roundtrip_case()
     if which == "handover":
         return handover_case("handover", lva.LV_Q4_0, 0, 512, 511)
     if which == "handover-q8":
