@@ -436,11 +436,41 @@ __device__ __forceinline__ float acquire_vector(float *xs, const float *src, con
     return inv;
 }
 
+// The same for a long vector without normalisation (the down projection's input): 16 bytes a thread and load, a quarter of
+// the load instructions per poll (a buffer load with sc1 = device scope; past the end of the vector it returns zeros).
+typedef uint32_t mega_u4v __attribute__((ext_vector_type(4)));
+template <int N, int NW, int SLEEP>
+__device__ __forceinline__ void acquire_vector_wide(float *xs, const float *src, uint32_t *status, uint32_t spin_limit)
+{
+    constexpr int T = NW * 64, PER = cdiv(N, 4 * T);
+    static_assert(N % 4 == 0, "whole 16-byte groups");
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(src), 0, N * 4, 0x00020000);
+    mega_u4v v[PER];
+    uint32_t spins = 0;
+    bool pending;
+    if constexpr (SLEEP > 0) __builtin_amdgcn_s_sleep(SLEEP);
+    do {
+        pending = false;
+        asm volatile("" ::: "memory");      // every turn issues the loads again
+#pragma unroll
+        for (int j = 0; j < PER; j++) {
+            v[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, 16 * ((int)threadIdx.x + j * T), 0, 16 /* sc1 */);
+            pending |= (v[j].x == kNotReady) | (v[j].y == kNotReady) | (v[j].z == kNotReady) | (v[j].w == kNotReady);
+        }
+    } while (pending && ++spins < spin_limit);
+    if (pending) *status = 1u;
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+        const int idx = 4 * ((int)threadIdx.x + j * T);
+        if (idx < N) *reinterpret_cast<mega_u4v *>(xs + xs_index(idx)) = v[j];
+    }
+    lds_barrier();
+}
+
 // Phase E, where every working wave owns one column slab (S::NRF == 1): a wave fetches the 2048 floats of its own slab and
 // nothing else, 16 bytes a lane and load, at device scope; it starts on its tiles when the producers of that slab have
 // stored, without a workgroup barrier, and the workgroup no longer moves the whole F-float vector with every thread.
 // The slab passes through the wave's own part of LDS to reach the block-per-lane order of load_slab.
-typedef uint32_t mega_u4v __attribute__((ext_vector_type(4)));
 template <class S, int SLEEP>
 __device__ __forceinline__ void acquire_own_slab(float (&xr)[32], float &xsum, float *xs, const float *src, int slab, int lane, bool active,
                                                  bool lane_has, uint32_t *status, uint32_t spin_limit)
@@ -757,7 +787,7 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
             acquire_own_slab<S, kPollDelay>(xr, xsum, xs, xc + S::OFF_FF, mw.sF, lane, mw.actF, mw.laneF, status, spin_limit);
             MEGA_STAMP(10);
         } else {
-            acquire_vector<F, NW, false, kPollDelay>(xs, xc + S::OFF_FF, nullptr, scratch, status, spin_limit);
+            acquire_vector_wide<F, NW, kPollDelay>(xs, xc + S::OFF_FF, status, spin_limit);
             MEGA_STAMP(10);
             load_slab(xr, xsum, xs, mw.sF * 64 + lane, mw.laneF);
         }
