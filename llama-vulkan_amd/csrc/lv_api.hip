@@ -103,8 +103,9 @@ struct UncachedBlock { int device; size_t bytes; void *ptr; };
 static std::mutex g_uncached_mutex;
 static std::vector<UncachedBlock> g_uncached_free;
 
-static int uncached_take(int device, void **out, size_t bytes)
+static int uncached_take(int device, void **out, size_t bytes, bool *pooled)
 {
+    *pooled = true;
     {
         std::lock_guard<std::mutex> lock(g_uncached_mutex);
         for (size_t i = 0; i < g_uncached_free.size(); i++)
@@ -116,16 +117,27 @@ static int uncached_take(int device, void **out, size_t bytes)
     }
     hipError_t e = hipExtMallocWithFlags(out, bytes, hipDeviceMallocUncached);
     if (e != hipSuccess) {
+        // a runtime without that kind of memory: ordinary memory does as well, only slower (the hand-overs are device scope
+        // either way); such a block is freed like any other
+        (void)hipGetLastError();
+        *pooled = false;
+        e = hipMalloc(out, bytes);
+    }
+    if (e != hipSuccess) {
         (void)hipGetLastError();
         *out = nullptr;
-        return fail(e == hipErrorOutOfMemory ? LV_ERR_OOM : LV_ERR_HIP, "uncached hand-over buffer of %llu bytes: %s", (unsigned long long)bytes, hipGetErrorString(e));
+        return fail(e == hipErrorOutOfMemory ? LV_ERR_OOM : LV_ERR_HIP, "hand-over buffer of %llu bytes: %s", (unsigned long long)bytes, hipGetErrorString(e));
     }
     return LV_OK;
 }
 
-static void uncached_give(int device, void *ptr, size_t bytes)
+static void uncached_give(int device, void *ptr, size_t bytes, bool pooled)
 {
     if (!ptr) return;
+    if (!pooled) {
+        (void)hipFree(ptr);
+        return;
+    }
     std::lock_guard<std::mutex> lock(g_uncached_mutex);
     g_uncached_free.push_back({device, bytes, ptr});
 }
@@ -220,6 +232,7 @@ struct lv_session {
     size_t pf_plane_halfs = 0;
     float *xchg[2] = {nullptr, nullptr};  // hand-over buffer sets of the persistent kernel: uncached memory (uncached_take / uncached_give) ...
     size_t xchg_bytes = 0;
+    bool xchg_pooled[2] = {true, true};   // false: the runtime had no uncached memory and the set lies in ordinary memory
     float *xl[2] = {nullptr, nullptr};    // ... and the part of them that stays inside an XCD, ordinary memory
     uint32_t xchg_turn = 0;
     uint32_t *status_host = nullptr;      // pinned, written by the persistent kernel: [0] a poll expired, [kStatusToken] greedy pick
@@ -1454,7 +1467,7 @@ extern "C" int lv_session_destroy(lv_session *s)
                    s->pf_xh, s->pf_xl, s->pf_xs, s->pf_planes, s->pf_fh, s->pf_fl};
     for (void *p : dev) (void)hipFree(p);
     for (int i = 0; i < 2; i++) {
-        uncached_give(s->model->ctx->device, s->xchg[i], s->xchg_bytes);
+        uncached_give(s->model->ctx->device, s->xchg[i], s->xchg_bytes, s->xchg_pooled[i]);
         (void)hipFree(s->xl[i]);
     }
     if (s->status_host) (void)hipHostFree(s->status_host);
@@ -1493,7 +1506,7 @@ static int session_alloc(lv_session *s)
         }));
         s->xchg_bytes = bytes;
         for (int i = 0; i < 2; i++) {
-            LV_TRY(uncached_take(s->model->ctx->device, reinterpret_cast<void **>(&s->xchg[i]), bytes));
+            LV_TRY(uncached_take(s->model->ctx->device, reinterpret_cast<void **>(&s->xchg[i]), bytes, &s->xchg_pooled[i]));
             HIP_TRY(hipMemsetAsync(s->xchg[i], 0xff, bytes, s->stream));
             HIP_TRY(hipMalloc(reinterpret_cast<void **>(&s->xl[i]), local_bytes));
             HIP_TRY(hipMemsetAsync(s->xl[i], 0xff, local_bytes, s->stream));
