@@ -199,22 +199,25 @@ struct MegaTile {
 template <class S>
 __device__ __forceinline__ void load_tile(MegaTile &t, const uint8_t *p, int lane)
 {
-    // q4_0: non-temporal loads.  The weights pass once per token and need no place in the caches, which the cache rows, the
-    // norm weights and the hand-over vectors then keep (measured: a pure read stream reaches 6.9 instead of 6.1-6.2 TB/s with
-    // them, and the 7B q4_0 token takes 3 % less; 13B q4_0 the same either way).  q8_0 keeps ordinary loads: a lane's two
-    // 16-byte loads fall into one cache line, and without the CU's cache the second one is a request of its own (the 7B
-    // q8_0 token takes 5 % more with non-temporal loads, the 13B one 15 %).
+    // Non-temporal loads: the weights pass once per token and need no place in the caches, which the cache rows, the norm
+    // weights and the hand-over vectors then keep (measured: a pure read stream reaches 6.9 instead of 6.1-6.2 TB/s with
+    // them; the 7B q4_0 token takes 3 % less, the q8_0 tokens 6-7 % less).  Every load of a wave covers one contiguous
+    // kilobyte: without the CU's cache a second load into the same cache line would be a request of its own.
     if constexpr (S::QT == 4) {
         typedef uint32_t nt_u4v __attribute__((ext_vector_type(4)));
         const nt_u4v v = __builtin_nontemporal_load(reinterpret_cast<const nt_u4v *>(p + lane * S::CODE));
         t.c = make_uint4(v.x, v.y, v.z, v.w);
     } else {
-        t.c = *reinterpret_cast<const uint4 *>(p + lane * S::CODE);
-        t.c2 = *reinterpret_cast<const uint4 *>(p + lane * S::CODE + 16);
+        // q8_0: the two halves of a block's codes lie in two planes of the tile (64 x 16 bytes each), so that either load of
+        // a wave covers one contiguous kilobyte
+        typedef uint32_t nt_u4v __attribute__((ext_vector_type(4)));
+        const nt_u4v v = __builtin_nontemporal_load(reinterpret_cast<const nt_u4v *>(p + lane * 16));
+        const nt_u4v v2 = __builtin_nontemporal_load(reinterpret_cast<const nt_u4v *>(p + 1024 + lane * 16));
+        t.c = make_uint4(v.x, v.y, v.z, v.w);
+        t.c2 = make_uint4(v2.x, v2.y, v2.z, v2.w);
     }
     if constexpr (S::SF32) t.d32 = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(p + 64 * S::CODE + lane * 4));
-    else if constexpr (S::QT == 4) t.d = __builtin_nontemporal_load(reinterpret_cast<const uint16_t *>(p + 64 * S::CODE + lane * 2));
-    else t.d = *reinterpret_cast<const uint16_t *>(p + 64 * S::CODE + lane * 2);
+    else t.d = __builtin_nontemporal_load(reinterpret_cast<const uint16_t *>(p + 64 * S::CODE + lane * 2));
 }
 
 // one block column of one row: sum over 32 weights of w * x, from the raw codes
@@ -965,8 +968,12 @@ __global__ void mega_pack_kernel(uint8_t *dst /* start of the phase region */, M
         if constexpr (S::SF32) scale32 = mv->scales_f32[sb];
         else scale = mv->scales[sb];
     }
-    *reinterpret_cast<uint4 *>(out + lane * S::CODE) = codes;
-    if constexpr (S::QT == 8) *reinterpret_cast<uint4 *>(out + lane * S::CODE + 16) = codes2;
+    if constexpr (S::QT == 8) {
+        *reinterpret_cast<uint4 *>(out + lane * 16) = codes;
+        *reinterpret_cast<uint4 *>(out + 1024 + lane * 16) = codes2;
+    } else {
+        *reinterpret_cast<uint4 *>(out + lane * S::CODE) = codes;
+    }
     if constexpr (S::SF32) *reinterpret_cast<float *>(out + 64 * S::CODE + lane * 4) = scale32;
     else *reinterpret_cast<uint16_t *>(out + 64 * S::CODE + lane * 2) = scale;
 }
