@@ -25,8 +25,8 @@
 // only, which a launch normally places on one XCD: those two hand-overs then go through the XCD's L2 (ld_xcd).
 //
 // Weight stream: for each (layer, phase, workgroup, wave) the tiles that wave will consume, in order.
-// A tile is one matrix row restricted to the wave's 64-block column slab: 64 x 16 B (q4_0) or 64 x 32 B
-// (q8_0) of codes + 64 x fp16 scales (1152 B / 2176 B).  Lane l of the wave always owns block column 64*slab + l, so the 32 activations of
+// A tile is one matrix row restricted to the wave's 64-block column slab: 64 x 16 B (q4_0) or two planes of 64 x 16 B
+// (q8_0: first and second half of every block's codes) + 64 x fp16 scales (1152 B / 2176 B).  Lane l of the wave always owns block column 64*slab + l, so the 32 activations of
 // that column sit in registers for the whole phase.
 #pragma once
 
