@@ -123,7 +123,16 @@ struct MegaShapeBase {
     // (acquire_own_slab).  Where waves are left over (7B: six slabs, eight waves) the common fetch by all threads is as fast.
     static constexpr bool OWN_SLAB_E = NRF == 1 && NSF == NW;
     static constexpr int ROWS_A = 3 * D / kMegaWGs, ROWS_C = D / kMegaWGs, ROWS_D = 2 * F / kMegaWGs, ROWS_E = D / kMegaWGs;
-    static constexpr int TA = cdiv(ROWS_A, NRD), TC = cdiv(ROWS_C, NRD), TD = cdiv(ROWS_D, NRD), TE = cdiv(ROWS_E, NRF);
+    // Down projection (phase E).  Where the waves outnumber the column slabs (7B: six slabs, eight waves) the spare waves take
+    // the last E_SPARE_ROWS rows of E_SPARE_SLABS slabs each, so that every wave has the same number of tiles (12 instead of 16
+    // for six waves); a spare wave's tile i is row ROWS_E - E_SPARE_ROWS + i % E_SPARE_ROWS of slab (w - NSF) * E_SPARE_SLABS + i / E_SPARE_ROWS.
+    static constexpr int E_SPARE = NRF == 1 ? NW - NSF : 0;
+    static constexpr bool E_REDEAL = E_SPARE > 0 && (ROWS_E * NSF) % NW == 0 && NSF % E_SPARE == 0 &&
+                                     (ROWS_E - ROWS_E * NSF / NW) % 4 == 0 && (ROWS_E * NSF / NW) % 4 == 0 &&
+                                     (ROWS_E - ROWS_E * NSF / NW) * (NSF / E_SPARE) == ROWS_E * NSF / NW;
+    static constexpr int E_SPARE_SLABS = E_REDEAL ? NSF / E_SPARE : 0, E_SPARE_ROWS = E_REDEAL ? ROWS_E - ROWS_E * NSF / NW : 0;
+    static constexpr int TA = cdiv(ROWS_A, NRD), TC = cdiv(ROWS_C, NRD), TD = cdiv(ROWS_D, NRD),
+                         TE = E_REDEAL ? ROWS_E * NSF / NW : cdiv(ROWS_E, NRF);
     static constexpr int SEQ_A = 0, SEQ_C = TA, SEQ_D = TA + TC, SEQ_E = TA + TC + TD;
     static constexpr int PER_LAYER = round_up(TA + TC + TD + TE, DEPTH);
     static constexpr int HEAD = round_up(cdiv(kMegaVocabRows, NRD), 4);   // head tiles per wave (static upper bound)
@@ -149,6 +158,14 @@ template <int D_, int F_, int H_, int NW_, int QT_, int DEPTH_ = 0>
 struct MegaShape : MegaShapeBase<D_, F_, H_, NW_, QT_, DEPTH_, false> {};
 template <int D_, int F_, int H_, int NW_, int QT_, int DEPTH_ = 0>
 struct MegaShapeV1 : MegaShapeBase<D_, F_, H_, NW_, QT_, DEPTH_, true> {};
+
+// phase E of a re-dealt shape: row (of the workgroup's ROWS_E) and column slab of tile i of wave w
+template <class S>
+__host__ __device__ __forceinline__ void mega_e_tile(int w, int i, int &row, int &slab)
+{
+    if (w < S::NSF) { row = i; slab = w; }
+    else { row = S::ROWS_E - S::E_SPARE_ROWS + i % S::E_SPARE_ROWS; slab = (w - S::NSF) * S::E_SPARE_SLABS + i / S::E_SPARE_ROWS; }
+}
 
 struct MegaArgs {
     const uint8_t *wstream;    // [layers] x LAYER_BYTES, then HEAD_BYTES, then one all-zero tile
@@ -317,7 +334,15 @@ struct MegaWave {
         if (k < S::SEQ_C) { i = k; tiles = S::TA; rows = S::ROWS_A; act = actD; lane_ok = laneD; rset = rD; }
         else if (k < S::SEQ_D) { i = k - S::SEQ_C; tiles = S::TC; rows = S::ROWS_C; act = actD; lane_ok = laneD; rset = rD; off = S::PHASE_A_BYTES; }
         else if (k < S::SEQ_E) { i = k - S::SEQ_D; tiles = S::TD; rows = S::ROWS_D; act = actD; lane_ok = laneD; rset = rD; off = S::PHASE_A_BYTES + S::PHASE_C_BYTES; }
-        else if (k < S::SEQ_E + S::TE) { i = k - S::SEQ_E; tiles = S::TE; rows = S::ROWS_E; act = actF; lane_ok = laneF; rset = rF; off = S::PHASE_A_BYTES + S::PHASE_C_BYTES + S::PHASE_D_BYTES; }
+        else if (k < S::SEQ_E + S::TE) {
+            i = k - S::SEQ_E; tiles = S::TE; rows = S::ROWS_E; act = actF; lane_ok = laneF; rset = rF; off = S::PHASE_A_BYTES + S::PHASE_C_BYTES + S::PHASE_D_BYTES;
+            if constexpr (S::E_REDEAL) {
+                int row, slab;
+                mega_e_tile<S>(w, i, row, slab);
+                act = true; rset = 0; rows = S::TE;          // every wave has TE tiles; only the lanes past the last block column have none
+                lane_ok = slab * 64 + lane < S::NBF;
+            }
+        }
         else real = false;                                   // padding slot of the layer sequence
         const bool head_slot = wrapped && k < S::HEAD;  // static
         if (!real && !head_slot) return;                     // static: this slot never loads
@@ -804,9 +829,36 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
         } else {
             acquire_vector_wide<F, NW, kPollDelay>(xs, xc + S::OFF_FF, status, spin_limit);
             MEGA_STAMP(10);
-            load_slab(xr, xsum, xs, mw.sF * 64 + lane, mw.laneF);
+            if constexpr (S::E_REDEAL) {
+                int row0, slab0;
+                mega_e_tile<S>(w, 0, row0, slab0);
+                load_slab(xr, xsum, xs, slab0 * 64 + lane, slab0 * 64 + lane < S::NBF);
+            } else {
+                load_slab(xr, xsum, xs, mw.sF * 64 + lane, mw.laneF);
+            }
         }
-        gemv_phase<S, S::SEQ_E, S::TE, S::NSF>(q, mw, layer, xr, xsum, mw.sF, mw.rF, mw.actF, S::ROWS_E, red);
+        if constexpr (S::E_REDEAL) {
+            // every wave TE tiles; the spare waves change their column slab every E_SPARE_ROWS tiles and fetch its activations anew
+            float p[4];
+#pragma unroll
+            for (int i = 0; i < S::TE; i++) {
+                int row, slab;
+                mega_e_tile<S>(w, i, row, slab);
+                if (i > 0 && i % S::E_SPARE_ROWS == 0 && w >= S::NSF) load_slab(xr, xsum, xs, slab * 64 + lane, slab * 64 + lane < S::NBF);
+                const int slot = (S::SEQ_E + i) % S::DEPTH;
+                const MegaTile t = q[slot];
+                p[i & 3] = tile_dot<S>(t, xr, xsum);
+                mw.fetch(q[slot], S::SEQ_E + i + S::DEPTH, layer);
+                if ((i & 3) == 3) {
+                    const float sum4 = quad_partials_sum(p[0], p[1], p[2], p[3]);
+                    int r0, sl;
+                    mega_e_tile<S>(w, i - 3, r0, sl);       // the four tiles are four consecutive rows of one slab
+                    if ((lane & 15) == 0) red[(r0 + quad_partial_of_lane(lane)) * S::NSF + sl] = sum4;
+                }
+            }
+        } else {
+            gemv_phase<S, S::SEQ_E, S::TE, S::NSF>(q, mw, layer, xr, xsum, mw.sF, mw.rF, mw.actF, S::ROWS_E, red);
+        }
         // padding slots of the layer's sequence carry no tile, but the slot S::DEPTH ahead of them does
 #pragma unroll
         for (int k = S::SEQ_E + S::TE; k < S::PER_LAYER; k++) mw.fetch(q[k % S::DEPTH], k + S::DEPTH, layer);
@@ -926,11 +978,16 @@ __global__ void mega_pack_kernel(uint8_t *dst /* start of the phase region */, M
     const int i = tile % tiles;
     const int w = (tile / tiles) % S::NW;
     const int b = tile / tiles / S::NW;
-    const int slab = w % ns, rset = w / ns;
+    int slab = w % ns, rset = w / ns;
     uint8_t *out = dst + tile * S::TILE;
     uint4 codes = make_uint4(0, 0, 0, 0), codes2 = codes;
     uint16_t scale = 0;
     float scale32 = 0.f;
+    int e_row = 0;
+    if (S::E_REDEAL && phase == 3) {
+        mega_e_tile<S>(w, i, e_row, slab);
+        rset = 0;
+    }
     const int blk = slab * 64 + lane;
     bool ok = rset < nr && blk < nb;
     const MatView *mv = nullptr;
@@ -944,7 +1001,7 @@ __global__ void mega_pack_kernel(uint8_t *dst /* start of the phase region */, M
             mv = &src.m[0];
         } else {
             const int rows = phase == 0 ? S::ROWS_A : phase == 1 ? S::ROWS_C : phase == 2 ? S::ROWS_D : S::ROWS_E;
-            const int j = rset * tiles + i;
+            const int j = (S::E_REDEAL && phase == 3) ? e_row : rset * tiles + i;
             ok = j < rows;
             const int g = b * rows + j;
             if (phase == 0) {
