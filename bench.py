@@ -7,7 +7,7 @@ Prints ONE JSON line:
   value      tokens/s over the K timed steps (wall clock, host sampling included)
   roofline   the persistent decode kernel (one launch = one token): algorithmic bytes per launch / average launch
              duration measured with HIP events on the session's stream, against the 8 TB/s HBM peak
-  cpu_baseline  the CPU checker (oracle/) timed on a few decode steps of the same model at the same positions, on
+  cpu_baseline  the CPU checker (oracle/) timed on the same decode steps (same model, same tokens and positions; 64 steps are 10-15 s), on
              this box's host cores; reported beside the GPU number, never the target
 
 Weights and prompt are synthetic (seeded writer, llama-vulkan_amd/mkggml.c).
@@ -122,7 +122,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--cpu-steps", type=int, default=3, help="decode steps the CPU checker is timed on (0 = skip)")
+    ap.add_argument("--cpu-steps", type=int, default=64, help="decode steps the CPU checker is timed on, the last ones of the timed region (0 = skip)")
     ap.add_argument("--no-cases", action="store_true", help="skip the other configurations (the \"cases\" key)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -195,14 +195,17 @@ def main():
             for which in (0, 1):
                 osess.kv_load(layer, which, sess.kv(layer, which, start))
         osess.set_pos(start)
-        worst = 0.0
+        worst, ties = 0.0, 0
         t1 = time.perf_counter()
         for i in range(n_cpu):
             want = osess.eval([tokens[start - timed_first + i]])
             tok_cpu = oracle.greedy(want)
-            if tok_cpu != tokens[start - timed_first + i + 1]:
+            tok_gpu = tokens[start - timed_first + i + 1]
+            # a different pick is an error unless the checker's own logits hold the two within the logits' tolerance
+            ties += tok_cpu != tok_gpu
+            if tok_cpu != tok_gpu and not float(want[tok_cpu] - want[tok_gpu]) <= 1e-3 * float(np.max(np.abs(want))):
                 raise SystemExit(f"bench.py: greedy token at position {start + i} differs from the CPU checker "
-                                 f"({tokens[start - timed_first + i + 1]} vs {tok_cpu})")
+                                 f"({tok_gpu} vs {tok_cpu})")
         cpu_dt = time.perf_counter() - t1
         # logits of the last step, GPU against checker
         sess.begin([tokens[pos - 1 - timed_first]], pos - 1)
@@ -211,7 +214,9 @@ def main():
             raise SystemExit(f"bench.py: logits differ from the CPU checker by {worst}")
         cpu = {"value": round(n_cpu / cpu_dt, 3), "unit": "tok/s", "cores": oracle.num_threads(), "kind": "port",
                "sample": f"{n_cpu} greedy decode steps of the same model at positions {start}..{pos - 1} "
-                         f"(cache restored from the GPU run; tokens identical, max |dlogit| {worst:.1e})",
+                         f"(cache restored from the GPU run; "
+                         + ("tokens identical" if ties == 0 else f"{ties} picks differ inside the logits' tolerance")
+                         + f", max |dlogit| of the last step {worst:.1e})",
                "lavapipe": lavapipe_status()}
         osess.close()
         om.close()
