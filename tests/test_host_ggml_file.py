@@ -214,3 +214,14 @@ def test_every_python_file_of_the_package_compiles():
     assert len(files) > 10
     for f in files:
         py_compile.compile(f, doraise=True)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; any other --gpus ends before anything touches a device, with a message that says so"""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0
+    assert "ONE GPU" in r.stderr and "--gpus 1" in r.stderr
+    assert r.stdout.strip() == ""
