@@ -163,8 +163,9 @@ struct MegaShapeV1 : MegaShapeBase<D_, F_, H_, NW_, QT_, DEPTH_, true> {};
 template <class S>
 __host__ __device__ __forceinline__ void mega_e_tile(int w, int i, int &row, int &slab)
 {
+    constexpr int SR = S::E_SPARE_ROWS > 0 ? S::E_SPARE_ROWS : 1;   // shapes without spare rows never take the second branch
     if (w < S::NSF) { row = i; slab = w; }
-    else { row = S::ROWS_E - S::E_SPARE_ROWS + i % S::E_SPARE_ROWS; slab = (w - S::NSF) * S::E_SPARE_SLABS + i / S::E_SPARE_ROWS; }
+    else { row = S::ROWS_E - S::E_SPARE_ROWS + i % SR; slab = (w - S::NSF) * S::E_SPARE_SLABS + i / SR; }
 }
 
 struct MegaArgs {
@@ -546,7 +547,7 @@ __device__ __forceinline__ void acquire_own_slab(float (&xr)[32], float &xsum, f
 template <class S>
 __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
 {
-    constexpr int D = S::D, F = S::F, H = S::H, R = S::R, NW = S::NW, T = NW * 64;
+    constexpr int D = S::D, F = S::F, R = S::R, NW = S::NW, T = NW * 64;
     __shared__ __attribute__((aligned(16))) MegaLds<S> l;
     float *xs = l.xs, *red = l.red, *xown = l.xown, *scratch = l.scratch;
 #ifdef LV_MEGA_TIMING
