@@ -13,7 +13,6 @@ PKG = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(PKG)
 
 HIP_LIB = os.path.join(PKG, "libllava_hip.so")
-HIP_TIMING_LIB = os.path.join(PKG, "libllava_hip_timing.so")
 HOST_LIB = os.path.join(PKG, "libllava_host.so")
 MKGGML_LIB = os.path.join(PKG, "libmkggml.so")
 MKGGML_BIN = os.path.join(PKG, "bin", "mkggml")
@@ -43,14 +42,6 @@ def build_hip():
     src = os.path.join(PKG, "csrc", "lv_api.hip")
     _run([hipcc(), *HIPCC_FLAGS, src, "-o", HIP_LIB])
     return HIP_LIB
-
-
-def build_hip_timing():
-    """the same library with the persistent kernel's phase timestamps compiled in (-DLV_MEGA_TIMING): a measuring aid that
-    `measure.py handover` loads; nothing else does"""
-    src = os.path.join(PKG, "csrc", "lv_api.hip")
-    _run([hipcc(), *HIPCC_FLAGS, "-DLV_MEGA_TIMING", src, "-o", HIP_TIMING_LIB])
-    return HIP_TIMING_LIB
 
 
 def build_mkggml():
@@ -87,7 +78,6 @@ def build_oracle():
 def build_all():
     build_mkggml()
     build_hip()
-    build_hip_timing()
     build_host()
     build_oracle()
 

@@ -2034,8 +2034,9 @@ extern "C" int lv_step_begin(lv_session *s, const uint32_t *tokens, uint32_t n, 
             LV_TRY(launch_mega(s, pos + done, tokens[done], &refused));
             if (refused) break;
             done++;
+            s->mega_step = true;
+            s->in_flight = true;       // from here on an error return leaves kernels on the stream: lv_step_wait has to follow
         }
-        s->mega_step = done > 0;
         if (refused) {
             // the tokens launched so far stay as they are; the rest of this step, and every later one, takes the other path
             s->mega_off = true;
@@ -2235,9 +2236,7 @@ extern "C" int lv_trace_read_rows(lv_session *s, uint32_t layer, int which, uint
         const size_t slot = hp.dim > hp.ff ? hp.dim : hp.ff, have = which == LV_TRACE_FF ? hp.ff : hp.dim;
         HIP_TRY(hipMemcpy2DAsync(dst, have * 4, trace_slot(s, layer, which, row0), slot * 4, have * 4, n_rows, hipMemcpyDeviceToHost, s->stream));
     }
-    HIP_TRY(hipStreamSynchronize(s->stream));
-    s->in_flight = false;
-    return LV_OK;
+    return lv_step_wait(s);     // the one place a step ends: stream wait, status word of the persistent kernel, its bookkeeping
 }
 
 extern "C" int lv_trace_read(lv_session *s, uint32_t layer, int which, float *dst, uint32_t count)
@@ -2255,98 +2254,3 @@ extern "C" int lv_trace_read(lv_session *s, uint32_t layer, int which, float *ds
     }
     return lv_trace_read_rows(s, layer, which, s->trace_n - 1, 1, dst);
 }
-
-#ifdef LV_MEGA_TIMING
-// timing builds only: {shader cycles, 100 MHz wall ticks, K steps} of workgroup 0 of the last gemm_kernel launch
-extern "C" int lv_debug_gemm_clock(unsigned long long *dst)
-{
-    if (!dst) return LV_ERR_ARG;
-    HIP_TRY(hipDeviceSynchronize());
-    HIP_TRY(hipMemcpyFromSymbol(dst, HIP_SYMBOL(gemm_clock_words), sizeof(gemm_clock_words)));
-    return LV_OK;
-}
-
-// Timing builds only: a counter bounced `rounds` times between workgroups wg_a and wg_b of a 256-workgroup launch, thread 0 of
-// each polling the other's word: what one hand-over of the persistent kernel costs at the least, by kind of memory
-// (0 ordinary, 1 uncached, 2 fine-grained) and by cache policy of the polling load (0 plain, 1 sc0, 2 sc1 = device scope,
-// 3 non-temporal) and of the store (0 plain, 2 sc1).  Every wait is bounded; a pair that never sees the other's store
-// reports expired = 1 (a load that keeps hitting its CU's cache).  out: {100 MHz ticks, expired, XCC id of a, XCC id of b}.
-template <int LD> __device__ __forceinline__ uint32_t flag_load(const uint32_t *p)
-{
-    uint32_t v;
-    if constexpr (LD == 0) asm volatile("global_load_dword %0, %1, off\n s_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
-    else if constexpr (LD == 1) asm volatile("global_load_dword %0, %1, off sc0\n s_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
-    else if constexpr (LD == 2) asm volatile("global_load_dword %0, %1, off sc1\n s_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
-    else asm volatile("global_load_dword %0, %1, off nt\n s_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
-    return v;
-}
-template <int ST> __device__ __forceinline__ void flag_store(uint32_t *p, uint32_t v)
-{
-    if constexpr (ST == 0) asm volatile("global_store_dword %0, %1, off\n s_waitcnt vmcnt(0)" ::"v"(p), "v"(v) : "memory");
-    else asm volatile("global_store_dword %0, %1, off sc1\n s_waitcnt vmcnt(0)" ::"v"(p), "v"(v) : "memory");
-}
-template <int LD, int ST>
-__global__ void flag_roundtrip_kernel(uint32_t *flag /* two words 256 bytes apart */, int a, int b, int rounds, uint32_t limit, uint32_t *out)
-{
-    if (threadIdx.x != 0) return;
-    const int me = (int)blockIdx.x == a ? 0 : (int)blockIdx.x == b ? 1 : -1;
-    if (me < 0) return;
-    uint32_t xcc;
-    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-    out[2 + me] = xcc & 0xfu;
-    uint32_t *mine = flag + 64 * me, *other = flag + 64 * (1 - me);
-    bool expired = false;
-    const uint64_t t0 = wall_clock64();
-    for (int r = 1; r <= rounds && !expired; r++) {
-        if (me == 0) flag_store<ST>(mine, (uint32_t)r);
-        uint32_t n = 0;
-        while (flag_load<LD>(other) < (uint32_t)r)
-            if (++n > limit) { expired = true; break; }
-        if (me == 1 && !expired) flag_store<ST>(mine, (uint32_t)r);
-    }
-    if (me == 0) out[0] = (uint32_t)(wall_clock64() - t0);
-    if (expired) out[1] = 1u;
-}
-
-extern "C" int lv_debug_flag_roundtrip(lv_ctx *c, int memory, int load_policy, int store_policy, int wg_a, int wg_b, int rounds, uint32_t *out4)
-{
-    if (!c || !out4 || memory < 0 || memory > 2 || wg_a < 0 || wg_b < 0 || wg_a >= 256 || wg_b >= 256 || wg_a == wg_b || rounds < 1) return LV_ERR_ARG;
-    HIP_TRY(hipSetDevice(c->device));
-    // the flag words are never freed: memory allocated after freeing an uncached buffer has held wrong values on this platform
-    static uint32_t *flags[3] = {nullptr, nullptr, nullptr};
-    static uint32_t *out = nullptr;
-    if (!flags[memory]) {
-        if (memory == 0) HIP_TRY(hipMalloc(reinterpret_cast<void **>(&flags[0]), 1024));
-        else HIP_TRY(hipExtMallocWithFlags(reinterpret_cast<void **>(&flags[memory]), 1024, memory == 1 ? hipDeviceMallocUncached : hipDeviceMallocFinegrained));
-    }
-    if (!out) HIP_TRY(hipMalloc(reinterpret_cast<void **>(&out), 16));
-    HIP_TRY(hipMemsetAsync(flags[memory], 0, 1024, c->stream));
-    HIP_TRY(hipMemsetAsync(out, 0, 16, c->stream));
-    const dim3 grid(256), block(64);
-    const uint32_t limit = 20000u;
-#define LV_FLAG_CASE(LD, ST) flag_roundtrip_kernel<LD, ST><<<grid, block, 0, c->stream>>>(flags[memory], wg_a, wg_b, rounds, limit, out)
-    const int key = load_policy * 4 + store_policy;
-    switch (key) {
-    case 0: LV_FLAG_CASE(0, 0); break;
-    case 4: LV_FLAG_CASE(1, 0); break;
-    case 8: LV_FLAG_CASE(2, 0); break;
-    case 10: LV_FLAG_CASE(2, 2); break;
-    case 12: LV_FLAG_CASE(3, 0); break;
-    case 14: LV_FLAG_CASE(3, 2); break;
-    default: return LV_ERR_ARG;
-    }
-#undef LV_FLAG_CASE
-    HIP_TRY(hipGetLastError());
-    HIP_TRY(hipMemcpyAsync(out4, out, 16, hipMemcpyDeviceToHost, c->stream));
-    HIP_TRY(hipStreamSynchronize(c->stream));
-    return LV_OK;
-}
-
-// debugging aid of timing builds only: the persistent kernel's phase timestamps
-extern "C" int lv_debug_status_words(lv_session *s, uint32_t *dst, uint32_t n)
-{
-    if (!s || !s->status_host || n > 1024) return LV_ERR_ARG;
-    memcpy(dst, s->status_host, (size_t)n * 4);
-    return LV_OK;
-}
-#endif

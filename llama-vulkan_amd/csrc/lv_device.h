@@ -6,6 +6,12 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+// The kernels lean on gfx950 behaviour the HIP memory model does not promise (write-through stores acknowledged once every
+// XCD can see them, non-temporal loads that pass the CU's cache, the XCC id register): no other device target is built.
+#if defined(__HIP_DEVICE_COMPILE__) && !defined(__gfx950__)
+#error "llama-vulkan_amd device code is written for gfx950 (MI355X) only"
+#endif
+
 namespace lv {
 
 constexpr int kWave = 64;

@@ -486,12 +486,6 @@ __global__ __launch_bounds__(256) void prefill_norm_kernel(PrefillNormArgs a)
     }
 }
 
-#ifdef LV_MEGA_TIMING
-// timing builds only: workgroup 0 of the last gemm_kernel launch leaves the shader cycles and the 100 MHz wall ticks of its
-// K loop and the number of steps here (lv_debug_gemm_clock reads them): the shader clock under this load, cycles per step
-__device__ unsigned long long gemm_clock_words[3];
-#endif
-
 // One workgroup: 128 tokens x 256 weight rows over a range of K.  The grid enumerates (matrix or K slice, row tile, token
 // tile) so that the token tiles of one row tile run on one XCD (workgroups are dealt to the 8 XCDs in turn) and find its
 // weights in that XCD's L2, and so that the XCDs get equal numbers of workgroups.
@@ -620,9 +614,6 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a)
         for (int r = 0; r < 4; r++) { cv[r] = T[14][r]; cv[4 + r] = T[15][r]; }
         cd[0] = cur.d[2]; cd[1] = cur.d[3];
     };
-#ifdef LV_MEGA_TIMING
-    const unsigned long long clk0 = clock64(), wall0 = wall_clock64();
-#endif
     Frag FA, FB;
 #pragma unroll
     for (int s = 0; s < NST; s++)
@@ -640,13 +631,6 @@ __device__ __forceinline__ void gemm_body(const GemmArgs &a)
 #pragma unroll
     for (int idx = 0; idx < 8; idx++) acc[3][2 + (idx >> 2)][idx & 3] = fmaf(cv[idx], cd[idx >> 2], acc[3][2 + (idx >> 2)][idx & 3]);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // the repeats past the end have landed before the workgroup gives up its LDS
-#ifdef LV_MEGA_TIMING
-    if (blockIdx.x == 0 && tid == 0) {
-        gemm_clock_words[0] = clock64() - clk0;
-        gemm_clock_words[1] = wall_clock64() - wall0;
-        gemm_clock_words[2] = steps;
-    }
-#endif
 
     // acc[ti][tj][r]: token tt * 128 + wm * 64 + ti * 16 + 4 * l4 + r, weight row rt * 256 + wn * 64 + tj * 16 + l15.
     // The per-token scales of this lane's 16 tokens, fetched before the first store (the stores may alias them for all the

@@ -512,22 +512,14 @@ __global__ __launch_bounds__(256) void attention_kernel(AttnArgs a)
     // write-through stores, the wave waits for their acknowledgement, then the workgroup counts itself in; the
     // last workgroup reads the partials with device-scope loads, which do not hit stale lines.
     // This leans on gfx950 hardware rules that the HIP memory model does not promise (stores are counted by vmcnt, and a
-    // write-through store is acknowledged only once every XCD can see it), so it is compiled for gfx950 alone; the
-    // parity tests run it with 2..32 splits per head.  Any other target gets the release / acquire pair of the model.
+    // write-through store is acknowledged only once every XCD can see it); lv_device.h refuses any other target.  The
+    // parity tests run it with 2..32 splits per head.
     __shared__ uint32_t arrived;
-#if defined(__gfx950__)
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (threadIdx.x == 0) arrived = __hip_atomic_fetch_add(&a.counters[(size_t)z * H + h], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (arrived != n_splits - 1) return;
-#else
-    __syncthreads();
-    if (threadIdx.x == 0) arrived = __hip_atomic_fetch_add(&a.counters[(size_t)z * H + h], 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads();
-    if (arrived != n_splits - 1) return;
-    __atomic_thread_fence(__ATOMIC_ACQUIRE);
-#endif
     const float *hp = a.part + ((size_t)z * H + h) * a.splits * (R + 1);
     if (threadIdx.x <= R) {
         float t = 0.f;

@@ -187,25 +187,10 @@ struct MegaArgs {
                                // where the launch placed all of them on one XCD; zero: device scope everywhere
 };
 
-// Optional phase timestamps (built only with -DLV_MEGA_TIMING): workgroup 0 records the 100 MHz wall clock at
-// every phase boundary of layers 0..3 into status[16 + ...].
-#ifdef LV_MEGA_TIMING
-#ifndef LV_MEGA_TIMING_WG
-#define LV_MEGA_TIMING_WG 0
-#endif
-#define MEGA_STAMP(idx)                                                                                        \
-    do {                                                                                                       \
-        if (blockIdx.x == LV_MEGA_TIMING_WG && threadIdx.x == 0 && layer < 4)                                  \
-            status[16 + layer * 16 + (idx)] = (uint32_t)wall_clock64();                                        \
-    } while (0)
-#define MEGA_STREAM_STAMP(idx)                                                                                 \
-    do {                                                                                                       \
-        if (blockIdx.x == LV_MEGA_TIMING_WG && threadIdx.x == 0 && layer < 4)                                  \
-            a.status[16 + layer * 16 + (idx)] = (uint32_t)wall_clock64();                                      \
-    } while (0)
-#else
+// Phase boundaries of a layer are marked MEGA_STAMP(n); the marks compile to nothing unless the including file has
+// defined the macro (it sees the kernel's `status`, `layer` and thread indices).
+#ifndef MEGA_STAMP
 #define MEGA_STAMP(idx) do { } while (0)
-#define MEGA_STREAM_STAMP(idx) do { } while (0)
 #endif
 
 struct MegaTile {
@@ -550,9 +535,6 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
     constexpr int D = S::D, F = S::F, R = S::R, NW = S::NW, T = NW * 64;
     __shared__ __attribute__((aligned(16))) MegaLds<S> l;
     float *xs = l.xs, *red = l.red, *xown = l.xown, *scratch = l.scratch;
-#ifdef LV_MEGA_TIMING
-    const uint64_t clk0 = clock64(), wall0 = wall_clock64();
-#endif
     MegaWave<S> mw;
     mw.init(a);
     const int b = mw.b, w = mw.w, lane = mw.lane;
@@ -950,12 +932,6 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
             if (st == 0) status[kStatusToken] = bi == kNotReady ? 0u : bi;
         }
     }
-#ifdef LV_MEGA_TIMING
-    if (blockIdx.x == LV_MEGA_TIMING_WG && threadIdx.x == 0) {
-        a.status[8] = (uint32_t)(clock64() - clk0);
-        a.status[9] = (uint32_t)(wall_clock64() - wall0);
-    }
-#endif
 }
 
 // ---------------------------------------------------------------------------------------------------------

@@ -82,12 +82,12 @@ static void note_interrupt(int) { g_interrupted = 1; }
 
 static void print_usage(const char *argv0)
 {
-    std::cerr << "usage: " << argv0 << " [-m|--model FILE] [--print_header] [--greedy] [--seed N] [-n TOKENS] [-d DEVICE] [-v] [-h] [PROMPT]\n"
+    std::cerr << "usage: " << argv0 << " [-m|--model FILE] [--print_header] [--greedy] [--seed N] [-n TOKENS] [-d DEVICE] [-v|--verbose] [-h] [PROMPT]\n"
               << "       " << argv0 << " [-m|--model FILE] -s|--server [--port N] [--bind ADDRESS]\n"
               << "       the model path may also come from the LLAVA_MODEL environment variable\n";
 }
 
-// Flags of the reference kept: -m/--model, --print_header, -h, -v, trailing positional prompt, LLAVA_MODEL
+// Flags of the reference kept: -m/--model, --print_header, -h, -v/--verbose, -c/--control (refused, as there), trailing positional prompt, LLAVA_MODEL
 // (llava_context.cpp:163-212).  --use-prebuilt, --debug and --sigdebug concern Vulkan shader builds, the
 // validation layer and signalfd debugging and are accepted and ignored.  -s/--server starts the token server after
 // the model is loaded (llava_context.cpp:333-336); --port and --bind are additions (the reference listens on 0.0.0.0:1337).
@@ -108,7 +108,8 @@ int llava_context::run(int argc, char **argv)
             return argv[++i];
         };
         if (a == "-h" || a == "--help") { print_usage(argv[0]); return 0; }
-        else if (a == "-v") ++verbosity;
+        else if (a == "-v" || a == "--verbose") ++verbosity;
+        else if (a == "-c" || a == "--control") { std::cerr << "Control disabled for now" << std::endl; return 1; }   // llava_context.cpp:186-187,202-205
         else if (a == "--print_header") print_header = true;
         else if (a == "--greedy") greedy = true;
         else if (a == "--use-prebuilt" || a == "--debug" || a == "--sigdebug") continue;

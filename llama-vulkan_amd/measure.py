@@ -13,10 +13,6 @@
     python llama-vulkan_amd/measure.py prefill-7b    7B q4_0, the same
     python llama-vulkan_amd/measure.py prefill-13b-q4  13B q4_0, the same
     python llama-vulkan_amd/measure.py gemm          isolated 512-token GEMMs at the 13B shapes, q8_0 (for kernel traces and counters)
-    python llama-vulkan_amd/measure.py handover      phases of the persistent kernel inside a layer (7B q4_0, position 511; timing build)
-    python llama-vulkan_amd/measure.py handover-q8   the same for 7B q8_0 at position 2047
-    python llama-vulkan_amd/measure.py flag-roundtrip  a flag bounced between two workgroups by memory kind and cache policy: the floor of a hand-over (timing build)
-    python llama-vulkan_amd/measure.py gemm-clock    shader clock and cycles per K step of gemm_kernel during the 13B q8_0 prompt (timing build)
     python llama-vulkan_amd/measure.py copy          1 GiB device-to-device copy: achievable bandwidth, counter calibration
     python llama-vulkan_amd/measure.py all
 
@@ -247,199 +243,6 @@ def prefill_case(ctx, case, name, wtype, report=emit):
     return r
 
 
-def board_power_watts():
-    """the board's power sensor (amdgpu hwmon, microwatts), or None where the driver does not show one"""
-    import glob
-    for f in glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input") + glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_average"):
-        try:
-            return int(open(f).read()) / 1e6
-        except (OSError, ValueError):
-            pass
-    return None
-
-
-def board_power_cap_watts():
-    import glob
-    for f in glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_cap"):
-        try:
-            return int(open(f).read()) / 1e6
-        except (OSError, ValueError):
-            pass
-    return None
-
-
-def prefill_power_case(ctx, case, name, wtype, seconds=4.0, report=emit):
-    """The 512-token prompt step repeated for `seconds` while a thread reads the board's power sensor every 10 ms:
-    the time per step and the sensor's readings from the idle board, over the run, and in its second half."""
-    import threading
-    import time
-    shape = SHAPES[name]
-    model = lva.Model(ctx, model_file(name, wtype, 3))
-    s = lva.Session(model, 512)
-    prompt = lva.synth_tokens(512, 3, shape["vocab"], seed=3)
-    idle = board_power_watts()
-    s.begin(prompt, 0)
-    s.wait()
-    samples, stop = [], threading.Event()
-
-    def sampler():
-        while not stop.is_set():
-            samples.append((time.monotonic(), board_power_watts()))
-            time.sleep(0.01)
-    th = threading.Thread(target=sampler)
-    th.start()
-    t0 = time.monotonic()
-    times = []
-    while time.monotonic() - t0 < seconds:
-        s.timer_start()
-        s.begin(prompt, 0)
-        times.append(s.timer_stop())
-    t1 = time.monotonic()
-    stop.set()
-    th.join()
-    w = [p for t, p in samples if p is not None and t0 <= t <= t1]
-    late = [p for t, p in samples if p is not None and (t0 + t1) / 2 <= t <= t1]
-    half = len(times) // 2
-    r = report(case=case, model=name, wtype="q4_0" if wtype == lva.LV_Q4_0 else "q8_0", tokens=512, steps=len(times),
-               ms_first=round(times[0], 2), ms_mean_first_half=round(sum(times[:half]) / max(1, half), 2),
-               ms_mean_second_half=round(sum(times[half:]) / max(1, len(times) - half), 2),
-               power_cap_W=board_power_cap_watts(), idle_W=idle, samples=len(w),
-               power_mean_W=round(sum(w) / len(w), 1) if w else None, power_max_W=max(w) if w else None,
-               power_mean_second_half_W=round(sum(late) / len(late), 1) if late else None)
-    s.close()
-    model.close()
-    return r
-
-
-def decode_power_case(ctx, case, seconds=3.0, report=emit):
-    """Greedy decode of the 7B q4_0 model at positions 448..511, the window repeated for `seconds`, with the board's power
-    sensor read every 10 ms: is the decode kernel anywhere near the board's power cap?"""
-    import threading
-    import time
-    shape = SHAPES["7b"]
-    model = lva.Model(ctx, model_file("7b", lva.LV_Q4_0, 0))
-    s = lva.Session(model, 512)
-    s.begin(lva.synth_tokens(440, 3, shape["vocab"], seed=0), 0)
-    tok = s.argmax()
-    for pos in range(440, 448):
-        s.begin([tok], pos)
-        tok = s.argmax()
-    samples, stop = [], threading.Event()
-
-    def sampler():
-        while not stop.is_set():
-            samples.append(board_power_watts())
-            time.sleep(0.01)
-    th = threading.Thread(target=sampler)
-    th.start()
-    t0 = time.monotonic()
-    steps = 0
-    while time.monotonic() - t0 < seconds:
-        for pos in range(448, 512):      # the same cache rows rewritten: a decode step's work does not depend on the token
-            s.begin([tok], pos)
-            tok = s.argmax()
-        steps += 64
-    dt = time.monotonic() - t0
-    stop.set()
-    th.join()
-    w = [p for p in samples if p is not None]
-    r = report(case=case, steps=steps, tok_s=round(steps / dt, 1), power_cap_W=board_power_cap_watts(), samples=len(w),
-               power_mean_W=round(sum(w) / len(w), 1) if w else None, power_max_W=max(w) if w else None)
-    s.close()
-    model.close()
-    return r
-
-
-def handover_case(name, wtype, seed, backlog, last):
-    """Loads the timing build of the library (libllava_hip_timing.so, -DLV_MEGA_TIMING: workgroup 0 of the persistent kernel
-    writes the 100 MHz wall clock at every phase boundary of layers 0..3) and prints, for the decode step at position
-    `last`, the time between the boundaries, averaged over 16 launches and the four layers.  acq = waiting for and fetching
-    the vector the workgroups before handed over; the rest is the phase's own work."""
-    import ctypes as C
-    import numpy as np
-    lva._libs["libllava_hip.so"] = C.CDLL(os.path.join(HERE, "libllava_hip_timing.so"), mode=C.RTLD_GLOBAL)
-    ctx = lva.Context(0)
-    shape = SHAPES["7b"]
-    model = lva.Model(ctx, model_file("7b", wtype, seed))
-    s = lva.Session(model, backlog)
-    first = last - 7
-    s.begin(lva.synth_tokens(first, 3, shape["vocab"], seed=seed), 0)
-    tok = s.argmax()
-    for pos in range(first, last):
-        s.begin([tok], pos)
-        tok = s.argmax()
-    ctx.lib.lv_debug_status_words.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32]
-    names = ["A acq (x)", "A norm+QKV", "B acq (q,k,v)", "B attention", "B' combine", "C acq (o)", "C Wo", "D acq (x)", "D norm+gate.up", "E acq (ff)", "E W2"]
-    acc, ms = np.zeros(len(names)), []
-    reps = 16
-    for _ in range(reps):
-        s.timer_start()
-        s.begin([tok], last)
-        ms.append(s.timer_stop())
-        words = np.zeros(256, dtype=np.uint32)
-        lva.check(ctx.lib.lv_debug_status_words(s.h, words.ctypes.data_as(C.c_void_p), 256))
-        for layer in range(4):
-            t = words[16 + layer * 16: 16 + layer * 16 + 12].astype(np.int64)
-            acc += np.diff(t) * 0.01 / (4 * reps)                      # 100 MHz ticks -> us
-    emit(case=name, wtype="q4_0" if wtype == lva.LV_Q4_0 else "q8_0", position=last, kernel_ms=round(float(np.mean(ms)), 4),
-         layer_us=round(float(acc.sum()), 2), phases_us={n: round(float(v), 2) for n, v in zip(names, acc)},
-         handover_us=round(float(acc[[0, 2, 4, 5, 7, 9]].sum()), 2), work_us=round(float(acc[[1, 3, 6, 8, 10]].sum()), 2),
-         head_handovers_inside_xcd=s.xcd_handover())
-    s.close()
-    model.close()
-    ctx.close()
-
-
-def flag_roundtrip_case():
-    """What a hand-over costs at the least (timing build): a counter bounced 2000 times between two workgroups of a
-    256-workgroup launch, on one XCD (workgroups 0 and 8) and on two (0 and 9), for the three kinds of device memory and the
-    cache policies of the polling load and of the store.  Every wait is bounded; "never" = the load kept hitting its CU's cache."""
-    import ctypes as C
-    import numpy as np
-    lva._libs["libllava_hip.so"] = C.CDLL(os.path.join(HERE, "libllava_hip_timing.so"), mode=C.RTLD_GLOBAL)
-    ctx = lva.Context(0)
-    ctx.lib.lv_debug_flag_roundtrip.argtypes = [C.c_void_p] + [C.c_int] * 6 + [C.c_void_p]
-    rounds = 2000
-    mem_names = ["ordinary", "uncached", "fine-grained"]
-    pol = [("plain", 0, "plain", 0), ("sc0", 1, "plain", 0), ("non-temporal", 3, "plain", 0), ("non-temporal", 3, "sc1", 2), ("sc1", 2, "plain", 0), ("sc1", 2, "sc1", 2)]
-    for mem in range(3):
-        for other in (8, 9):
-            for lname, ld, sname, st in pol:
-                out = np.zeros(4, dtype=np.uint32)
-                lva.check(ctx.lib.lv_debug_flag_roundtrip(ctx.h, mem, ld, st, 0, other, rounds, out.ctypes.data_as(C.c_void_p)))
-                emit(case="flag-roundtrip", memory=mem_names[mem], load=lname, store=sname, workgroups=[0, other], xcc=[int(out[2]), int(out[3])],
-                     us_per_round_trip=None if out[1] else round(float(out[0]) / 100.0 / rounds, 3), seen="never" if out[1] else "yes")
-    ctx.close()
-
-
-def gemm_clock_case():
-    """Loads the timing build and evaluates the 13B q8_0 512-token prompt eight times; after each pass reads what workgroup 0
-    of the last gemm_kernel launch (the last layer's down projection: a K slice of 4608 = 144 steps) measured around its K
-    loop: shader cycles (clock64) against the 100 MHz wall clock = the shader clock the launch ran at, and cycles per step
-    (the MFMAs of a SIMD's two waves take 1024)."""
-    import ctypes as C
-    lva._libs["libllava_hip.so"] = C.CDLL(os.path.join(HERE, "libllava_hip_timing.so"), mode=C.RTLD_GLOBAL)
-    ctx = lva.Context(0)
-    shape = SHAPES["13b"]
-    model = lva.Model(ctx, model_file("13b", lva.LV_Q8_0, 3))
-    s = lva.Session(model, 512)
-    prompt = lva.synth_tokens(512, 3, shape["vocab"], seed=3)
-    s.begin(prompt, 0)
-    s.wait()
-    words = (C.c_ulonglong * 3)()
-    for rep in range(8):
-        s.timer_start()
-        s.begin(prompt, 0)
-        ms = s.timer_stop()
-        lva.check(ctx.lib.lv_debug_gemm_clock(words))
-        cycles, ticks, steps = words[0], words[1], words[2]
-        emit(case="gemm-clock", pass_ms=round(ms, 2), steps=int(steps), shader_cycles=int(cycles), wall_us=round(ticks / 100.0, 1),
-             shader_MHz=round(cycles / (ticks / 100.0)), cycles_per_step=round(cycles / max(steps, 1)))
-    s.close()
-    model.close()
-    ctx.close()
-
-
 def gemm_cases(ctx, report=emit):
     """reference: the *_batch shaders on 512 pending tokens (llava_session.cpp:243-255).  One lv_kernel_gemm call = the split of
     the activations into fp16 halves + gemm_kernel (+ the sum of the K slices where the grid would not fill the device), at
@@ -471,14 +274,6 @@ def gemm_cases(ctx, report=emit):
 
 def main():
     which = sys.argv[1] if len(sys.argv) > 1 else "all"
-    if which == "gemm-clock":
-        return gemm_clock_case()
-    if which == "flag-roundtrip":
-        return flag_roundtrip_case()
-    if which == "handover":
-        return handover_case("handover", lva.LV_Q4_0, 0, 512, 511)
-    if which == "handover-q8":
-        return handover_case("handover-q8", lva.LV_Q8_0, 1, 2048, 2047)
     ctx = lva.Context(0)
     name, cus, hbm = ctx.info()
     emit(case="device", name=name, compute_units=cus, hbm_GiB=hbm >> 30)
@@ -506,10 +301,6 @@ def main():
         decode_case(ctx, "decode-7b-graph", "7b", lva.LV_Q4_0, 0, 512, 440, 68, force_path=lva.PATH_GRAPH)
     if which in ("prefill-13b", "all"):
         prefill_case(ctx, "prefill-13b", "13b", lva.LV_Q8_0)
-    if which == "decode-7b-power":
-        decode_power_case(ctx, "decode-7b-power")
-    if which == "prefill-13b-power":
-        prefill_power_case(ctx, "prefill-13b-power", "13b", lva.LV_Q8_0)
     if which in ("prefill-13b-q4", "all"):
         prefill_case(ctx, "prefill-13b-q4", "13b", lva.LV_Q4_0)
     if which in ("prefill-7b", "all"):
