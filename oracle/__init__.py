@@ -83,6 +83,7 @@ def lib():
         L.orc_session_kv_load.argtypes = [vp, u32, C.c_int, vp, u32]
         L.orc_session_set_pos.argtypes = [vp, u32]
         L.orc_num_threads.argtypes = []
+        L.orc_forward_f64.argtypes = [vp, vp, u32, u32, vp, vp, vp]
         _lib = L
     return _lib
 
@@ -213,6 +214,25 @@ class Model:
         t = self.tensor(name)
         addr = lib().orc_model_data(self.h, t["offset"])
         return np.ctypeslib.as_array(C.cast(addr, C.POINTER(C.c_uint8)), shape=(t["size"],)), t
+
+    def forward_f64(self, tokens, kv=None):
+        """logits of the last of `tokens` in double precision (new cache rows still rounded to fp16): the yardstick for
+        tolerances between fp32 implementations.  kv = None: a prompt from position 0; else a list with one (k_rows, v_rows)
+        pair of uint16 arrays [pos0][dim] per layer, the cache the tokens continue from."""
+        t = np.ascontiguousarray(tokens, dtype=np.uint32)
+        out = np.empty(self.hp["vocab"], dtype=np.float64)
+        pos0, kp, vp_ = 0, None, None
+        if kv is not None:
+            ks = [np.ascontiguousarray(k, dtype=np.uint16) for k, _ in kv]
+            vs = [np.ascontiguousarray(v, dtype=np.uint16) for _, v in kv]
+            pos0 = ks[0].shape[0]
+            assert len(ks) == self.hp["layers"] and all(a.shape == (pos0, self.hp["dim"]) for a in ks + vs)
+            kp = (C.c_void_p * len(ks))(*[a.ctypes.data for a in ks])
+            vp_ = (C.c_void_p * len(vs))(*[a.ctypes.data for a in vs])
+        rc = lib().orc_forward_f64(self.h, _p(t), t.shape[0], pos0, kp, vp_, _p(out))
+        if rc:
+            raise ValueError(f"orc_forward_f64 failed ({rc})")
+        return out
 
     def close(self):
         if self.h:

@@ -816,3 +816,176 @@ int orc_session_eval(orc_session *s, const uint32_t *tokens, uint32_t n, float *
     free(x); free(nrm); free(q); free(k); free(v); free(vo); free(ff); free(att); free(logits);
     return rc;
 }
+
+/* ------------------------------------------------------------------------------------------
+ * The yardstick for tolerances: the same step in double precision.
+ *
+ * Same operations in the same places as orc_session_eval (llava_layer.cpp:39-75, the shaders cited above), but every
+ * sum, product, exp, sin and cos in double, so that what is left is the result the formulas define plus the one
+ * rounding the reference's data format imposes: cache rows are fp16 (copy_to_cache.comp:35), rounded here once from
+ * the double value.  Two fp32 implementations that sum in different orders each stay within some distance of this
+ * result; a test that compares both with it can tell reassociation noise from a wrong kernel.  n tokens at positions
+ * pos0 .. pos0 + n - 1, logits of the last one; the cache rows 0 .. pos0 - 1 of every layer are the caller's (per-layer
+ * pointers to [pos0][dim] fp16 rows, taken as they are), so a long context can be continued from a copy of a cache.
+ * ---------------------------------------------------------------------------------------- */
+static uint16_t double_to_half(double d)
+{
+    float f = (float)d;
+    if ((double)f != d) { /* make f the round-to-odd value so that the second rounding is the only one that counts */
+        uint32_t u;
+        memcpy(&u, &f, 4);
+        if (fabs((double)f) > fabs(d))
+            u -= 1;
+        u |= 1u;
+        memcpy(&f, &u, 4);
+    }
+    return orc_float_to_half(f);
+}
+
+/* out[z][r] (+)= sum_k W[r][k] x[z][k] */
+static void gemm_f64(double *out, const orc_model *m, const orc_tensor *t, uint32_t rows, uint32_t cols, const double *x,
+                     uint32_t n, int accumulate)
+{
+    const uint32_t ver = m->hp.file_version;
+    const size_t row_bytes = orc_tensor_bytes(t->ftype, ver, cols);
+#pragma omp parallel
+    {
+        float *wf = (float *)malloc(sizeof(float) * cols);
+        double *wd = (double *)malloc(sizeof(double) * cols);
+#pragma omp for schedule(static)
+        for (uint32_t r = 0; r < rows; r++) {
+            orc_dequant((const uint8_t *)tdata(m, t) + (size_t)r * row_bytes, t->ftype, ver, wf, cols);
+            for (uint32_t k = 0; k < cols; k++)
+                wd[k] = (double)wf[k];
+            for (uint32_t z = 0; z < n; z++) {
+                const double *xz = x + (size_t)z * cols;
+                double a0 = 0, a1 = 0, a2 = 0, a3 = 0;
+                uint32_t k = 0;
+                for (; k + 4 <= cols; k += 4) {
+                    a0 += wd[k] * xz[k];
+                    a1 += wd[k + 1] * xz[k + 1];
+                    a2 += wd[k + 2] * xz[k + 2];
+                    a3 += wd[k + 3] * xz[k + 3];
+                }
+                for (; k < cols; k++)
+                    a0 += wd[k] * xz[k];
+                const double sum = (a0 + a1) + (a2 + a3);
+                double *o = out + (size_t)z * rows + r;
+                *o = accumulate ? *o + sum : sum;
+            }
+        }
+        free(wf);
+        free(wd);
+    }
+}
+
+static void normalize_f64(double *out, const double *x, const float *w, uint32_t dim, uint32_t n)
+{
+    for (uint32_t z = 0; z < n; z++) {
+        const double *xr = x + (size_t)z * dim;
+        double mean = 0, var = 0;
+        for (uint32_t i = 0; i < dim; i++)
+            mean += xr[i];
+        mean /= dim;
+        for (uint32_t i = 0; i < dim; i++)
+            var += (xr[i] - mean) * (xr[i] - mean);
+        const double inv = 1.0 / sqrt(var / dim); /* normalize.comp:34-64: centred variance, no epsilon, x itself not centred */
+        for (uint32_t i = 0; i < dim; i++)
+            out[(size_t)z * dim + i] = xr[i] * (double)w[i] * inv;
+    }
+}
+
+int orc_forward_f64(const orc_model *m, const uint32_t *tokens, uint32_t n, uint32_t pos0, const uint16_t *const *kcache,
+                    const uint16_t *const *vcache, double *logits_last)
+{
+    if (!m || !tokens || !logits_last || n == 0 || (pos0 && (!kcache || !vcache)))
+        return -1;
+    const uint32_t D = m->hp.dim, F = m->hp.ff, H = m->hp.heads, R = m->hp.rot, V = m->hp.vocab, half = R / 2;
+    const uint32_t ver = m->hp.file_version, T = pos0 + n;
+    const orc_tensor *tok = find_tensor(m, "tok_embeddings"), *normw = find_tensor(m, "norm"), *outw = find_tensor(m, "output");
+    if (!tok || !normw || !outw)
+        return -3;
+    for (uint32_t i = 0; i < n; i++)
+        if (tokens[i] >= V)
+            return -2;
+    double *x = (double *)malloc(sizeof(double) * n * D), *nrm = (double *)malloc(sizeof(double) * n * D);
+    double *q = (double *)malloc(sizeof(double) * n * D), *vo = (double *)malloc(sizeof(double) * n * D);
+    double *k = (double *)malloc(sizeof(double) * (size_t)T * D), *v = (double *)malloc(sizeof(double) * (size_t)T * D);
+    double *g1 = (double *)malloc(sizeof(double) * n * F), *g3 = (double *)malloc(sizeof(double) * n * F);
+    double *freq = (double *)malloc(sizeof(double) * half);
+    float *row = (float *)malloc(sizeof(float) * D);
+    int rc = 0;
+    for (uint32_t i = 0; i < half; i++)
+        freq[i] = pow(10000.0, -(double)i / (double)half);
+    const size_t row_bytes = tok->size / V;
+    for (uint32_t i = 0; i < n; i++) {
+        orc_dequant((const uint8_t *)tdata(m, tok) + (size_t)tokens[i] * row_bytes, tok->ftype, ver, row, D);
+        for (uint32_t j = 0; j < D; j++)
+            x[(size_t)i * D + j] = (double)row[j];
+    }
+    for (uint32_t li = 0; li < m->hp.layers && rc == 0; li++) {
+        const orc_tensor *wq = need(m, "layers.%u.attention.wq", li), *wk = need(m, "layers.%u.attention.wk", li);
+        const orc_tensor *wv = need(m, "layers.%u.attention.wv", li), *wo = need(m, "layers.%u.attention.wo", li);
+        const orc_tensor *w1 = need(m, "layers.%u.feed_forward.w1", li), *w2 = need(m, "layers.%u.feed_forward.w2", li);
+        const orc_tensor *w3 = need(m, "layers.%u.feed_forward.w3", li);
+        const orc_tensor *an = need(m, "layers.%u.attention_norm", li), *fn = need(m, "layers.%u.ffn_norm", li);
+        if (!wq || !wk || !wv || !wo || !w1 || !w2 || !w3 || !an || !fn) {
+            rc = -3;
+            break;
+        }
+        double *knew = k + (size_t)pos0 * D, *vnew = v + (size_t)pos0 * D;
+        for (size_t i = 0; i < (size_t)pos0 * D; i++) { /* rows the caller's cache already holds, as they are */
+            k[i] = (double)orc_half_to_float(kcache[li][i]);
+            v[i] = (double)orc_half_to_float(vcache[li][i]);
+        }
+        normalize_f64(nrm, x, (const float *)tdata(m, an), D, n);
+        gemm_f64(knew, m, wk, D, D, nrm, n, 0);
+        gemm_f64(q, m, wq, D, D, nrm, n, 0);
+        gemm_f64(vnew, m, wv, D, D, nrm, n, 0);
+        for (size_t i = 0; i < (size_t)n * D; i++) { /* the cache keeps fp16 (copy_to_cache.comp:35) */
+            knew[i] = (double)orc_half_to_float(double_to_half(knew[i]));
+            vnew[i] = (double)orc_half_to_float(double_to_half(vnew[i]));
+        }
+        /* mhsa.comp:32-60, softmax.comp:26-44, kqv_matching.comp:27-42: row z (position pos0 + z) over the rows p <= pos0 + z */
+#pragma omp parallel for schedule(dynamic, 1) collapse(2)
+        for (uint32_t z = 0; z < n; z++) {
+            for (uint32_t h = 0; h < H; h++) {
+                const uint32_t cur = pos0 + z;
+                double *a = (double *)malloc(sizeof(double) * (cur + 1));
+                const double *qr = q + (size_t)z * D + (size_t)h * R;
+                double total = 0;
+                for (uint32_t p = 0; p <= cur; p++) {
+                    const double *kr = k + (size_t)p * D + (size_t)h * R;
+                    double sc = 0;
+                    for (uint32_t i = 0; i < half; i++) {
+                        const double th = (double)(cur - p) * freq[i], ct = cos(th), st = sin(th);
+                        const double rx = ct * kr[2 * i] + st * kr[2 * i + 1], ry = -st * kr[2 * i] + ct * kr[2 * i + 1];
+                        sc += qr[2 * i] * rx + qr[2 * i + 1] * ry;
+                    }
+                    a[p] = exp(sc / sqrt((double)R));
+                    total += a[p];
+                }
+                for (uint32_t c = 0; c < R; c++) {
+                    double acc = 0;
+                    for (uint32_t p = 0; p <= cur; p++)
+                        acc += v[(size_t)p * D + (size_t)h * R + c] * (a[p] / total);
+                    vo[(size_t)z * D + (size_t)h * R + c] = acc;
+                }
+                free(a);
+            }
+        }
+        gemm_f64(x, m, wo, D, D, vo, n, 1);
+        normalize_f64(nrm, x, (const float *)tdata(m, fn), D, n);
+        gemm_f64(g3, m, w3, F, D, nrm, n, 0);
+        gemm_f64(g1, m, w1, F, D, nrm, n, 0);
+        for (size_t i = 0; i < (size_t)n * F; i++) /* matmul_silu_ff.comp:96 */
+            g3[i] = g3[i] * g1[i] / (exp(-g1[i]) + 1.0);
+        gemm_f64(x, m, w2, D, F, g3, n, 1);
+    }
+    if (rc == 0) {
+        normalize_f64(nrm, x + (size_t)(n - 1) * D, (const float *)tdata(m, normw), D, 1);
+        gemm_f64(logits_last, m, outw, V, D, nrm, 1, 0);
+    }
+    free(x); free(nrm); free(q); free(k); free(v); free(vo); free(g1); free(g3); free(freq); free(row);
+    return rc;
+}

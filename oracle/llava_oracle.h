@@ -22,6 +22,7 @@
  *                                                               self-consistency; token identity against
  *                                                               a run of the Vulkan binary: parity unpinned
  *   orc_sample_greedy ......................................... pinned (first strict max by construction)
+ *   orc_forward_f64 (double-precision yardstick) .............. pinned (independent numpy fp64 forward pass)
  */
 #ifndef LLAVA_ORACLE_H
 #define LLAVA_ORACLE_H
@@ -96,6 +97,13 @@ int orc_num_threads(void);
 /* per-layer intermediates of the LAST row of the last eval (trace); dim, ff or (which 5, the softmax weights
  * attn_result laid out [backlog][heads], llava_layer.cpp:60-61) backlog*heads floats */
 const float *orc_session_trace(const orc_session *s, uint32_t layer, int which, uint32_t *count);
+
+/* The same step in double precision: n tokens at positions pos0 .. pos0 + n - 1, logits of the last one.  Every sum,
+ * product, exp, sin and cos in double, new cache rows rounded once to fp16; rows 0 .. pos0 - 1 of layer l are
+ * kcache[l] / vcache[l] ([pos0][dim] fp16, may be null when pos0 is 0).  The yardstick two fp32 implementations are
+ * measured against where their own difference is at the tolerance (pinned by an independent numpy forward pass). */
+int orc_forward_f64(const orc_model *m, const uint32_t *tokens, uint32_t n, uint32_t pos0, const uint16_t *const *kcache,
+                    const uint16_t *const *vcache, double *logits_last);
 
 #ifdef __cplusplus
 }

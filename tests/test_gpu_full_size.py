@@ -178,6 +178,60 @@ def test_13b_q4_0_prompt_of_32_as_one_step_then_steps_on_graph_and_persistent_pa
     _prompt_then_steps_on_two_paths(lva, orc, ctx, path, SHAPE_13B, 32, seed=2, steps=8)
 
 
+def _checker_from_cache(orc, om, sess, layers, pos, backlog):
+    """a checker session that continues from a copy of the GPU session's first `pos` cache rows"""
+    o = orc.Session(om, backlog)
+    for layer in range(layers):
+        for which in (0, 1):
+            o.kv_load(layer, which, sess.kv(layer, which, pos))
+    o.set_pos(pos)
+    return o
+
+
+def test_13b_q4_0_256_greedy_steps_on_graph_and_persistent_paths(lva, orc, ctx):
+    """The whole length of the 13B q4_0 configuration: a 32-token prompt, then 256 greedy steps (positions 32..287) on the
+    hipGraph of the operator chain and on the persistent kernel side by side.  Every step the two paths have to pick the
+    same token; at steps 0..7, 128 and 255 the checker evaluates that step from a copy of the path's own cache rows and
+    the logits have to agree within the tolerance (the checker needs 0.4 s a token: following all 256 would take minutes)."""
+    path = _model_file(lva, "13b_q4_0", lva.LV_Q4_0, 2, SHAPE_13B)
+    om = orc.Model(path)
+    model = lva.Model(ctx, path)
+    L = SHAPE_13B["layers"]
+    graph, pers = lva.Session(model, 512), lva.Session(model, 512)
+    graph.set_path(lva.PATH_GRAPH)
+    prompt = lva.synth_tokens(32, 3, SHAPE_13B["vocab"], seed=2)
+    for s in (graph, pers):
+        s.begin(prompt, 0)
+    tok = pers.argmax()
+    assert graph.argmax() == tok
+    pos, worst = 32, 0.0
+    for step in range(256):
+        check = step < 8 or step in (128, 255)
+        if check:
+            want = {}
+            for label, s in (("graph", graph), ("persistent", pers)):
+                o = _checker_from_cache(orc, om, s, L, pos, 512)
+                want[label] = o.eval(np.array([tok], dtype=np.uint32))
+                o.close()
+        for s in (graph, pers):
+            s.begin([tok], pos)
+        if check:
+            for label, s in (("graph", graph), ("persistent", pers)):
+                got = s.logits()
+                err = float(np.max(np.abs(got - want[label]) / (1e-2 + 1e-3 * np.abs(want[label]))))
+                assert err <= 1.0, (label, step, err)
+                worst = max(worst, err)
+                assert s.argmax() == orc.greedy(want[label]), (label, step)
+        tg, tp = graph.argmax(), pers.argmax()
+        assert tg == tp, (step, tg, tp)
+        tok = tp
+        pos += 1
+    assert pos == 288
+    print(f"13B q4_0, 256 steps on two paths: same tokens throughout; worst checked error {worst:.2f} x tolerance")
+    for h in (graph, pers, model, om):
+        h.close()
+
+
 def test_7b_q4_0_prompt_of_128_as_one_step_then_steps(lva, orc, ctx, model_7b):
     """a 128-token prompt on the 7B q4_0 model: the q4_0 GEMM forms at K = 4096 and 11008 with full token tiles, checked
     against the oracle evaluating the 128 tokens itself"""
@@ -185,9 +239,11 @@ def test_7b_q4_0_prompt_of_128_as_one_step_then_steps(lva, orc, ctx, model_7b):
 
 
 def test_7b_q8_0_long_context_steps_match_oracle(lva, orc, ctx):
-    """7B q8_0 with the cache filled to position 1920 by the batched prompt path, then greedy steps on the persistent
-    kernel; the oracle continues from a copy of that cache (evaluating 1920 tokens on the CPU would take minutes), so
-    this pins the decode steps at a long context, not the prompt evaluation (tests/test_gpu_gemm.py does that)."""
+    """7B q8_0 with the cache filled to position 1920 by the batched prompt path, then the configuration's 128 greedy
+    steps (positions 1920..2047, the last row of a 2048-row cache) on the persistent kernel.  The checker follows steps
+    0..3 from a copy of the cache after the prompt (evaluating 1920 tokens on the CPU would take minutes), and evaluates
+    steps 64 and 127 from a copy of the cache as it stands then; so this pins the decode steps at a long context, not
+    the prompt evaluation (tests/test_gpu_gemm.py does that)."""
     path = _model_file(lva, "7b_q8_0", lva.LV_Q8_0, 1, SHAPE)
     model = lva.Model(ctx, path)
     s = lva.Session(model, 2048)
@@ -197,47 +253,110 @@ def test_7b_q8_0_long_context_steps_match_oracle(lva, orc, ctx):
     s.begin(prompt, 0)
     tok = s.argmax()
     om = orc.Model(path)
-    osess = orc.Session(om, 2048)
-    for layer in range(SHAPE["layers"]):
-        for which in (0, 1):
-            osess.kv_load(layer, which, s.kv(layer, which, first))
-    osess.set_pos(first)
+    osess = _checker_from_cache(orc, om, s, SHAPE["layers"], first, 2048)
     pos = first
-    for step in range(4):
-        want = osess.eval(np.array([tok], dtype=np.uint32))
+    for step in range(128):
+        if step in (64, 127):
+            osess = _checker_from_cache(orc, om, s, SHAPE["layers"], pos, 2048)
+        check = step < 4 or step in (64, 127)
+        if check:
+            want = osess.eval(np.array([tok], dtype=np.uint32))
         s.begin([tok], pos)
-        got = s.logits()
-        assert np.all(np.abs(got - want) <= 1e-2 + 1e-3 * np.abs(want)), (step, float(np.max(np.abs(got - want))))
-        tok = orc.greedy(want)
-        assert s.argmax() == tok, step
+        if check:
+            got = s.logits()
+            assert np.all(np.abs(got - want) <= 1e-2 + 1e-3 * np.abs(want)), (step, float(np.max(np.abs(got - want))))
+            assert s.argmax() == orc.greedy(want), step
+            if step in (3, 64):
+                osess.close()
+        tok = s.argmax()
         pos += 1
-    s.close(); model.close(); osess.close(); om.close()
+    assert pos == 2048
+    osess.close()
+    s.close(); model.close(); om.close()
+
+
+def _within(got, truth, factor=1.0):
+    """every logit within factor x (1e-2 absolute + 1e-3 relative) of `truth`; returns the largest error as a multiple of the tolerance"""
+    ratio = np.abs(np.asarray(got, dtype=np.float64) - truth) / (1e-2 + 1e-3 * np.abs(truth))
+    worst = float(np.max(ratio))
+    assert worst <= factor, worst
+    return worst
+
+
+def _rms(got, truth):
+    return float(np.sqrt(np.mean((np.asarray(got, dtype=np.float64) - truth) ** 2)))
 
 
 def test_13b_q8_0_prompt_of_512_as_one_batch(lva, orc, ctx):
-    """the prompt case at full size: 512 tokens through the matrix-core GEMM and the batched attention of a 40-layer 13B
-    q8_0 model.  The oracle would need minutes for all of it on the CPU, so the check is in three steps that together
-    reach it: (0) directly against the oracle on the first 32 tokens (their cache rows inside the 512-token batch, and
-    the logits of a 32-token batch); (1) the same 512 tokens evaluated one by one by the persistent kernel, whose steps are pinned against the
-    oracle (above, and at every tile shape in tests/test_gpu_model.py), must leave the same cache rows and logits
-    within TWICE the tolerance (two paths that each round fp16 cache rows their own way, 40 layers deep: if each is
-    within the tolerance of the exact result they are within twice of each other; measured: 0.004 typical, 0.018 the
-    worst of 32000 logits of magnitude 5); (2) from a copy of that cache the oracle itself evaluates the next token,
-    at the tolerance itself."""
+    """The prompt case at full size: 512 tokens through the matrix-core GEMM and the batched attention of a 40-layer 13B
+    q8_0 model.  This model is the least forgiving of the configurations: q8_0 codes up to 127 give every layer weights of
+    order 1, attention scores so large that the softmax picks single rows, logits up to 9 — and it amplifies fp32 rounding
+    ten-thousandfold: measured against the step in double precision (orc_forward_f64, pinned by an independent numpy
+    forward pass) on the first 32 tokens, the CPU checker itself, which follows the shaders' own summation order, is 0.0023
+    rms and 0.88 x the tolerance at the worst of its 32000 logits away; the persistent kernel 0.0026 rms / 1.00 x, the
+    operator chain 0.0026 / 1.07 x, the batched path 0.0029 / 1.08 x.  The tolerance of 1e-2 + 1e-3 |l| is four standard
+    deviations of that noise, so two fp32 evaluations that sum in different orders cannot be held to it against each other
+    (expected worst of 32000: 0.014), and none can be held to it against the exact result more firmly than the checker is.
+    What is asserted instead says that the GPU's error IS that noise and nothing else:
+    (0) first 32 tokens, against double precision: the checker within the tolerance; the 32-token batch and the
+        persistent kernel token by token no noisier than 1.3 x the checker's rms error and nowhere beyond 1.25 x the
+        tolerance; GPU against checker within twice the tolerance (which follows), greedy token the same for all four;
+        the first 32 cache rows inside the 512-token batch against the checker's;
+    (1) all 512 tokens as one batch and token by token: each path's logits within the tolerance of the double-precision
+        evaluation of the last token on top of that path's own 511 cache rows (evaluating all 512 rows in double would
+        take minutes; a single step does not amplify), the cache rows of the two paths against each other;
+    (2) from a copy of the batch path's cache the checker evaluates the next token, at the tolerance itself."""
     path = _model_file(lva, "13b_q8_0", lva.LV_Q8_0, 3, SHAPE_13B)
     model = lva.Model(ctx, path)
+    om = orc.Model(path)
+    L = SHAPE_13B["layers"]
     n = 512
     prompt = lva.synth_tokens(n, 3, SHAPE_13B["vocab"], seed=3)
     batch, single = lva.Session(model, 1024), lva.Session(model, 1024)
     assert single.path() == lva.PATH_PERSISTENT
     batch.begin(prompt, 0)
     got = batch.logits().copy()
+    single_head = None
     for i in range(n):
         single.begin(prompt[i:i + 1], i)
         single.wait()
+        if i == 31:
+            single_head = single.logits().copy()
     want = single.logits().copy()
-    assert np.all(np.abs(got - want) <= 2 * (1e-2 + 1e-3 * np.abs(want))), float(np.max(np.abs(got - want)))
     assert batch.argmax() == single.argmax()
+
+    # (0) the first 32 tokens against the double-precision step
+    truth32 = om.forward_f64(prompt[:32])
+    ohead = orc.Session(om, 128)
+    head_want = ohead.eval(prompt[:32])
+    head = lva.Session(model, 128)
+    head.begin(prompt[:32], 0)
+    head_got = head.logits()
+    d_checker, r_checker = _within(head_want, truth32), _rms(head_want, truth32)
+    report = [f"checker {d_checker:.2f} x tolerance at worst, rms {r_checker:.4f}"]
+    for label, logits in (("32-token batch", head_got), ("persistent kernel", single_head)):
+        d, r = _within(logits, truth32, 1.25), _rms(logits, truth32)
+        assert r <= 1.3 * r_checker, (label, r, r_checker)
+        between = _within(logits, head_want.astype(np.float64), 2.0)
+        report.append(f"{label} {d:.2f} x, rms {r:.4f}, against the checker {between:.2f} x")
+    print("32 tokens against double precision: " + "; ".join(report))
+    assert head.argmax() == orc.greedy(head_want) == int(np.argmax(truth32))
+    for layer, bound in ((0, 2.0 ** -10), (19, 4e-3), (39, 4e-3)):
+        for which in (0, 1):
+            b = ohead.kv(layer, which, 32).view(np.float16).astype(np.float32)
+            for rows in (batch.kv(layer, which, 32), head.kv(layer, which, 32)):
+                a = rows.view(np.float16).astype(np.float32)
+                assert float(np.max(np.abs(a - b))) <= bound * float(np.max(np.abs(b))), (layer, which)
+    head.close(); ohead.close()
+
+    # (1) 512 tokens: each path against the double-precision evaluation of the last token on its own cache
+    for label, sess, logits in (("batch", batch, got), ("token by token", single, want)):
+        kv = [(sess.kv(layer, 0, n - 1), sess.kv(layer, 1, n - 1)) for layer in range(L)]
+        truth = om.forward_f64(prompt[n - 1:], kv=kv)
+        worst = _within(logits, truth)
+        print(f"512 tokens, {label}: worst error / tolerance against double precision on its own cache {worst:.2f}")
+        del kv
+    _within(got, want.astype(np.float64), 2.0)
     # cache rows: fp16 values of fp32 sums taken in two different orders; they may differ by an fp16 ulp where a sum
     # falls near a rounding boundary, and by more only through error carried from layer to layer
     for layer, bound in ((0, 2.0 ** -10), (19, 1e-2), (39, 1e-2)):
@@ -246,33 +365,10 @@ def test_13b_q8_0_prompt_of_512_as_one_batch(lva, orc, ctx):
             b = single.kv(layer, which, n).view(np.float16).astype(np.float32)
             worst = float(np.max(np.abs(a - b))) / float(np.max(np.abs(b)))
             assert worst <= bound, (layer, which, worst)
-    # directly against the oracle on a prefix the CPU can afford: the first 32 cache rows of the 512-token batch (causal:
-    # later tokens do not change them), and the logits of a 32-token batch of its own
-    om = orc.Model(path)
-    ohead = orc.Session(om, 128)
-    head_want = ohead.eval(prompt[:32])
-    head = lva.Session(model, 128)
-    head.begin(prompt[:32], 0)
-    head_got = head.logits()
-    # This model is the least forgiving of the configurations: q8_0 codes up to 127 give every layer weights of order 1,
-    # attention scores so large that the softmax picks single rows, and logits up to 9.  The persistent kernel, whose
-    # arithmetic is fp32 throughout, leaves one of the 32000 logits a hair beyond the tolerance here (0.0110 against
-    # 0.0108); the batch path about ten, none beyond 0.0135.  Hence: all within 1.5 x the tolerance, at most 32 (0.1 %)
-    # beyond the tolerance itself, the greedy token identical.
-    err, tol = np.abs(head_got - head_want), 1e-2 + 1e-3 * np.abs(head_want)
-    assert np.all(err <= 1.5 * tol), float(np.max(err))
-    assert int(np.sum(err > tol)) <= 32, int(np.sum(err > tol))
-    assert head.argmax() == orc.greedy(head_want)
-    for layer, bound in ((0, 2.0 ** -10), (19, 4e-3), (39, 4e-3)):
-        for which in (0, 1):
-            b = ohead.kv(layer, which, 32).view(np.float16).astype(np.float32)
-            for rows in (batch.kv(layer, which, 32), head.kv(layer, which, 32)):
-                a = rows.view(np.float16).astype(np.float32)
-                assert float(np.max(np.abs(a - b))) <= bound * float(np.max(np.abs(b))), (layer, which)
-    head.close(); ohead.close()
-    # the oracle continues from the batch path's cache
+
+    # (2) the checker continues from the batch path's cache
     osess = orc.Session(om, 1024)
-    for layer in range(SHAPE_13B["layers"]):
+    for layer in range(L):
         for which in (0, 1):
             osess.kv_load(layer, which, batch.kv(layer, which, n))
     osess.set_pos(n)

@@ -49,6 +49,9 @@ def test_dequant_bit_exact(lva, orc, ctx, ftype_name, rows, cols):
     # 2048 rows and more: the streaming kernel (256 workgroups, x in LDS); ragged row counts, 1..12 column slabs per
     # row (24576 columns is the widest row the library accepts)
     (2048, 32, 1), (2049, 2048 + 64, 2), (4096, 4096, 1), (2500, 11008, 1), (2051, 13824, 3), (2048, 24576, 1),
+    # the decode shapes the isolated-kernel figures are quoted on, whole: down projection (with accumulate = the fused
+    # residual add) and output matrix of the 7B model, and the 13B down projection
+    (4096, 11008, 1), (32000, 4096, 1), (5120, 13824, 1),
 ])
 @pytest.mark.parametrize("accumulate", [False, True])
 def test_gemv_matches_oracle(lva, orc, ctx, ftype_name, rows, cols, batch, accumulate):

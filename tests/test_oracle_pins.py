@@ -324,7 +324,7 @@ def test_greedy_is_first_strict_maximum(orc):
 # whole step: an independent fp64 forward pass (textbook RoPE on q and k, standard softmax, SwiGLU, the
 # reference's centred-variance normalisation) on a tiny seeded model
 # ---------------------------------------------------------------------------------------------------------------
-def _forward_np(orc_model, tokens):
+def _forward_np(orc_model, tokens, half_from_double=False):
     hp = orc_model.hp
     D, H, R, L, V = hp["dim"], hp["heads"], hp["rot"], hp["layers"], hp["vocab"]
 
@@ -347,8 +347,11 @@ def _forward_np(orc_model, tokens):
         p = f"layers.{l}."
         h = norm(x, vec(p + "attention_norm"))
         q, k, v = h @ mat(p + "attention.wq").T, h @ mat(p + "attention.wk").T, h @ mat(p + "attention.wv").T
-        k16 = k.astype(np.float32).astype(np.float16).astype(np.float64)       # the cache keeps fp16
-        v16 = v.astype(np.float32).astype(np.float16).astype(np.float64)
+        if half_from_double:     # one rounding, from the double value (what orc_forward_f64 does)
+            k16, v16 = k.astype(np.float16).astype(np.float64), v.astype(np.float16).astype(np.float64)
+        else:                    # the cache keeps fp16, rounded from an fp32 value as in the shader
+            k16 = k.astype(np.float32).astype(np.float16).astype(np.float64)
+            v16 = v.astype(np.float32).astype(np.float16).astype(np.float64)
         kcache.append(k16.astype(np.float16)); vcache.append(v16.astype(np.float16))
         o = np.zeros_like(x)
         for z in range(n):
@@ -379,6 +382,32 @@ def test_whole_step_against_independent_forward_pass(lva, orc, tiny_models, name
         gv = s.kv(layer, 1, 9).view(np.float16).astype(np.float32)
         assert np.max(np.abs(gk - kc[layer].astype(np.float32))) <= np.max(np.abs(gk)) * 2.0 ** -9
         assert np.max(np.abs(gv - vc[layer].astype(np.float32))) <= np.max(np.abs(gv)) * 2.0 ** -9
+    s.close()
+    om.close()
+
+
+@pytest.mark.parametrize("name", ["tiny_q4", "tiny_q8", "small_q4"])
+def test_double_precision_yardstick_against_independent_forward_pass(lva, orc, tiny_models, name):
+    """orc_forward_f64 is what the full-size tests measure both the GPU and the fp32 checker against: it has to be the
+    formulas' own result.  Pinned by the numpy forward pass above (textbook RoPE on q and k separately, scipy softmax with
+    max subtraction, numpy std), which shares no code with it; both are double and round cache rows to fp16 once, from the
+    double value, so they agree to the rounding of double sums (a cache value within 1e-16 of an fp16 rounding boundary
+    could flip an ulp: not seen with these seeds)."""
+    om = orc.Model(tiny_models[name])
+    toks = lva.synth_tokens(9, 3, om.hp["vocab"], seed=11)
+    want, _, _ = _forward_np(om, toks, half_from_double=True)
+    got = om.forward_f64(toks)
+    scale = np.max(np.abs(want[-1]))
+    assert np.max(np.abs(got - want[-1])) <= 1e-12 * scale
+    # and the fp32 checker sits within fp32 rounding of it
+    s = orc.Session(om, 128)
+    f32 = s.eval(toks)
+    assert np.max(np.abs(f32 - got)) <= 2e-4 * scale
+    # continued from a cache: the last three tokens on top of the first six rows of the checker's cache give what the
+    # checker's own continuation gives (to fp32 rounding), and exactly the whole-prompt result when the rows are its own
+    kv = [(s.kv(l, 0, 6), s.kv(l, 1, 6)) for l in range(om.hp["layers"])]
+    cont = om.forward_f64(toks[6:], kv=kv)
+    assert np.max(np.abs(cont - f32)) <= 2e-4 * scale
     s.close()
     om.close()
 
