@@ -166,6 +166,10 @@ int lv_dev_download(lv_ctx *ctx, void *dst, const void *dptr, uint64_t bytes);
 int lv_dev_zero(lv_ctx *ctx, void *dptr, uint64_t bytes);
 /* device-to-device copy on the context's stream (asynchronous); size and pointers multiples of 16 */
 int lv_dev_copy(lv_ctx *ctx, void *dst, const void *src, uint64_t bytes);
+/* read-only pass over device memory on the context's stream (asynchronous), the result discarded: with lv_ctx_timer_* it
+ * gives the read bandwidth this device reaches, the denominator a weight-streaming kernel is also measured against
+ * (no counterpart in the reference: a measuring aid like the timers); size and pointer multiples of 16 */
+int lv_dev_read(lv_ctx *ctx, const void *src, uint64_t bytes);
 int lv_ctx_sync(lv_ctx *ctx);
 
 /* ---- GPU time between two points of a stream, by HIP events recorded on that very stream (the reference has

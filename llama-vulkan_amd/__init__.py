@@ -111,6 +111,7 @@ _HIP_SIGS = {
     "lv_dev_download": [_VP, _VP, _VP, _U64],
     "lv_dev_zero": [_VP, _VP, _U64],
     "lv_dev_copy": [_VP, _VP, _VP, _U64],
+    "lv_dev_read": [_VP, _VP, _U64],
     "lv_matrix_upload": [_VP, _VP, _U32, _U32, _U32, _U32, C.POINTER(_VP)],
     "lv_matrix_destroy": [_VP],
     "lv_matrix_bytes": [_VP, C.POINTER(_U64)],

@@ -14,6 +14,7 @@
     python llama-vulkan_amd/measure.py prefill-13b-q4  13B q4_0, the same
     python llama-vulkan_amd/measure.py gemm          isolated 512-token GEMMs at the 13B shapes, q8_0 (for kernel traces and counters)
     python llama-vulkan_amd/measure.py copy          1 GiB device-to-device copy: achievable bandwidth, counter calibration
+    python llama-vulkan_amd/measure.py read-stream   4 GiB read by a kernel that only reads: the bandwidth a weight stream can reach
     python llama-vulkan_amd/measure.py all
 
 Every figure is algorithmic bytes (weights as stored in the GGML file, 18 B / 34 B per 32 weights, plus vectors and the
@@ -34,7 +35,7 @@ SHAPES = {"7b": dict(vocab=32000, dim=4096, heads=32, layers=32, ff=11008), "13b
 
 
 def emit(**kw):
-    print(json.dumps(kw), flush=True)
+    print(json.dumps({k: v for k, v in kw.items() if k != "picks"}), flush=True)
     return kw
 
 
@@ -167,6 +168,23 @@ def copy_case(ctx):
     ctx.free(dst)
 
 
+def read_stream_case(ctx, report=emit, gib=4):
+    """What a kernel that only reads memory reaches on this device (lv_dev_read: contiguous share per workgroup, 16-byte
+    non-temporal loads, eight in flight): a buffer far larger than the 256 MB last-level cache, read 8 times.  The decode
+    kernel's bytes per second are reported against this figure as well as against the 8 TB/s of the datasheet."""
+    n = gib << 30
+    src = ctx.zeros(n)
+    lva.check(ctx.lib.lv_dev_read(ctx.h, src, n))
+    ctx.sync()
+    reps = 8
+    ctx.timer_start()
+    for _ in range(reps):
+        lva.check(ctx.lib.lv_dev_read(ctx.h, src, n))
+    ms = ctx.timer_stop() / reps
+    ctx.free(src)
+    return report(case="read-stream", bytes_read=n, ms=round(ms, 4), GBps=round(n / ms / 1e6, 1), frac_of_peak=round(n / ms / 1e6 / HBM_PEAK_GBS, 4))
+
+
 def model_file(preset, wtype, seed):
     base = "/dev/shm" if os.access("/dev/shm", os.W_OK) else "/tmp"
     path = os.path.join(base, f"llava_measure_{preset}_{'q4_0' if wtype == lva.LV_Q4_0 else 'q8_0'}_seed{seed}.ggml")
@@ -184,7 +202,7 @@ def step_bytes(shape, wtype, pos):
     return L * per_layer + V * D // 32 * block_bytes(wtype) + (2 * L + 1) * D * 4 + L * 2 * D * 2 * (pos + 2) + V * 4 + D * 4
 
 
-def decode_case(ctx, name, preset, wtype, seed, backlog, first, steps, force_path=None, report=emit):
+def decode_case(ctx, name, preset, wtype, seed, backlog, first, steps, force_path=None, report=emit, expect_picks=None):
     shape = SHAPES[preset]
     path = model_file(preset, wtype, seed)
     model = lva.Model(ctx, path)
@@ -198,23 +216,34 @@ def decode_case(ctx, name, preset, wtype, seed, backlog, first, steps, force_pat
     tok = s.argmax()
     prefill_s = time.perf_counter() - t0
     pos = first
+    picks = [tok]                      # picks[k] is the token fed at position first + k
     for _ in range(4):
         s.begin([tok], pos)
         tok = s.argmax()
+        picks.append(tok)
         pos += 1
     t0 = time.perf_counter()
     total = 0
     for _ in range(steps):
         s.begin([tok], pos)
         tok = s.argmax()
+        picks.append(tok)
         total += step_bytes(shape, wtype, pos)
         pos += 1
     dt = time.perf_counter() - t0
+    if expect_picks is not None:       # another path's run of the same case: the greedy continuation has to be the same
+        n = min(len(expect_picks), len(picks))
+        diff = [k for k in range(n) if picks[k] != expect_picks[k]]
+        if diff:
+            raise RuntimeError(f"{name}: greedy token at position {first + diff[0]} differs from the other path's ({picks[diff[0]]} vs {expect_picks[diff[0]]})")
     r = report(case=name, model=preset, wtype="q4_0" if wtype == lva.LV_Q4_0 else "q8_0", path=kind, positions=[first + 4, pos - 1], steps=steps,
                tok_s=round(steps / dt, 1), ms_per_token=round(dt / steps * 1e3, 4), GBps=round(total / dt / 1e9, 1),
-               frac_of_peak=round(total / dt / 1e9 / HBM_PEAK_GBS, 4), prompt_tokens=first, prompt_s=round(prefill_s, 3))
+               frac_of_peak=round(total / dt / 1e9 / HBM_PEAK_GBS, 4), prompt_tokens=first, prompt_s=round(prefill_s, 3),
+               same_picks_as_other_path=None if expect_picks is None else True)
     s.close()
     model.close()
+    r = dict(r)
+    r["picks"] = picks
     return r
 
 
@@ -234,10 +263,11 @@ def prefill_case(ctx, case, name, wtype, report=emit):
     ms = s.timer_stop()
     D, F, V, L = shape["dim"], shape["ff"], shape["vocab"], shape["layers"]
     flops = 2.0 * 512 * L * (4 * D * D + 3 * D * F) + 2.0 * V * D      # the output matrix sees the last row only
-    # every product is executed twice (activations are a pair of halves), so the matrix cores run at twice the useful rate
+    # frac_of_mfma_peak counts the flops the prompt needs (2 per weight and token); the GEMM executes every product twice
+    # (activations are a pair of fp16 halves), so the matrix cores run at twice that rate: executed_frac
     r = report(case=case, model=name, wtype="q4_0" if wtype == lva.LV_Q4_0 else "q8_0", tokens=512, ms=round(ms, 2),
                tok_s=round(512 / ms * 1e3, 1), TFLOPs=round(flops / ms / 1e9, 2), executed_TFLOPs=round(2 * flops / ms / 1e9, 2),
-               frac_of_mfma_peak=round(2 * flops / ms / 1e9 / MFMA_PEAK_TFLOPS, 4))
+               frac_of_mfma_peak=round(flops / ms / 1e9 / MFMA_PEAK_TFLOPS, 4), executed_frac=round(2 * flops / ms / 1e9 / MFMA_PEAK_TFLOPS, 4))
     s.close()
     model.close()
     return r
@@ -265,7 +295,7 @@ def gemm_cases(ctx, report=emit):
         useful = 2.0 * n * rows * cols / us / 1e6
         out_cases.append(report(case="gemm", wtype="q8_0", rows=rows, cols=cols, tokens=n, launches=reps, us=round(us, 1),
                                 useful_TFLOPs=round(useful, 1), executed_TFLOPs=round(2 * useful, 1),
-                                executed_frac_of_peak=round(2 * useful / MFMA_PEAK_TFLOPS, 4)))
+                                frac_of_mfma_peak=round(useful / MFMA_PEAK_TFLOPS, 4), executed_frac=round(2 * useful / MFMA_PEAK_TFLOPS, 4)))
         ctx.matrix_free(m)
         ctx.free(x)
         ctx.free(out)
@@ -279,6 +309,8 @@ def main():
     emit(case="device", name=name, compute_units=cus, hbm_GiB=hbm >> 30)
     if which in ("copy", "all"):
         copy_case(ctx)
+    if which in ("read-stream", "all"):
+        read_stream_case(ctx)
     if which in ("gemv", "all"):
         gemv_cases(ctx)
     if which == "gemv-13b":
@@ -305,6 +337,7 @@ def main():
         prefill_case(ctx, "prefill-13b-q4", "13b", lva.LV_Q4_0)
     if which in ("prefill-7b", "all"):
         prefill_case(ctx, "prefill-7b", "7b", lva.LV_Q4_0)
+    ctx.close()       # nothing of the library is left to the interpreter's exit
 
 
 if __name__ == "__main__":
