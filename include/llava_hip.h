@@ -109,7 +109,7 @@ int lv_session_use_graph(lv_session *s, int enable);
  *                       256-CU device)
  *   LV_PATH_AUTO        persistent when the model has that form, else graph (or kernels if graphs are off)
  * A session stops using the persistent kernel, and lv_session_path reports the graph path (kernels if graphs are off)
- * from then on, when the runtime refuses its cooperative launch (the step goes on in the other path and succeeds) or when
+ * from then on, when its 256 workgroups cannot all be resident on the device (the step goes on in the other path and succeeds) or when
  * two steps in a row end with an expired hand-over wait (both report LV_ERR_HIP; the step issued again then succeeds).
  * lv_session_set_path(LV_PATH_PERSISTENT) gives the kernel another try. */
 enum { LV_PATH_AUTO = 0, LV_PATH_KERNELS = 1, LV_PATH_GRAPH = 2, LV_PATH_PERSISTENT = 3 };
@@ -225,6 +225,8 @@ int lv_kernel_attention(lv_ctx *ctx, float *out, const void *kcache, const void 
  * table, the partial sums and the split counters live in a fixed 2 MiB work area that every device holds from library
  * load to process end, so the call allocates nothing and frees nothing.  Limits (LV_ERR_RANGE beyond them):
  * backlog * rot / 2 <= 131072, batch * heads * ceil(backlog / 64) * (rot + 1) <= 262144, batch * heads <= 256.
+ * Every call rewrites the rotation table for its backlog and head size (a small kernel in front of the attention: up to
+ * 1 MiB written) and clears the split counters, so nothing is carried from call to call.
  * All calls on one device share the work area: calls that overlap on one device (different contexts, different threads)
  * race; calls on one context are ordered by its stream. */
 int lv_kernel_attention_static(lv_ctx *ctx, float *out, const void *kcache, const void *vcache, const float *q,

@@ -85,6 +85,7 @@ struct lv_ctx {
     std::mutex mega_mutex;
     hipEvent_t mega_done = nullptr;
     const void *mega_last = nullptr;      // session whose launch mega_done belongs to
+    int mega_fits[8] = {-1, -1, -1, -1, -1, -1, -1, -1};   // per shape class of the persistent kernel: can all its workgroups be resident at once (-1 = not asked yet)
 };
 
 struct lv_matrix {
@@ -1704,9 +1705,14 @@ extern "C" int lv_session_path(const lv_session *s, int *path)
     return LV_OK;
 }
 
-// One token through the persistent kernel.  *refused is set, and LV_OK returned, when the runtime will not launch the
-// grid cooperatively (its 256 workgroups cannot all be resident: another process holds part of the device, or the
-// device is smaller than the kernel was built for); nothing has run then.
+// One token through the persistent kernel.  Its workgroups hand vectors to each other, so all 256 of them have to be
+// resident at once: one per CU, on a device of at least 256 CUs that grants the kernel a workgroup per CU (lv_ctx::mega_fits
+// asks the runtime once per shape class).  *refused is set, and LV_OK returned, when that does not hold or the launch is
+// turned down for lack of resources; nothing has run then.  The launch is an ordinary one: hipLaunchCooperativeKernel's own
+// test is the same occupancy arithmetic and adds nothing to it (kernels of other streams can hold CUs for a while under
+// either; the waits inside the kernel are bounded for that), the two launch at the same rate (measured in alternation), and
+// the separate queue the runtime opens for cooperative launches makes a process under rocprofv3 end with a segmentation
+// fault in its exit handlers (a forty-line program with one cooperative launch of an empty kernel does the same).
 static int launch_mega(lv_session *s, uint32_t pos, uint32_t token, bool *refused)
 {
     const lv_model *m = s->model;
@@ -1732,9 +1738,20 @@ static int launch_mega(lv_session *s, uint32_t pos, uint32_t token, bool *refuse
     if (c->mega_last && c->mega_last != s) HIP_TRY(hipStreamWaitEvent(s->stream, c->mega_done, 0));
     LV_TRY(mega_dispatch(m->mega_kind, [&](auto shape) -> int {
         using S = decltype(shape);
-        const hipError_t e = hipLaunchCooperativeKernel(reinterpret_cast<const void *>(&mega_decode_kernel<S>), dim3(kMegaWGs), dim3(S::NW * 64),
-                                                        params, 0, s->stream);
-        if (e == hipErrorCooperativeLaunchTooLarge || e == hipErrorLaunchOutOfResources || e == hipErrorNotSupported) {
+        const void *kernel = reinterpret_cast<const void *>(&mega_decode_kernel<S>);
+        int &fits = c->mega_fits[m->mega_kind];
+        if (fits < 0) {
+            int per_cu = 0;
+            const hipError_t oe = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, S::NW * 64, 0);
+            if (oe != hipSuccess) (void)hipGetLastError();
+            fits = oe == hipSuccess && per_cu >= 1 && c->props.multiProcessorCount >= kMegaWGs ? 1 : 0;
+        }
+        if (!fits) {
+            *refused = true;
+            return LV_OK;
+        }
+        const hipError_t e = hipLaunchKernel(kernel, dim3(kMegaWGs), dim3(S::NW * 64), params, 0, s->stream);
+        if (e == hipErrorLaunchOutOfResources || e == hipErrorNotSupported) {
             (void)hipGetLastError();
             *refused = true;
             return LV_OK;

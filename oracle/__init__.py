@@ -84,6 +84,8 @@ def lib():
         L.orc_session_set_pos.argtypes = [vp, u32]
         L.orc_num_threads.argtypes = []
         L.orc_forward_f64.argtypes = [vp, vp, u32, u32, vp, vp, vp]
+        L.orc_forward_f64_activation_bits.argtypes = [C.c_int]
+        L.orc_forward_f64_activation_bits.restype = None
         _lib = L
     return _lib
 
@@ -215,7 +217,7 @@ class Model:
         addr = lib().orc_model_data(self.h, t["offset"])
         return np.ctypeslib.as_array(C.cast(addr, C.POINTER(C.c_uint8)), shape=(t["size"],)), t
 
-    def forward_f64(self, tokens, kv=None):
+    def forward_f64(self, tokens, kv=None, activation_bits=0):
         """logits of the last of `tokens` in double precision (new cache rows still rounded to fp16): the yardstick for
         tolerances between fp32 implementations.  kv = None: a prompt from position 0; else a list with one (k_rows, v_rows)
         pair of uint16 arrays [pos0][dim] per layer, the cache the tokens continue from."""
@@ -229,7 +231,9 @@ class Model:
             assert len(ks) == self.hp["layers"] and all(a.shape == (pos0, self.hp["dim"]) for a in ks + vs)
             kp = (C.c_void_p * len(ks))(*[a.ctypes.data for a in ks])
             vp_ = (C.c_void_p * len(vs))(*[a.ctypes.data for a in vs])
+        lib().orc_forward_f64_activation_bits(activation_bits)   # > 0: GEMM inputs quantised per block to that many bits (experiment)
         rc = lib().orc_forward_f64(self.h, _p(t), t.shape[0], pos0, kp, vp_, _p(out))
+        lib().orc_forward_f64_activation_bits(0)
         if rc:
             raise ValueError(f"orc_forward_f64 failed ({rc})")
         return out

@@ -842,12 +842,40 @@ static uint16_t double_to_half(double d)
     return orc_float_to_half(f);
 }
 
+/* Experiment knob (0 = off, the yardstick proper): every GEMM input row is first quantised block by block (32 elements) to
+ * signed integers of this many bits with one scale per block, s = max|x| / (2^(bits-1) - 1), x' = s * rint(x / s) -- what a
+ * kernel that multiplies integer codes by integer activations on the int8 matrix cores would feed them (8 bits), everything
+ * else staying exact.  The logits' distance from the unquantised run is the price of that kernel, measured without building it. */
+static int g_act_bits = 0;
+void orc_forward_f64_activation_bits(int bits) { g_act_bits = bits; }
+
+static const double *quantised_rows(const double *x, uint32_t cols, uint32_t n, double **owned)
+{
+    *owned = NULL;
+    if (g_act_bits <= 1 || cols % 32)
+        return x;
+    double *y = (double *)malloc(sizeof(double) * (size_t)n * cols);
+    const double top = (double)((1u << (g_act_bits - 1)) - 1);
+    for (size_t b = 0; b < (size_t)n * cols / 32; b++) {
+        double mx = 0;
+        for (int j = 0; j < 32; j++)
+            mx = fmax(mx, fabs(x[b * 32 + j]));
+        const double sc = mx / top;
+        for (int j = 0; j < 32; j++)
+            y[b * 32 + j] = sc > 0 ? sc * rint(x[b * 32 + j] / sc) : 0.0;
+    }
+    *owned = y;
+    return y;
+}
+
 /* out[z][r] (+)= sum_k W[r][k] x[z][k] */
-static void gemm_f64(double *out, const orc_model *m, const orc_tensor *t, uint32_t rows, uint32_t cols, const double *x,
+static void gemm_f64(double *out, const orc_model *m, const orc_tensor *t, uint32_t rows, uint32_t cols, const double *x_in,
                      uint32_t n, int accumulate)
 {
     const uint32_t ver = m->hp.file_version;
     const size_t row_bytes = orc_tensor_bytes(t->ftype, ver, cols);
+    double *owned;
+    const double *x = quantised_rows(x_in, cols, n, &owned);
 #pragma omp parallel
     {
         float *wf = (float *)malloc(sizeof(float) * cols);
@@ -877,6 +905,7 @@ static void gemm_f64(double *out, const orc_model *m, const orc_tensor *t, uint3
         free(wf);
         free(wd);
     }
+    free(owned);
 }
 
 static void normalize_f64(double *out, const double *x, const float *w, uint32_t dim, uint32_t n)

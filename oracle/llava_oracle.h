@@ -105,6 +105,10 @@ const float *orc_session_trace(const orc_session *s, uint32_t layer, int which, 
 int orc_forward_f64(const orc_model *m, const uint32_t *tokens, uint32_t n, uint32_t pos0, const uint16_t *const *kcache,
                     const uint16_t *const *vcache, double *logits_last);
 
+/* experiment knob of orc_forward_f64 (0 = off): quantise every GEMM input row per block of 32 to signed integers of `bits`
+ * bits, as a kernel on the int8 matrix cores would; the logits' distance from the unquantised run prices such a kernel */
+void orc_forward_f64_activation_bits(int bits);
+
 #ifdef __cplusplus
 }
 #endif

@@ -97,6 +97,33 @@ def test_7b_operator_chain_agrees_with_persistent_kernel(lva, ctx, model_7b):
 SHAPE_13B = dict(vocab=32000, dim=5120, heads=40, layers=40, ff=13824)
 
 
+@pytest.mark.parametrize("name,steps", [("7b", 300), ("13b", 150)])
+def test_hand_overs_inside_an_xcd_and_at_device_scope_give_the_same_bits_at_full_depth(lva, ctx, model_7b, name, steps):
+    """The hand-overs inside a head go through the XCD's L2 with plain stores and non-temporal loads where a launch places the
+    head's workgroups on one XCD, at device scope otherwise.  Only the transport differs, so every logit of every step has
+    to be the same bits, here over a few hundred steps of the full-depth 7B and 13B q4_0 models (a stale value read through
+    the short way would change a logit; a value that never arrives ends the step with an error instead).  Stops at the first
+    difference."""
+    path = model_7b if name == "7b" else _model_file(lva, "13b_q4_0", lva.LV_Q4_0, 2, SHAPE_13B)
+    shape = SHAPE if name == "7b" else SHAPE_13B
+    model = lva.Model(ctx, path)
+    a, b = lva.Session(model, 512), lva.Session(model, 512)
+    b.set_xcd_handover(False)
+    tok, inside = 17, 0
+    for i in range(steps):
+        a.begin([tok], i)
+        la = a.logits()
+        inside += a.xcd_handover()
+        b.begin([tok], i)
+        lb = b.logits()
+        assert not b.xcd_handover()
+        assert np.array_equal(la.view(np.uint32), lb.view(np.uint32)), (name, i)
+        tok = a.argmax()
+        assert tok == b.argmax() and tok < shape["vocab"]
+    print(f"{name}: {inside} of {steps} steps handed over inside an XCD")
+    a.close(); b.close(); model.close()
+
+
 def _model_file(lva, name, wtype, seed, shape):
     base = "/dev/shm" if os.access("/dev/shm", os.W_OK) else "/tmp"
     path = os.path.join(base, f"llava_measure_{name}_seed{seed}.ggml")     # shared with llama-vulkan_amd/measure.py

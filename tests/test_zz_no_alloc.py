@@ -47,6 +47,37 @@ def test_static_attention_two_calls_in_a_row(lva, orc, ctx):
     _case(lva, orc, ctx, heads=40, rot=128, backlog=512, pos=300, batch=1, seed=73)
 
 
+def _free_device_bytes():
+    """hipMemGetInfo of the runtime the library is linked against (already loaded into this process)"""
+    import ctypes as C
+    hip = C.CDLL("libamdhip64.so")
+    free, total = C.c_size_t(), C.c_size_t()
+    assert hip.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+    return free.value
+
+
+def test_static_attention_leaves_device_memory_as_it_was(lva, ctx):
+    """what the entry point is for: calls that allocate nothing.  Free device memory (hipMemGetInfo) is read before and after
+    calls of three different sizes, each the first of its size on this context (so a workspace that grew with the input, as
+    lv_kernel_attention's does, would show), and is the same to the byte."""
+    rng = np.random.default_rng(5)
+    bufs = []
+    for heads, rot, backlog, pos, batch in ((32, 128, 2048, 2047, 1), (8, 64, 1024, 1000, 4), (40, 128, 1024, 700, 2)):
+        dim = heads * rot
+        kc = (rng.standard_normal((backlog, dim)) * 0.5).astype(np.float16).view(np.uint16)
+        q = rng.standard_normal((batch, dim)).astype(np.float32)
+        bufs.append((ctx.to_device(kc), ctx.to_device(kc), ctx.to_device(q), ctx.alloc(batch * dim * 4), pos, backlog, heads, rot, batch))
+    ctx.sync()
+    before = _free_device_bytes()
+    for dk, dv, dq, dout, pos, backlog, heads, rot, batch in bufs:
+        lva.check(ctx.lib.lv_kernel_attention_static(ctx.h, dout, dk, dv, dq, pos, backlog, heads, rot, batch))
+        ctx.sync()
+        assert _free_device_bytes() == before
+    for dk, dv, dq, dout, *_ in bufs:
+        for p in (dk, dv, dq, dout):
+            ctx.free(p)
+
+
 def test_static_attention_rejects_sizes_beyond_the_work_area(lva, ctx):
     lib = ctx.lib
     p = lva.C.c_void_p(256)          # never dereferenced: the call is refused on its sizes
