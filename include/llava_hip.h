@@ -96,6 +96,13 @@ int lv_step_wait(lv_session *s);
 /* replaces output_probs->map in get_last_predicted_token (llava_session.cpp:129-135): logits of the LAST row
  * of the last step, `vocab` floats.  Implies lv_step_wait. */
 int lv_logits_read(lv_session *s, float *dst);
+/* The reference computes the logits of EVERY row of a step (output_probs is batch x vocab, llava_session.cpp:49-79; the
+ * head runs over all rows, llava_command_buffer.cpp:38-39) and its interface reads the last (llava_session.cpp:131-135).
+ * With this switch on, a step keeps all of them on the device and lv_logits_read_rows returns rows row0 .. row0 + n_rows - 1
+ * of the last step (row z = the token at position pos + z), `vocab` floats each; implies lv_step_wait.  Off by default:
+ * a 512-token prompt then multiplies one row by the output matrix instead of 512. */
+int lv_session_set_all_logits(lv_session *s, int enable);
+int lv_logits_read_rows(lv_session *s, uint32_t row0, uint32_t n_rows, float *dst);
 /* index of the first strict maximum of those logits, computed on the device (the greedy rule of
  * llava_session.cpp:144-152).  Implies lv_step_wait. */
 int lv_argmax(lv_session *s, uint32_t *token);

@@ -98,6 +98,8 @@ _HIP_SIGS = {
     "lv_step_begin": [_VP, _VP, _U32, _U32],
     "lv_step_wait": [_VP],
     "lv_logits_read": [_VP, _VP],
+    "lv_session_set_all_logits": [_VP, _I],
+    "lv_logits_read_rows": [_VP, _U32, _U32, _VP],
     "lv_argmax": [_VP, C.POINTER(_U32)],
     "lv_kv_read": [_VP, _U32, _I, _U32, _VP],
     "lv_kv_write": [_VP, _U32, _I, _U32, _VP],
@@ -397,6 +399,15 @@ class Session:
     def logits(self):
         out = np.empty(self.model.header["vocab"], dtype=np.float32)
         check(self.lib.lv_logits_read(self.h, _ptr(out)))
+        return out
+
+    def keep_all_logits(self, on=True):
+        check(self.lib.lv_session_set_all_logits(self.h, int(on)))
+
+    def logits_rows(self, row0, n_rows):
+        """logits of rows row0 .. row0 + n_rows - 1 of the last step (needs keep_all_logits before that step)"""
+        out = np.empty((n_rows, self.model.header["vocab"]), dtype=np.float32)
+        check(self.lib.lv_logits_read_rows(self.h, row0, n_rows, _ptr(out)))
         return out
 
     def argmax(self):

@@ -170,6 +170,8 @@ struct lv_model {
     std::mutex prompt_mutex;
     int prompt_state = 0;           // 0 not made yet, 1 ready, -1 could not be made (batches then go token by token)
     uint16_t *prompt_arena = nullptr;
+    int output_state = 0;           // the same for the prompt copy of the output matrix, which only steps that keep every row's logits need
+    uint16_t *output_copy = nullptr;
 };
 
 // Shape classes the persistent kernel is compiled for: LLaMA-7B and LLaMA-13B layer shapes, q4_0 and q8_0.
@@ -246,6 +248,10 @@ struct lv_session {
     bool mega_off = false;                // the persistent kernel is no longer used by this session (refused launch, or two such steps)
     bool in_flight = false;
     bool have_logits = false;
+    // logits of EVERY row of a step (the reference's output_probs holds batch x vocab, llava_session.cpp:49-79), kept on request
+    bool all_logits = false;
+    float *logits_all = nullptr;          // [logits_cap][vocab]
+    uint32_t logits_cap = 0, logits_rows = 0;
     bool trace = false;
     // record mode keeps every row of a step, as the reference's batch-sized buffers do (llava_layer_session_data.cpp:79-86)
     float *trace_buf = nullptr;  // [layers][LV_TRACE_ATTN][trace_cap][max(dim, ff)]: the five vector buffers
@@ -1456,6 +1462,7 @@ extern "C" int lv_model_destroy(lv_model *m)
     if (!m) return LV_OK;
     (void)hipSetDevice(m->ctx->device);
     (void)hipFree(m->prompt_arena);
+    (void)hipFree(m->output_copy);
     (void)hipFree(m->mega_stream);
     (void)hipFree(m->mega_norms);
     (void)hipFree(m->tok_f32_own);
@@ -1501,7 +1508,7 @@ extern "C" int lv_session_destroy(lv_session *s)
     drop_graph(s);
     void *dev[] = {s->kv, s->trig, s->trig_abs, s->x, s->xn, s->q, s->k, s->v, s->vo, s->ff, s->logits, s->attn_part, s->attn_counters,
                    s->cfg, s->argmax_dev, s->trace_buf, s->trace_attn, s->pf_x, s->pf_xn, s->pf_q, s->pf_k, s->pf_v, s->pf_vo, s->pf_g1, s->pf_g2,
-                   s->pf_xh, s->pf_xl, s->pf_xs, s->pf_planes, s->pf_fh, s->pf_fl};
+                   s->pf_xh, s->pf_xl, s->pf_xs, s->pf_planes, s->pf_fh, s->pf_fl, s->logits_all};
     for (void *p : dev) (void)hipFree(p);
     for (int i = 0; i < 2; i++) {
         uncached_give(s->model->ctx->device, s->xchg[i], s->xchg_bytes, s->xchg_pooled[i]);
@@ -1713,7 +1720,7 @@ extern "C" int lv_session_path(const lv_session *s, int *path)
 // either; the waits inside the kernel are bounded for that), the two launch at the same rate (measured in alternation), and
 // the separate queue the runtime opens for cooperative launches makes a process under rocprofv3 end with a segmentation
 // fault in its exit handlers (a forty-line program with one cooperative launch of an empty kernel does the same).
-static int launch_mega(lv_session *s, uint32_t pos, uint32_t token, bool *refused)
+static int launch_mega(lv_session *s, uint32_t pos, uint32_t token, bool *refused, float *logits_dst)
 {
     const lv_model *m = s->model;
     MegaArgs a{};
@@ -1726,7 +1733,7 @@ static int launch_mega(lv_session *s, uint32_t pos, uint32_t token, bool *refuse
     a.xchg_rearm = s->xchg[(s->xchg_turn + 1) & 1];
     a.xl = s->xl[s->xchg_turn & 1];
     a.xl_rearm = s->xl[(s->xchg_turn + 1) & 1];
-    a.logits = s->logits;
+    a.logits = logits_dst;
     a.status = s->status_host;
     a.layers = m->hp.layers; a.vocab = m->hp.vocab; a.backlog = s->backlog; a.pos = pos; a.token = token;
     a.spin_limit = s->wait_limit ? s->wait_limit : kSpinLimit;
@@ -1906,6 +1913,24 @@ static bool ensure_prompt_copy(lv_model *m)
     return true;
 }
 
+// the prompt copy of the output matrix: only a batch that keeps the logits of every row multiplies all its rows by it
+static bool ensure_output_copy(lv_model *m)
+{
+    std::lock_guard<std::mutex> lock(m->prompt_mutex);
+    if (m->output_state) return m->output_state > 0;
+    m->output_state = -1;
+    if (m->output.view.cols % 32 || (m->output.ftype != LV_Q4_0 && m->output.ftype != LV_Q8_0)) return false;
+    if (hipMalloc(reinterpret_cast<void **>(&m->output_copy), (size_t)prompt_copy_halfs(m->output) * 2) != hipSuccess) {
+        (void)hipGetLastError();
+        m->output_copy = nullptr;
+        return false;
+    }
+    if (launch_expand(m->ctx->stream, m->output_copy, m->output) != LV_OK || hipStreamSynchronize(m->ctx->stream) != hipSuccess) return false;
+    m->output.h16 = m->output_copy;
+    m->output_state = 1;
+    return true;
+}
+
 constexpr uint32_t kPrefillChunk = 512;    // tokens evaluated together (bounds the workspace)
 
 static int prefill_reserve(lv_session *s, uint32_t n)
@@ -1970,7 +1995,7 @@ static int launch_prefill_norm(hipStream_t st, lv_session *s, const float *w, ui
 
 // Rows idx0 .. idx0+n-1 of the step at once (llava_layer.cpp:39-75 with batch > 1).  Row z sees cache rows
 // 0..pos+z: all K/V rows of the chunk are appended before any row attends, rows above its own are masked.
-static int record_prefill(lv_session *s, uint32_t idx0, uint32_t n, bool with_head)
+static int record_prefill(lv_session *s, uint32_t idx0, uint32_t n, bool with_head, uint32_t row_base)
 {
     const lv_model *m = s->model;
     const lv_hparams &hp = m->hp;
@@ -2044,6 +2069,23 @@ static int record_prefill(lv_session *s, uint32_t idx0, uint32_t n, bool with_he
         }
         LV_TRY(launch_gemm_sliced(st, s->pf_x, D, lw.w2, n, fh, fl, nullptr, true, parts, &pending));
     }
+    if (s->all_logits) {
+        // every row's logits, as the reference computes them (llava_command_buffer.cpp:38-39): final norm of all n rows, then the
+        // output matrix on the matrix cores where its prompt copy exists, as a batched GEMV otherwise
+        float *dst = s->logits_all + (size_t)(row_base + idx0) * hp.vocab;
+        if (ensure_output_copy(s->model)) {
+            const float *xscale = nullptr;
+            LV_TRY(launch_prefill_norm(st, s, m->norm, n, D, parts, pending, false, &xscale));
+            LV_TRY(launch_gemm_presplit(st, dst, hp.vocab, m->output, n, s->pf_xh, s->pf_xl, false, xscale));
+        } else {
+            if (pending) LV_TRY(launch_gemm_reduce(st, s->pf_x, D, parts, pending, D, n, true));
+            normalize_kernel<<<dim3(n), dim3(256), 0, st>>>(s->pf_xn, s->pf_x, m->norm, D);
+            HIP_TRY(hipGetLastError());
+            LV_TRY(launch_gemv(st, dst, m->output, nullptr, s->pf_xn, n, kGemvStore));
+        }
+        if (with_head) HIP_TRY(hipMemcpyAsync(s->logits, dst + (size_t)(n - 1) * hp.vocab, (size_t)hp.vocab * 4, hipMemcpyDeviceToDevice, st));
+        return LV_OK;
+    }
     if (pending) LV_TRY(launch_gemm_reduce(st, s->pf_x, D, parts, pending, D, n, true));
     if (with_head) {
         // only the last row's logits are ever read (llava_session.cpp:131-139)
@@ -2069,6 +2111,24 @@ extern "C" int lv_step_begin(lv_session *s, const uint32_t *tokens, uint32_t n, 
 
     s->have_logits = false;
     s->pick_in_status = false;
+    s->logits_rows = 0;
+    if (s->all_logits) {
+        if (n > s->logits_cap) {
+            HIP_TRY(hipStreamSynchronize(s->stream));
+            (void)hipFree(s->logits_all);
+            s->logits_all = nullptr;
+            s->logits_cap = 0;
+            const hipError_t e = hipMalloc(reinterpret_cast<void **>(&s->logits_all), (size_t)n * s->model->hp.vocab * 4);
+            if (e != hipSuccess) {
+                (void)hipGetLastError();
+                s->logits_all = nullptr;
+                return fail(e == hipErrorOutOfMemory ? LV_ERR_OOM : LV_ERR_HIP, "lv_step_begin: logits of %u rows: %s", n, hipGetErrorString(e));
+            }
+            s->logits_cap = n;
+        }
+    }
+    const uint32_t n_rows = n, V = s->model->hp.vocab;
+    uint32_t row_base = 0;          // rows of this step already launched on the persistent kernel when the rest takes another path
     if (s->trace) {
         LV_TRY(trace_reserve(s, n));
         s->trace_n = n;
@@ -2084,7 +2144,7 @@ extern "C" int lv_step_begin(lv_session *s, const uint32_t *tokens, uint32_t n, 
         uint32_t done = 0;
         bool refused = false;
         while (done < n) {
-            LV_TRY(launch_mega(s, pos + done, tokens[done], &refused));
+            LV_TRY(launch_mega(s, pos + done, tokens[done], &refused, s->all_logits ? s->logits_all + (size_t)done * V : s->logits));
             if (refused) break;
             done++;
             s->mega_step = true;
@@ -2096,8 +2156,11 @@ extern "C" int lv_step_begin(lv_session *s, const uint32_t *tokens, uint32_t n, 
             persistent = false;
             (void)lv_session_path(s, &path);
             tokens += done; n -= done; pos += done;
+            row_base = done;
         } else {
             s->pick_in_status = true;  // the kernel leaves the greedy pick (of the last token) in the pinned status block
+            if (s->all_logits)         // lv_logits_read takes the last row from where every path leaves it
+                HIP_TRY(hipMemcpyAsync(s->logits, s->logits_all + (size_t)(n - 1) * V, (size_t)V * 4, hipMemcpyDeviceToDevice, s->stream));
         }
     }
     if (!persistent) {             // the persistent kernel takes position and token id as launch arguments
@@ -2122,20 +2185,26 @@ extern "C" int lv_step_begin(lv_session *s, const uint32_t *tokens, uint32_t n, 
             HIP_TRY(hipGraphInstantiate(&s->graph_exec, s->graph, nullptr, nullptr, 0));
         }
         HIP_TRY(hipGraphLaunch(s->graph_exec, s->stream));
+        if (s->all_logits) HIP_TRY(hipMemcpyAsync(s->logits_all + (size_t)row_base * V, s->logits, (size_t)V * 4, hipMemcpyDeviceToDevice, s->stream));
     } else {
         // rows are evaluated one after the other: row z sees cache rows 0..pos+z, which is what the batched
         // shaders compute (every row's K/V is appended before any row attends, and rows above are masked)
         if (n >= kPrefillMin && !s->trace && ensure_prompt_copy(s->model)) {
             for (uint32_t i = 0; i < n; i += kPrefillChunk) {
                 const uint32_t m = n - i < kPrefillChunk ? n - i : kPrefillChunk;
-                LV_TRY(record_prefill(s, i, m, i + m == n));
+                LV_TRY(record_prefill(s, i, m, i + m == n, row_base));
             }
         } else {
-            for (uint32_t i = 0; i < n; i++) LV_TRY(record_token(s, i, i + 1 == n));
+            for (uint32_t i = 0; i < n; i++) {
+                LV_TRY(record_token(s, i, s->all_logits || i + 1 == n));
+                if (s->all_logits)
+                    HIP_TRY(hipMemcpyAsync(s->logits_all + (size_t)(row_base + i) * V, s->logits, (size_t)V * 4, hipMemcpyDeviceToDevice, s->stream));
+            }
         }
     }
     s->in_flight = true;
     s->have_logits = true;
+    if (s->all_logits) s->logits_rows = n_rows;
     return LV_OK;
 }
 
@@ -2164,6 +2233,28 @@ extern "C" int lv_logits_read(lv_session *s, float *dst)
     if (!s || !dst) return fail(LV_ERR_ARG, "lv_logits_read: null argument");
     if (!s->have_logits) return fail(LV_ERR_STATE, "lv_logits_read: no step has produced logits");
     HIP_TRY(hipMemcpyAsync(dst, s->logits, (size_t)s->model->hp.vocab * 4, hipMemcpyDeviceToHost, s->stream));
+    return lv_step_wait(s);
+}
+
+extern "C" int lv_session_set_all_logits(lv_session *s, int enable)
+{
+    if (!s) return fail(LV_ERR_ARG, "lv_session_set_all_logits: session is null");
+    if (s->in_flight) return fail(LV_ERR_STATE, "lv_session_set_all_logits: a step is in flight");
+    s->all_logits = enable != 0;
+    if (!s->all_logits) s->logits_rows = 0;
+    return LV_OK;
+}
+
+extern "C" int lv_logits_read_rows(lv_session *s, uint32_t row0, uint32_t n_rows, float *dst)
+{
+    if (!s || (n_rows && !dst)) return fail(LV_ERR_ARG, "lv_logits_read_rows: null argument");
+    if (!s->have_logits || s->logits_rows == 0) return fail(LV_ERR_STATE, "lv_logits_read_rows: no step has kept the logits of all its rows (lv_session_set_all_logits)");
+    if (row0 > s->logits_rows || n_rows > s->logits_rows - row0)
+        return fail(LV_ERR_RANGE, "lv_logits_read_rows: rows %u..%u of a step of %u", row0, row0 + n_rows, s->logits_rows);
+    if (n_rows) {
+        const size_t V = s->model->hp.vocab;
+        HIP_TRY(hipMemcpyAsync(dst, s->logits_all + (size_t)row0 * V, (size_t)n_rows * V * 4, hipMemcpyDeviceToHost, s->stream));
+    }
     return lv_step_wait(s);
 }
 

@@ -259,6 +259,26 @@ def test_13b_q4_0_256_greedy_steps_on_graph_and_persistent_paths(lva, orc, ctx):
         h.close()
 
 
+def test_7b_q4_0_logits_of_all_128_prompt_rows(lva, orc, ctx, model_7b):
+    """the reference's head runs over every row of a step (llava_command_buffer.cpp:38-39): with lv_session_set_all_logits the
+    128-token prompt keeps 128 x 32000 logits (final norm of all rows, the 32000 x 4096 output matrix on the matrix
+    cores), each row against the checker's"""
+    om = orc.Model(model_7b)
+    osess = orc.Session(om, 128)
+    model = lva.Model(ctx, model_7b)
+    s = lva.Session(model, 128)
+    s.keep_all_logits()
+    prompt = lva.synth_tokens(128, 3, SHAPE["vocab"], seed=5)
+    want = osess.eval(prompt, all_rows=True)
+    s.begin(prompt, 0)
+    got = s.logits_rows(0, 128)
+    worst = float(np.max(np.abs(got - want) / (1e-2 + 1e-3 * np.abs(want))))
+    assert worst <= 1.0, worst
+    assert np.array_equal(np.argmax(got, axis=1), np.argmax(want, axis=1))
+    print(f"128 x 32000 logits: worst error {worst:.3f} x tolerance")
+    s.close(); model.close(); osess.close(); om.close()
+
+
 def test_7b_q4_0_prompt_of_128_as_one_step_then_steps(lva, orc, ctx, model_7b):
     """a 128-token prompt on the 7B q4_0 model: the q4_0 GEMM forms at K = 4096 and 11008 with full token tiles, checked
     against the oracle evaluating the 128 tokens itself"""

@@ -440,3 +440,63 @@ def test_persistent_kernel_up_to_the_last_cache_row(lva, orc, ctx, wide_model):
     with pytest.raises(lva.LvError):
         s.begin([tok], 128)
     s.close(); model.close(); osess.close(); om.close()
+
+
+def _rows_match(got, want):
+    tol = 1e-2 + 1e-3 * np.abs(want)
+    assert got.shape == want.shape
+    assert np.all(np.abs(got - want) <= tol), float(np.max(np.abs(got - want) / tol))
+
+
+@pytest.mark.parametrize("name", ["tiny_q4", "tiny_q8", "pair_q8"])
+def test_logits_of_every_row_of_a_step(lva, orc, ctx, tiny_models, name):
+    """the reference's output_probs holds the logits of every row of a step (llava_session.cpp:49-79,
+    llava_command_buffer.cpp:38-39); with lv_session_set_all_logits a step keeps them: a 5-token step (token by token on the
+    operator chain), a 20-token step behind it (the batched path: final norm of all rows, output matrix on the matrix
+    cores) and a one-token step (the captured graph), each row against the checker's row"""
+    om = orc.Model(tiny_models[name])
+    osess = orc.Session(om, 128)
+    model = lva.Model(ctx, tiny_models[name])
+    s = lva.Session(model, 128)
+    with pytest.raises(lva.LvError):
+        s.begin([5], 0)
+        s.logits_rows(0, 1)                  # the switch is off: nothing was kept
+    s.wait()
+    s.keep_all_logits()
+    toks = lva.synth_tokens(26, 3, om.hp["vocab"], seed=21)
+    pos = 0
+    for n in (5, 20, 1):
+        want = osess.eval(toks[pos:pos + n], all_rows=True)
+        s.begin(toks[pos:pos + n], pos)
+        _rows_match(s.logits_rows(0, n), want)
+        _rows_match(s.logits()[None, :], want[-1:])          # the last row is still where lv_logits_read finds it
+        if n > 2:
+            _rows_match(s.logits_rows(1, n - 2), want[1:n - 1])
+            with pytest.raises(lva.LvError):
+                s.logits_rows(1, n)          # past the end of the step
+        pos += n
+    s.keep_all_logits(False)
+    s.begin(toks[:3], 0)
+    with pytest.raises(lva.LvError):
+        s.logits_rows(0, 1)
+    s.close(); model.close(); osess.close(); om.close()
+
+
+def test_logits_of_every_row_on_the_persistent_kernel(lva, orc, ctx, wide_model):
+    """a short step on the persistent kernel is one launch per token, and every launch computes its logits: kept row by row"""
+    om = orc.Model(wide_model)
+    osess = orc.Session(om, 128)
+    model = lva.Model(ctx, wide_model)
+    s = lva.Session(model, 128)
+    assert s.path() == lva.PATH_PERSISTENT
+    s.keep_all_logits()
+    toks = lva.synth_tokens(9, 3, 2048, seed=22)
+    want = osess.eval(toks[:6], all_rows=True)
+    s.begin(toks[:6], 0)
+    _rows_match(s.logits_rows(0, 6), want)
+    assert s.argmax() == orc.greedy(want[-1])
+    want = osess.eval(toks[6:7], all_rows=True)
+    s.begin(toks[6:7], 6)
+    _rows_match(s.logits_rows(0, 1), want)
+    _rows_match(s.logits()[None, :], want)
+    s.close(); model.close(); osess.close(); om.close()
