@@ -187,12 +187,6 @@ struct MegaArgs {
                                // where the launch placed all of them on one XCD; zero: device scope everywhere
 };
 
-// Phase boundaries of a layer are marked MEGA_STAMP(n); the marks compile to nothing unless the including file has
-// defined the macro (it sees the kernel's `status`, `layer` and thread indices).
-#ifndef MEGA_STAMP
-#define MEGA_STAMP(idx) do { } while (0)
-#endif
-
 struct MegaTile {
     uint4 c, c2;   // c2: second half of the codes of a q8_0 block (unused for q4_0)
     uint16_t d;    // fp16 scale bits
@@ -580,9 +574,7 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
         uint16_t *kc = a.kv + (size_t)layer * 2 * a.backlog * D, *vc = kc + (size_t)a.backlog * D;
 
         // ================= A: norm + QKV ====================================================================
-        MEGA_STAMP(0);
         const float inv_a = acquire_vector<D, NW, true, kPollDelay>(xs, x_src, norm_w, scratch, status, spin_limit);
-        MEGA_STAMP(1);
         load_slab(xr, xsum, xs, mw.sD * 64 + lane, mw.laneD);
         gemv_phase<S, S::SEQ_A, S::TA, S::NSD>(q, mw, layer, xr, xsum, mw.sD, mw.rD, mw.actD, S::ROWS_A, red);
         if (layer == 0 && a.xcd_local && w == 0) {
@@ -615,7 +607,6 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
         }
 
         // ================= B: attention chunk (head h, chunk c) ================================================
-        MEGA_STAMP(2);
         {
             const int h = place.h, c = place.c;
             if (place.attends) {
@@ -679,7 +670,6 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
                         for (int i = 0; i < 8; i++) { qkv[8 + i] = l.qkv[R + sub * 8 + i]; qkv[16 + i] = l.qkv[2 * R + sub * 8 + i]; }
                     }
                 }
-                MEGA_STAMP(3);
                 const float scale = rsqrtf((float)R);
                 float den = 0.f;
                 // exp(score / sqrt(R)) of cache row p for this 16-lane group's query head; every lane of the group gets it
@@ -753,7 +743,6 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
         }
 
         // ================= B': combine the chunks of head b (one wait for numerators and denominators) ==========
-        MEGA_STAMP(4);
         if (place.attends && place.c == 0 && st < R) {
             float nd[2 * S::CPH];
             const uint32_t *hp = reinterpret_cast<const uint32_t *>(xlc + S::OFF_PART + (size_t)place.h * S::CPH * S::PART);
@@ -779,9 +768,7 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
         }
 
         // ================= C: x += Wo o ============================================================================
-        MEGA_STAMP(5);
         acquire_vector<D, NW, false, kPollDelay>(xs, xc + S::OFF_O, nullptr, scratch, status, spin_limit);
-        MEGA_STAMP(6);
         load_slab(xr, xsum, xs, mw.sD * 64 + lane, mw.laneD);
         gemv_phase<S, S::SEQ_C, S::TC, S::NSD>(q, mw, layer, xr, xsum, mw.sD, mw.rD, mw.actD, S::ROWS_C, red);
         lds_barrier();
@@ -792,9 +779,7 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
         }
 
         // ================= D: norm + SwiGLU ========================================================================
-        MEGA_STAMP(7);
         const float inv_d = acquire_vector<D, NW, true, kPollDelay>(xs, xc + S::OFF_X1, norm_w + D, scratch, status, spin_limit);
-        MEGA_STAMP(8);
         load_slab(xr, xsum, xs, mw.sD * 64 + lane, mw.laneD);
         gemv_phase<S, S::SEQ_D, S::TD, S::NSD>(q, mw, layer, xr, xsum, mw.sD, mw.rD, mw.actD, S::ROWS_D, red);
         lds_barrier();
@@ -805,13 +790,10 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
         }
 
         // ================= E: x += W2 ff ===========================================================================
-        MEGA_STAMP(9);
         if constexpr (S::OWN_SLAB_E) {
             acquire_own_slab<S, kPollDelay>(xr, xsum, xs, xc + S::OFF_FF, mw.sF, lane, mw.actF, mw.laneF, status, spin_limit);
-            MEGA_STAMP(10);
         } else {
             acquire_vector_wide<F, NW, kPollDelay>(xs, xc + S::OFF_FF, status, spin_limit);
-            MEGA_STAMP(10);
             if constexpr (S::E_REDEAL) {
                 int row0, slab0;
                 mega_e_tile<S>(w, 0, row0, slab0);
@@ -851,7 +833,6 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
             xown[st] = v;
             st_dev(xc + S::OFF_X2 + b * S::ROWS_E + st, v);
         }
-        MEGA_STAMP(11);
         x_src = xc + S::OFF_X2;
     }
 
