@@ -175,17 +175,18 @@ struct lv_model {
 };
 
 // Shape classes the persistent kernel is compiled for: LLaMA-7B and LLaMA-13B layer shapes, q4_0 and q8_0.
-// Wavefronts per workgroup and queue depth per shape class, measured (tok/s at 12 waves with the shallow queue the
-// register file then allows -> as below): 7B q4_0 845 -> 897, 7B q8_0 469 -> 538, 13B q4_0 462 -> 499, 13B q8_0
-// 286 -> 322.  Two waves per SIMD leave each wave 256 registers, which buys the deeper queue; the 13B shapes have three
-// column slabs in the D-wide phases and seven in the F-wide one, so seven waves keep all but one busy everywhere.
+// Eight wavefronts per workgroup (two per SIMD leave each wave 256 registers, which buys a queue 8 q4_0 tiles or 4 q8_0 tiles
+// deep; twelve waves with the shallow queue the register file then allows lost 6-13 %).  The 13B classes ran on seven waves
+// while a wave was tied to one of three column slabs, the third half empty; with the half slab's tiles carrying two rows
+// and the waves dealt 3 + 3 + 2 (MegaShapeBase) all eight work in the D-wide phases: 13B q4_0 544 -> 592-607 tok/s, 13B q8_0
+// 357-370 -> 379-392.
 using Mega7Bq4 = MegaShape<4096, 11008, 32, 8, 4, 8>;
 using Mega7Bq8 = MegaShape<4096, 11008, 32, 8, 8, 4>;
-using Mega13Bq4 = MegaShape<5120, 13824, 40, 7, 4, 8>;
-using Mega13Bq8 = MegaShape<5120, 13824, 40, 7, 8, 4>;
+using Mega13Bq4 = MegaShape<5120, 13824, 40, 8, 4, 8>;
+using Mega13Bq8 = MegaShape<5120, 13824, 40, 8, 8, 4>;
 // the same for version-1 files (fp32 block scales; the reference loads q4_0 of that version only, llava_buffer.cpp:66-71)
 using Mega7Bq4v1 = MegaShapeV1<4096, 11008, 32, 8, 4, 8>;
-using Mega13Bq4v1 = MegaShapeV1<5120, 13824, 40, 7, 4, 8>;
+using Mega13Bq4v1 = MegaShapeV1<5120, 13824, 40, 8, 4, 8>;
 constexpr int kMegaKinds = 6;
 
 template <class Fn>
@@ -1310,7 +1311,7 @@ static int build_mega(lv_model *m)
         (void)mega_dispatch(kind, [&](auto shape) -> int {
             using S = decltype(shape);
             fits = hp.dim == (uint32_t)S::D && hp.ff == (uint32_t)S::F && hp.heads == (uint32_t)S::H && ft == (S::QT == 4 ? LV_Q4_0 : LV_Q8_0) && S::SF32 == sf32 &&
-                   (hp.vocab + kMegaWGs - 1) / kMegaWGs <= (uint32_t)(S::HEAD * S::NRD);
+                   (hp.vocab + kMegaWGs - 1) / kMegaWGs <= (uint32_t)S::MAX_VOCAB_ROWS;
             return LV_OK;
         });
         if (!fits) continue;

@@ -66,6 +66,18 @@ __device__ __forceinline__ float quad_partials_sum(float p0, float p1, float p2,
     const float c = __uint_as_float(t[0]) + __uint_as_float(t[1]);      // rows of 16 lanes hold p0, p2, p1, p3
     return group16_sum(c);
 }
+// The same for partials whose lanes 0-31 and 32-63 belong to two different matrix rows (tiles that carry 32 blocks of each
+// of two rows): eight totals.  In s01 the 16-lane rows hold the totals of [p0 lower half, p0 upper half, p1 lower, p1 upper],
+// in s23 those of p2 and p3.
+__device__ __forceinline__ void quad_partials_sum_halves(float p0, float p1, float p2, float p3, float &s01, float &s23)
+{
+    auto a = __builtin_amdgcn_permlane32_swap(__float_as_uint(p0), __float_as_uint(p1), false, false);  // [p0.lo | p1.lo], [p0.hi | p1.hi]
+    auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(p2), __float_as_uint(p3), false, false);
+    auto ta = __builtin_amdgcn_permlane16_swap(a[0], a[1], false, false);   // [lo.r0 hi.r0 lo.r2 hi.r2], [lo.r1 hi.r1 lo.r3 hi.r3]
+    auto tb = __builtin_amdgcn_permlane16_swap(b[0], b[1], false, false);
+    s01 = group16_sum(__uint_as_float(ta[0]) + __uint_as_float(ta[1]));
+    s23 = group16_sum(__uint_as_float(tb[0]) + __uint_as_float(tb[1]));
+}
 // which of the four partials ends up in 16-lane row j of the result above
 __device__ __forceinline__ int quad_partial_of_lane(int lane)
 {

@@ -26,8 +26,9 @@
 //
 // Weight stream: for each (layer, phase, workgroup, wave) the tiles that wave will consume, in order.
 // A tile is one matrix row restricted to the wave's 64-block column slab: 64 x 16 B (q4_0) or two planes of 64 x 16 B
-// (q8_0: first and second half of every block's codes) + 64 x fp16 scales (1152 B / 2176 B).  Lane l of the wave always owns block column 64*slab + l, so the 32 activations of
-// that column sit in registers for the whole phase.
+// (q8_0: first and second half of every block's codes) + 64 x fp16 scales (1152 B / 2176 B).  Lane l of the wave always owns
+// block column 64*slab + l, so the 32 activations of that column sit in registers for the whole phase.  Where a row ends in
+// half a slab (D = 5120: 2.5 slabs) the tiles of that half slab carry two rows, 32 blocks of each, so that no lane idles.
 #pragma once
 
 #include "lv_device.h"
@@ -103,6 +104,16 @@ __device__ __forceinline__ void lds_barrier()
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
+// A value the compiler has to take as new each time: what is computed from it inside the layer loop (LDS addresses above
+// all) is then computed there, a few instructions each, instead of once in front of the loop and kept in registers.  Used
+// (OPAQUE) by the shape classes whose kernel would otherwise spill; where registers suffice, keeping the values is faster.
+template <bool OPAQUE>
+__device__ __forceinline__ int maybe_opaque(int v)
+{
+    if constexpr (OPAQUE) asm volatile("" : "+v"(v));
+    return v;
+}
+
 constexpr int cdiv(int a, int b) { return (a + b - 1) / b; }
 constexpr int round_up(int a, int b) { return cdiv(a, b) * b; }
 
@@ -118,10 +129,19 @@ struct MegaShapeBase {
     static constexpr int DEPTH = DEPTH_ ? DEPTH_ : (QT == 4 ? 4 : 2);   // tiles in flight per wave
     static constexpr int NBD = D / 32, NBF = F / 32;            // blocks per row
     static constexpr int NSD = cdiv(NBD, 64), NSF = cdiv(NBF, 64);  // column slabs
-    static constexpr int NRD = NW / NSD, NRF = NW / NSF;        // row sets (waves sharing a slab split the rows)
-    // phase E: every wave of the workgroup owns exactly one column slab; each then fetches its own part of the input vector
-    // (acquire_own_slab).  Where waves are left over (7B: six slabs, eight waves) the common fetch by all threads is as fast.
-    static constexpr bool OWN_SLAB_E = NRF == 1 && NSF == NW;
+    // D-wide phases (A, C, D, head).  A row of D = 4096 is two full slabs of 64 blocks; a row of D = 5120 is two full slabs and
+    // HALF a slab (32 blocks).  Tiles of the half slab carry TWO rows, 32 blocks of each (lanes 0-31 row 2p, lanes 32-63 row
+    // 2p + 1; a lane's block column is the same for both), so every lane of every tile works and every queue slot holds a
+    // full tile.  The waves are dealt to the slabs by their work: WPF waves to each full slab (one tile per row), WPH to the
+    // half slab (one tile per two rows).
+    static constexpr int FULLD = NBD / 64, HALFD = NBD % 64 ? 1 : 0;
+    static_assert(NBD % 64 == 0 || NBD % 64 == 32, "a row is full slabs plus at most half a slab");
+    static constexpr int WPH = HALFD ? (NW + FULLD) / (2 * FULLD + 1) : 0, WPF = (NW - WPH) / FULLD;
+    static_assert(WPF >= 1 && (!HALFD || WPH >= 1), "waves for every slab");
+    // tiles (queue slots) a wave has in a D-wide phase of `rows` rows, and the tiles a half-slab wave really has of them
+    static constexpr int tiles_half(int rows) { return HALFD ? cdiv(cdiv(rows, 2), WPH) : 0; }
+    static constexpr int tiles_d(int rows) { return cdiv(rows, WPF) > tiles_half(rows) ? cdiv(rows, WPF) : tiles_half(rows); }
+    static constexpr int NRF = NW / NSF;                        // row sets of the F-wide phase (waves sharing a slab split the rows)
     static constexpr int ROWS_A = 3 * D / kMegaWGs, ROWS_C = D / kMegaWGs, ROWS_D = 2 * F / kMegaWGs, ROWS_E = D / kMegaWGs;
     // Down projection (phase E).  Where the waves outnumber the column slabs (7B: six slabs, eight waves) the spare waves take
     // the last E_SPARE_ROWS rows of E_SPARE_SLABS slabs each, so that every wave has the same number of tiles (12 instead of 16
@@ -131,11 +151,16 @@ struct MegaShapeBase {
                                      (ROWS_E - ROWS_E * NSF / NW) % 4 == 0 && (ROWS_E * NSF / NW) % 4 == 0 &&
                                      (ROWS_E - ROWS_E * NSF / NW) * (NSF / E_SPARE) == ROWS_E * NSF / NW;
     static constexpr int E_SPARE_SLABS = E_REDEAL ? NSF / E_SPARE : 0, E_SPARE_ROWS = E_REDEAL ? ROWS_E - ROWS_E * NSF / NW : 0;
-    static constexpr int TA = cdiv(ROWS_A, NRD), TC = cdiv(ROWS_C, NRD), TD = cdiv(ROWS_D, NRD),
+    // phase E where every working wave owns exactly one column slab (a wave without one idles): each fetches its own part of
+    // the input vector (acquire_own_slab).  Where spare waves take rows of several slabs (E_REDEAL) the common fetch by all
+    // threads is as fast.
+    static constexpr bool OWN_SLAB_E = NRF == 1 && !E_REDEAL;
+    static constexpr int TA = tiles_d(ROWS_A), TC = tiles_d(ROWS_C), TD = tiles_d(ROWS_D),
                          TE = E_REDEAL ? ROWS_E * NSF / NW : cdiv(ROWS_E, NRF);
     static constexpr int SEQ_A = 0, SEQ_C = TA, SEQ_D = TA + TC, SEQ_E = TA + TC + TD;
     static constexpr int PER_LAYER = round_up(TA + TC + TD + TE, DEPTH);
-    static constexpr int HEAD = round_up(cdiv(kMegaVocabRows, NRD), 4);   // head tiles per wave (static upper bound)
+    static constexpr int MAX_VOCAB_ROWS = kMegaVocabRows + 3;           // output-matrix rows per workgroup the kernel has room for (vocabularies up to 32768)
+    static constexpr int HEAD = round_up(tiles_d(MAX_VOCAB_ROWS), 4);   // head tiles per wave (static upper bound)
     static constexpr int CPH = kMegaWGs / H;                    // position chunks per head
     static constexpr int PART = R + 4;                          // floats per partial (128 numerators, denominator, pad)
     // floats of one layer's hand-over buffers
@@ -146,7 +171,7 @@ struct MegaShapeBase {
     // after the layers: every workgroup's best logit (value, index), then the XCD every workgroup found itself on
     static constexpr int XCHG_TAIL = 3 * kMegaWGs, OFF_XCC = 2 * kMegaWGs;
     static_assert((3 * D) % kMegaWGs == 0 && (2 * F) % kMegaWGs == 0 && D % kMegaWGs == 0, "rows must split over 256 workgroups");
-    static_assert(H * R == D && CPH >= 1 && NRD >= 1 && NRF >= 1, "shape");
+    static_assert(H * R == D && CPH >= 1 && NRF >= 1, "shape");
     // bytes of the weight stream of one layer
     static constexpr size_t PHASE_A_BYTES = (size_t)kMegaWGs * NW * TA * TILE, PHASE_C_BYTES = (size_t)kMegaWGs * NW * TC * TILE,
                             PHASE_D_BYTES = (size_t)kMegaWGs * NW * TD * TILE, PHASE_E_BYTES = (size_t)kMegaWGs * NW * TE * TILE;
@@ -262,9 +287,10 @@ __device__ __forceinline__ int xs_index(int idx)
 }
 
 // the 32 activations of this lane's block column, from LDS
+template <bool OPAQUE = false>
 __device__ __forceinline__ void load_slab(float (&xr)[32], float &xsum, const float *xs, int block, bool have)
 {
-    const int blk = have ? block : 0;
+    const int blk = maybe_opaque<OPAQUE>(have ? block : 0);
     const float *src = xs + blk * 32;
     float s = 0.f;
 #pragma unroll
@@ -284,8 +310,8 @@ struct MegaWave {
     uint32_t layers, vocab_rows /* head rows per workgroup */, vocab;
     int b, w, lane;
     // per phase geometry (column slab, row set, whether the wave works in the phase, whether the lane has a column)
-    int sD, rD, sF, rF;
-    bool actD, actF, laneD, laneF;
+    int sD, rD, sF, rF, blockD /* this lane's block column in the D-wide phases */;
+    bool actD, actF, laneF, halfD /* the wave works on the half slab: two rows per tile */;
 
     __device__ __forceinline__ void init(const MegaArgs &a)
     {
@@ -294,7 +320,11 @@ struct MegaWave {
         vocab_rows = (a.vocab + kMegaWGs - 1) / kMegaWGs;
         // the wave index is uniform: telling the compiler so keeps every tile address in scalar registers
         b = blockIdx.x; w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); lane = threadIdx.x & 63;
-        sD = w % S::NSD; rD = w / S::NSD; actD = rD < S::NRD; laneD = sD * 64 + lane < S::NBD;
+        halfD = S::HALFD && w >= S::FULLD * S::WPF && w < S::FULLD * S::WPF + S::WPH;
+        actD = w < S::FULLD * S::WPF + S::WPH;
+        sD = halfD ? S::FULLD : w % S::FULLD;
+        rD = halfD ? w - S::FULLD * S::WPF : w / S::FULLD;
+        blockD = halfD ? S::FULLD * 64 + (lane & 31) : sD * 64 + lane;
         sF = w % S::NSF; rF = w / S::NSF; actF = rF < S::NRF; laneF = sF * 64 + lane < S::NBF;
     }
 
@@ -309,12 +339,13 @@ struct MegaWave {
         if (wrapped) { k -= S::PER_LAYER; layer += 1; }
         const bool into_head = wrapped && layer >= layers;  // uniform, runtime
         int i = 0, tiles = 0, rows = 0, rset = 0;
-        bool act = false, lane_ok = false, real = true;
+        bool act = false, lane_ok = false, real = true, dwide = true;
         size_t off = 0;
-        if (k < S::SEQ_C) { i = k; tiles = S::TA; rows = S::ROWS_A; act = actD; lane_ok = laneD; rset = rD; }
-        else if (k < S::SEQ_D) { i = k - S::SEQ_C; tiles = S::TC; rows = S::ROWS_C; act = actD; lane_ok = laneD; rset = rD; off = S::PHASE_A_BYTES; }
-        else if (k < S::SEQ_E) { i = k - S::SEQ_D; tiles = S::TD; rows = S::ROWS_D; act = actD; lane_ok = laneD; rset = rD; off = S::PHASE_A_BYTES + S::PHASE_C_BYTES; }
+        if (k < S::SEQ_C) { i = k; tiles = S::TA; rows = S::ROWS_A; }
+        else if (k < S::SEQ_D) { i = k - S::SEQ_C; tiles = S::TC; rows = S::ROWS_C; off = S::PHASE_A_BYTES; }
+        else if (k < S::SEQ_E) { i = k - S::SEQ_D; tiles = S::TD; rows = S::ROWS_D; off = S::PHASE_A_BYTES + S::PHASE_C_BYTES; }
         else if (k < S::SEQ_E + S::TE) {
+            dwide = false;
             i = k - S::SEQ_E; tiles = S::TE; rows = S::ROWS_E; act = actF; lane_ok = laneF; rset = rF; off = S::PHASE_A_BYTES + S::PHASE_C_BYTES + S::PHASE_D_BYTES;
             if constexpr (S::E_REDEAL) {
                 int row, slab;
@@ -328,7 +359,9 @@ struct MegaWave {
         if (!real && !head_slot) return;                     // static: this slot never loads
         const uint8_t *p = dummy;
         if (real) {
-            const bool ok = !into_head && act && lane_ok && rset * tiles + i < rows;
+            bool ok;
+            if (dwide) ok = !into_head && d_tile_valid(i, tiles, S::tiles_half(rows), rows);
+            else ok = !into_head && act && lane_ok && rset * tiles + i < rows;
             const uint8_t *q = wstream + (size_t)layer * S::LAYER_BYTES + off + ((size_t)(b * S::NW + w) * tiles + i) * S::TILE;
             p = ok ? q : p;
         }
@@ -339,12 +372,24 @@ struct MegaWave {
         load_tile<S>(t, p, lane);
     }
 
+    // D-wide phases: the row (of the workgroup's `rows`) this lane works on in the wave's tile i, or -1 when it has none.  A
+    // full-slab wave takes rows rD * stride + i, stride = the phase's tiles per wave; a half-slab wave takes the row pairs
+    // rD * stride_half + i, its lower lanes the first row of a pair, its upper lanes the second.
+    __device__ __forceinline__ int d_row(int i, int stride, int stride_half, int rows) const
+    {
+        if (!actD) return -1;
+        if (!halfD) { const int r = rD * stride + i; return i < stride && r < rows ? r : -1; }
+        const int r = 2 * (rD * stride_half + i) + (lane >> 5);
+        return i < stride_half && r < rows ? r : -1;
+    }
+    __device__ __forceinline__ bool d_tile_valid(int i, int stride, int stride_half, int rows) const { return d_row(i, stride, stride_half, rows) >= 0; }
+
     // address of head tile k of this wave, or null when the wave/lane/row has none
     __device__ __forceinline__ const uint8_t *head_tile(int k) const
     {
-        const int rows = (int)vocab_rows, per_set = (rows + S::NRD - 1) / S::NRD;
-        const int j = rD * per_set + k;
-        const bool ok = actD && laneD && k < per_set && j < rows && (uint32_t)(b * rows + j) < vocab;
+        const int rows = (int)vocab_rows;
+        const int j = d_row(k, cdiv(rows, S::WPF), S::HALFD ? cdiv(cdiv(rows, 2), S::WPH) : 0, rows);
+        const bool ok = j >= 0 && (uint32_t)(b * rows + j) < vocab;
         return ok ? wstream + (size_t)layers * S::LAYER_BYTES + ((size_t)(b * S::NW + w) * S::HEAD + k) * S::TILE : nullptr;
     }
 
@@ -385,6 +430,47 @@ __device__ __forceinline__ void gemv_phase(MegaTile (&q)[S::DEPTH], const MegaWa
     }
 }
 
+// A D-wide GEMV phase (input vector of D floats, ROWS rows per workgroup): waves on a full slab take one row per tile, waves
+// on the half slab two (MegaShapeBase).  Leaves per-row sums in red[row * NSD + slab].
+template <class S, int SEQ0, int ROWS>
+__device__ __forceinline__ void gemv_phase_d(MegaTile (&q)[S::DEPTH], const MegaWave<S> &mw, uint32_t layer, const float (&xr)[32],
+                                             float xsum, float *red)
+{
+    constexpr int NT = S::tiles_d(ROWS), TH = S::tiles_half(ROWS), NT4 = round_up(NT, 4), NS = S::NSD;
+    float p[4];
+#pragma unroll
+    for (int i = 0; i < NT4; i++) {
+        if (i < NT) {
+            const int slot = (SEQ0 + i) % S::DEPTH;
+            const MegaTile t = q[slot];
+            p[i & 3] = tile_dot<S>(t, xr, xsum);
+            mw.fetch(q[slot], SEQ0 + i + S::DEPTH, layer);
+        } else {
+            p[i & 3] = 0.f;
+        }
+        if ((i & 3) == 3) {
+            // where the sums go is computed here, every time (shapes with a half slab: dozens of addresses kept from in front
+            // of the layer loop would spill)
+            const int ln = maybe_opaque<S::HALFD != 0>(mw.lane);
+            if (S::HALFD && mw.halfD) {          // uniform over the wave
+                float s01, s23;
+                quad_partials_sum_halves(p[0], p[1], p[2], p[3], s01, s23);
+                const int g = ln >> 4;
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    const int ii = (i - 3) + 2 * h + (g >> 1), row = 2 * (mw.rD * TH + ii) + (g & 1);
+                    if ((ln & 15) == 0 && ii < TH && row < ROWS) red[row * NS + mw.sD] = h ? s23 : s01;
+                }
+            } else {
+                const float s = quad_partials_sum(p[0], p[1], p[2], p[3]);
+                const int ii = (i - 3) + quad_partial_of_lane(ln);
+                const int row = mw.rD * NT + ii;
+                if (mw.actD && (ln & 15) == 0 && row < ROWS && ii < NT) red[row * NS + mw.sD] = s;
+            }
+        }
+    }
+}
+
 template <int NS>
 __device__ __forceinline__ float red_row(const float *red, int row)
 {
@@ -398,7 +484,7 @@ __device__ __forceinline__ float red_row(const float *red, int row)
 template <class S>
 struct MegaLds {
     static constexpr int XS = S::F > S::D ? S::F : S::D;
-    static constexpr int RED_ROWS = S::ROWS_D > S::HEAD * S::NRD ? S::ROWS_D : S::HEAD * S::NRD;
+    static constexpr int RED_ROWS = S::ROWS_D > S::MAX_VOCAB_ROWS ? S::ROWS_D : S::MAX_VOCAB_ROWS;
     static constexpr int RED_COLS = S::NSF > S::NSD ? S::NSF : S::NSD;
     float xs[XS];                    // the phase's input vector (during attention: exp(score) of the chunk)
     float red[RED_ROWS * RED_COLS];  // per-row partial sums, one column per slab
@@ -414,20 +500,21 @@ struct MegaLds {
 // rsqrt(variance), the same for every element, is returned for the caller to apply to its row sums.  The waves so
 // start on their tiles one barrier after the vector has arrived instead of three; the variance is taken as
 // mean(x^2) - mean(x)^2 from one pass over the registers.  The norm weights are requested before the wait, not after.
-template <int N, int NW, bool NORM, int SLEEP = 0>
+template <int N, int NW, bool NORM, int SLEEP = 0, bool OPAQUE = false>
 __device__ __forceinline__ float acquire_vector(float *xs, const float *src, const float *w, float *scratch, uint32_t *status, uint32_t spin_limit)
 {
     constexpr int T = NW * 64, PER = cdiv(N, T);
+    const int tx = maybe_opaque<OPAQUE>((int)threadIdx.x);
     float v[PER];
     bool want[PER];
 #pragma unroll
-    for (int j = 0; j < PER; j++) want[j] = (int)threadIdx.x + j * T < N;
+    for (int j = 0; j < PER; j++) want[j] = tx + j * T < N;
     float wn[NORM ? PER : 1];
     if constexpr (NORM) {
 #pragma unroll
-        for (int j = 0; j < PER; j++) wn[j] = want[j] ? w[threadIdx.x + j * T] : 0.f;
+        for (int j = 0; j < PER; j++) wn[j] = want[j] ? w[tx + j * T] : 0.f;
     }
-    poll_values<PER, SLEEP>(v, src + threadIdx.x, T, want, status, spin_limit);
+    poll_values<PER, SLEEP>(v, src + tx, T, want, status, spin_limit);
     float inv = 1.f;
     if constexpr (NORM) {
         float s1 = 0.f, s2 = 0.f;
@@ -436,11 +523,11 @@ __device__ __forceinline__ float acquire_vector(float *xs, const float *src, con
             const float x = want[j] ? v[j] : 0.f;
             s1 += x;
             s2 = fmaf(x, x, s2);
-            if (want[j]) xs[xs_index(threadIdx.x + j * T)] = x * wn[j];
+            if (want[j]) xs[xs_index(tx + j * T)] = x * wn[j];
         }
         s1 = wave_sum(s1);
         s2 = wave_sum(s2);
-        if ((threadIdx.x & 63) == 0) { scratch[threadIdx.x >> 6] = s1; scratch[NW + (threadIdx.x >> 6)] = s2; }
+        if ((tx & 63) == 0) { scratch[tx >> 6] = s1; scratch[NW + (tx >> 6)] = s2; }
         lds_barrier();
         float t1 = 0.f, t2 = 0.f;
 #pragma unroll
@@ -450,7 +537,7 @@ __device__ __forceinline__ float acquire_vector(float *xs, const float *src, con
     } else {
 #pragma unroll
         for (int j = 0; j < PER; j++)
-            if (want[j]) xs[xs_index(threadIdx.x + j * T)] = v[j];
+            if (want[j]) xs[xs_index(tx + j * T)] = v[j];
         lds_barrier();
     }
     return inv;
@@ -574,9 +661,9 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
         uint16_t *kc = a.kv + (size_t)layer * 2 * a.backlog * D, *vc = kc + (size_t)a.backlog * D;
 
         // ================= A: norm + QKV ====================================================================
-        const float inv_a = acquire_vector<D, NW, true, kPollDelay>(xs, x_src, norm_w, scratch, status, spin_limit);
-        load_slab(xr, xsum, xs, mw.sD * 64 + lane, mw.laneD);
-        gemv_phase<S, S::SEQ_A, S::TA, S::NSD>(q, mw, layer, xr, xsum, mw.sD, mw.rD, mw.actD, S::ROWS_A, red);
+        const float inv_a = acquire_vector<D, NW, true, kPollDelay, S::HALFD != 0>(xs, x_src, norm_w, scratch, status, spin_limit);
+        load_slab<S::HALFD != 0>(xr, xsum, xs, mw.blockD, mw.actD);
+        gemv_phase_d<S, S::SEQ_A, S::ROWS_A>(q, mw, layer, xr, xsum, red);
         if (layer == 0 && a.xcd_local && w == 0) {
             // lane j asks for workgroup (b % 8) + 8 j; the words were stored when the kernel started
             float got[1];
@@ -768,9 +855,9 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
         }
 
         // ================= C: x += Wo o ============================================================================
-        acquire_vector<D, NW, false, kPollDelay>(xs, xc + S::OFF_O, nullptr, scratch, status, spin_limit);
-        load_slab(xr, xsum, xs, mw.sD * 64 + lane, mw.laneD);
-        gemv_phase<S, S::SEQ_C, S::TC, S::NSD>(q, mw, layer, xr, xsum, mw.sD, mw.rD, mw.actD, S::ROWS_C, red);
+        acquire_vector<D, NW, false, kPollDelay, S::HALFD != 0>(xs, xc + S::OFF_O, nullptr, scratch, status, spin_limit);
+        load_slab<S::HALFD != 0>(xr, xsum, xs, mw.blockD, mw.actD);
+        gemv_phase_d<S, S::SEQ_C, S::ROWS_C>(q, mw, layer, xr, xsum, red);
         lds_barrier();
         if (st < S::ROWS_C) {
             const float v = xown[st] + red_row<S::NSD>(red, st);
@@ -779,9 +866,9 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
         }
 
         // ================= D: norm + SwiGLU ========================================================================
-        const float inv_d = acquire_vector<D, NW, true, kPollDelay>(xs, xc + S::OFF_X1, norm_w + D, scratch, status, spin_limit);
-        load_slab(xr, xsum, xs, mw.sD * 64 + lane, mw.laneD);
-        gemv_phase<S, S::SEQ_D, S::TD, S::NSD>(q, mw, layer, xr, xsum, mw.sD, mw.rD, mw.actD, S::ROWS_D, red);
+        const float inv_d = acquire_vector<D, NW, true, kPollDelay, S::HALFD != 0>(xs, xc + S::OFF_X1, norm_w + D, scratch, status, spin_limit);
+        load_slab<S::HALFD != 0>(xr, xsum, xs, mw.blockD, mw.actD);
+        gemv_phase_d<S, S::SEQ_D, S::ROWS_D>(q, mw, layer, xr, xsum, red);
         lds_barrier();
         if (st < S::ROWS_D / 2) {
             // rows alternate W3 row k, W1 row k (matmul_silu_ff.comp:96: result1 * result2 / (exp(-result2) + 1))
@@ -838,9 +925,9 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
 
     // ================= head: norm + output matrix ====================================================================
     {
-        const float inv_h = acquire_vector<D, NW, true, kPollDelay>(xs, x_src, a.norms + (size_t)a.layers * 2 * D, scratch, status, spin_limit);
-        load_slab(xr, xsum, xs, mw.sD * 64 + lane, mw.laneD);
-        const int rows = (int)mw.vocab_rows, per_set = (rows + S::NRD - 1) / S::NRD;
+        const float inv_h = acquire_vector<D, NW, true, kPollDelay, S::HALFD != 0>(xs, x_src, a.norms + (size_t)a.layers * 2 * D, scratch, status, spin_limit);
+        load_slab<S::HALFD != 0>(xr, xsum, xs, mw.blockD, mw.actD);
+        const int rows = (int)mw.vocab_rows, per_set = cdiv(rows, S::WPF), per_half = S::HALFD ? cdiv(cdiv(rows, 2), S::WPH) : 0;
         // the head's slots are numbered from 0; tiles beyond per_set read the dummy tile
         float p[4];
 #pragma unroll
@@ -850,10 +937,21 @@ __global__ __launch_bounds__(S::NW * 64, 1) void mega_decode_kernel(MegaArgs a)
             p[i & 3] = tile_dot<S>(t, xr, xsum);
             mw.fetch_head(q[slot], i + S::DEPTH);
             if ((i & 3) == 3) {
-                const float s = quad_partials_sum(p[0], p[1], p[2], p[3]);
-                const int ii = (i - 3) + quad_partial_of_lane(lane);
-                const int row = mw.rD * per_set + ii;
-                if (mw.actD && (lane & 15) == 0 && ii < per_set && row < rows) red[row * S::NSD + mw.sD] = s;
+                if (S::HALFD && mw.halfD) {      // uniform over the wave: two rows per tile
+                    float s01, s23;
+                    quad_partials_sum_halves(p[0], p[1], p[2], p[3], s01, s23);
+                    const int g = lane >> 4;
+#pragma unroll
+                    for (int h = 0; h < 2; h++) {
+                        const int ii = (i - 3) + 2 * h + (g >> 1), row = 2 * (mw.rD * per_half + ii) + (g & 1);
+                        if ((lane & 15) == 0 && ii < per_half && row < rows) red[row * S::NSD + mw.sD] = h ? s23 : s01;
+                    }
+                } else {
+                    const float s = quad_partials_sum(p[0], p[1], p[2], p[3]);
+                    const int ii = (i - 3) + quad_partial_of_lane(lane);
+                    const int row = mw.rD * per_set + ii;
+                    if (mw.actD && (lane & 15) == 0 && ii < per_set && row < rows) red[row * S::NSD + mw.sD] = s;
+                }
             }
         }
         lds_barrier();
@@ -927,7 +1025,8 @@ template <class S>
 __global__ void mega_pack_kernel(uint8_t *dst /* start of the phase region */, MegaPackSrc src, int phase, uint32_t vocab)
 {
     const int tiles = phase == 0 ? S::TA : phase == 1 ? S::TC : phase == 2 ? S::TD : phase == 3 ? S::TE : S::HEAD;
-    const int ns = phase == 3 ? S::NSF : S::NSD, nr = phase == 3 ? S::NRF : S::NRD, nb = phase == 3 ? S::NBF : S::NBD;
+    const bool dwide = phase != 3;
+    const int nb = dwide ? S::NBD : S::NBF;
     const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t total = (size_t)kMegaWGs * S::NW * tiles * 64;
     if (idx >= total) return;
@@ -936,41 +1035,51 @@ __global__ void mega_pack_kernel(uint8_t *dst /* start of the phase region */, M
     const int i = tile % tiles;
     const int w = (tile / tiles) % S::NW;
     const int b = tile / tiles / S::NW;
-    int slab = w % ns, rset = w / ns;
     uint8_t *out = dst + tile * S::TILE;
     uint4 codes = make_uint4(0, 0, 0, 0), codes2 = codes;
     uint16_t scale = 0;
     float scale32 = 0.f;
-    int e_row = 0;
-    if (S::E_REDEAL && phase == 3) {
-        mega_e_tile<S>(w, i, e_row, slab);
-        rset = 0;
+    // which row of the workgroup's rows and which block column this lane of this tile holds (-1: none) -- the same rules as
+    // MegaWave::init / d_row for the D-wide phases, as MegaWave::fetch for phase E
+    int j = -1, blk = 0;
+    const int rows = phase == 0 ? S::ROWS_A : phase == 1 ? S::ROWS_C : phase == 2 ? S::ROWS_D : phase == 3 ? S::ROWS_E : (int)((vocab + kMegaWGs - 1) / kMegaWGs);
+    if (dwide) {
+        const bool half = S::HALFD && w >= S::FULLD * S::WPF && w < S::FULLD * S::WPF + S::WPH;
+        const bool act = w < S::FULLD * S::WPF + S::WPH;
+        const int stride = phase == 4 ? cdiv(rows, S::WPF) : tiles;
+        const int stride_half = S::HALFD ? cdiv(cdiv(rows, 2), S::WPH) : 0;
+        if (act && !half) {
+            const int rset = w / S::FULLD, r = rset * stride + i;
+            blk = (w % S::FULLD) * 64 + lane;
+            if (i < stride && r < rows) j = r;
+        } else if (act) {
+            const int rset = w - S::FULLD * S::WPF, r = 2 * (rset * stride_half + i) + (lane >> 5);
+            blk = S::FULLD * 64 + (lane & 31);
+            if (i < stride_half && r < rows) j = r;
+        }
+    } else {
+        int slab = w % S::NSF, rset = w / S::NSF, r = rset * tiles + i;
+        if (S::E_REDEAL) { mega_e_tile<S>(w, i, r, slab); rset = 0; }
+        blk = slab * 64 + lane;
+        if (rset < S::NRF && blk < nb && r < rows) j = r;
     }
-    const int blk = slab * 64 + lane;
-    bool ok = rset < nr && blk < nb;
+    bool ok = j >= 0;
     const MatView *mv = nullptr;
     uint32_t row = 0;
     if (ok) {
+        const int g = b * rows + j;
         if (phase == 4) {
-            const int rows = (vocab + kMegaWGs - 1) / kMegaWGs, per_set = (rows + nr - 1) / nr;
-            const int j = rset * per_set + i;
-            ok = i < per_set && j < rows && (uint32_t)(b * rows + j) < vocab;
-            row = b * rows + j;
+            ok = (uint32_t)g < vocab;
+            row = g;
             mv = &src.m[0];
-        } else {
-            const int rows = phase == 0 ? S::ROWS_A : phase == 1 ? S::ROWS_C : phase == 2 ? S::ROWS_D : S::ROWS_E;
-            const int j = (S::E_REDEAL && phase == 3) ? e_row : rset * tiles + i;
-            ok = j < rows;
-            const int g = b * rows + j;
-            if (phase == 0) {
-                int which = 0, r = 0;
-                if (ok) mega_qkv_row<S>(b, j, which, r);
-                mv = &src.m[which];
-                row = r;
-            }
-            else if (phase == 2) { mv = &src.m[g & 1]; row = g >> 1; }
-            else { mv = &src.m[0]; row = g; }
+        } else if (phase == 0) {
+            int which = 0, r = 0;
+            mega_qkv_row<S>(b, j, which, r);
+            mv = &src.m[which];
+            row = r;
         }
+        else if (phase == 2) { mv = &src.m[g & 1]; row = g >> 1; }
+        else { mv = &src.m[0]; row = g; }
     }
     if (ok) {
         const size_t sb = (size_t)row * nb + blk;
